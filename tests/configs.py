@@ -1,0 +1,29 @@
+"""Tiny Qwen3 configurations for tests.  A and B differ in every size and option; W adds
+a sliding window on some layers (two cache groups) and a head size that is no power of
+two; all have widths and vocabularies that are no power of two where they can."""
+
+def _cfg(**kw):
+    base = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", hidden_act="silu")
+    base.update(kw)
+    return base
+
+
+TINY = {
+    "A": dict(
+        config=_cfg(num_hidden_layers=2, hidden_size=64, num_attention_heads=4, num_key_value_heads=2,
+                    head_dim=32, intermediate_size=128, vocab_size=256, rope_theta=10000.0,
+                    rms_norm_eps=1e-6, tie_word_embeddings=True, max_position_embeddings=128),
+        seed=0, linear_std=0.02, norm_std=0.1, page_size=16),
+    "B": dict(
+        config=_cfg(num_hidden_layers=3, hidden_size=96, num_attention_heads=6, num_key_value_heads=2,
+                    head_dim=16, intermediate_size=224, vocab_size=509, rope_theta=1e6,
+                    rms_norm_eps=1e-5, tie_word_embeddings=False, max_position_embeddings=512),
+        seed=1, linear_std=0.03, norm_std=0.05, page_size=8),
+    "W": dict(
+        config=_cfg(num_hidden_layers=3, hidden_size=80, num_attention_heads=5, num_key_value_heads=5,
+                    head_dim=48, intermediate_size=176, vocab_size=300, rope_theta=50000.0,
+                    rms_norm_eps=1e-5, tie_word_embeddings=False, max_position_embeddings=320,
+                    sliding_window=24,
+                    layer_types=["sliding_attention", "full_attention", "sliding_attention"]),
+        seed=2, linear_std=0.05, norm_std=0.2, page_size=16),
+}

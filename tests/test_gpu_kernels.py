@@ -1,0 +1,320 @@
+"""Each HIP kernel alone against a plain float32 reference of the same operation, at sizes
+other than the tiny models': head sizes in steps of 16, head counts and groups that are
+no power of two, widths and vocabularies that are no power of two."""
+import math
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def _tol(dtype, n_round=1):
+    # float32: a few ulp over a reduction; bfloat16: half an ulp (2^-9) per rounding
+    return 2e-5 if dtype == torch.float32 else 2.0 ** -8 * n_round
+
+
+def _rand(shape, dtype, gen, scale=1.0):
+    return (torch.randn(shape, generator=gen) * scale).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("V,H,T", [(301, 72, 37), (1000, 4096, 5)])
+def test_embed(dtype, V, H, T):
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(1)
+    table = _rand((V, H), dtype, g)
+    ids = torch.randint(0, V, (T,), generator=g, dtype=torch.int32)
+    ids[0], ids[-1] = 0, V - 1
+    out = kernels.embed(table.to(DEV), ids.to(DEV)).cpu()
+    assert torch.equal(out, table.float()[ids.long()])
+
+
+@pytest.mark.parametrize("out_dtype", DTYPES)
+@pytest.mark.parametrize("y_dtype", [None, torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,H,eps", [(9, 200, 1e-5), (3, 4096, 1e-6), (70, 33, 1e-3)])
+def test_add_rmsnorm(out_dtype, y_dtype, T, H, eps):
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(2)
+    resid = _rand((T, H), torch.float32, g, 3.0)
+    y = _rand((T, H), y_dtype, g, 2.0) if y_dtype is not None else None
+    w = 1 + 0.2 * torch.randn(H, generator=g)
+    s = resid + (y.float() if y is not None else 0)
+    ref = plain.rms_norm(s.double(), w.double(), eps)
+    r_dev = resid.to(DEV)
+    out = kernels.add_rmsnorm(r_dev, y.to(DEV) if y is not None else None, w.to(DEV), eps, out_dtype)
+    assert out.dtype == out_dtype
+    err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
+    assert err < _tol(out_dtype), err
+    # the sum is written back into the residual stream, exactly
+    assert torch.equal(r_dev.cpu(), s)
+    # with rows: only those rows, and the residual stream is left alone
+    rows = torch.tensor([T - 1, 0, T // 2], dtype=torch.int32)
+    r_dev = resid.to(DEV)
+    out2 = kernels.add_rmsnorm(r_dev, y.to(DEV) if y is not None else None, w.to(DEV), eps, out_dtype,
+                               rows=rows.to(DEV))
+    assert torch.equal(r_dev.cpu(), resid)
+    assert torch.equal(out2.cpu(), out.cpu()[rows.long()])
+
+
+def test_rmsnorm_matches_library_and_scale_invariance():
+    """Pins the plain formula: equals torch's rms_norm; rms(c*x) = rms(x) as eps -> 0."""
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(5, 48, generator=g, dtype=torch.float64)
+    w = torch.randn(48, generator=g, dtype=torch.float64)
+    lib = torch.nn.functional.rms_norm(x, (48,), w, 1e-6)
+    assert torch.allclose(plain.rms_norm(x, w, 1e-6), lib, rtol=1e-12, atol=1e-12)
+    assert torch.allclose(plain.rms_norm(7.0 * x, w, 0.0), plain.rms_norm(x, w, 0.0), rtol=1e-12)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,I", [(13, 48), (5, 1001), (2, 12288)])
+def test_silu_mul(dtype, T, I):
+    """(13, 48) is the shape of the reference's own probe
+    (/root/reference/tests/probes/attention_misc_precision_probe.rs)."""
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(4)
+    gu = _rand((T, 2 * I), dtype, g, 2.0)
+    ref = plain.swiglu(gu[:, :I].double(), gu[:, I:].double())
+    lib = torch.nn.functional.silu(gu[:, :I].double()) * gu[:, I:].double()
+    assert torch.allclose(ref, lib, rtol=1e-12, atol=1e-12)
+    out = kernels.silu_mul(gu.to(DEV)).cpu().double()
+    err = (out - ref).abs().max() / ref.abs().max()
+    assert err < _tol(dtype), err
+
+
+@pytest.mark.parametrize("in_dtype,out_dtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                                (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("M,N,K", [(1, 77, 130), (5, 509, 96), (67, 130, 33), (130, 64, 4096)])
+def test_gemm_fixed_order(in_dtype, out_dtype, M, N, K):
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(5)
+    x = _rand((M, K), in_dtype, g)
+    w = _rand((N, K), in_dtype, g, 0.1)
+    ref = x.double() @ w.double().T
+    y = kernels.gemm_tn(x.to(DEV), w.to(DEV), out_dtype=out_dtype)
+    err = (y.cpu().double() - ref).abs().max() / ref.abs().max()
+    assert err < (1e-5 if out_dtype == torch.float32 else 2.0 ** -8), err
+    # a row's result does not depend on the rows beside it: bit-equal alone and in the batch
+    y1 = kernels.gemm_tn(x[M // 2:M // 2 + 1].contiguous().to(DEV), w.to(DEV), out_dtype=out_dtype)
+    assert torch.equal(y1.cpu()[0], y.cpu()[M // 2])
+    if out_dtype == torch.float32:
+        acc = torch.ones((M, N), dtype=torch.float32, device=DEV)
+        kernels.gemm_tn(x.to(DEV), w.to(DEV), out=acc, accumulate=True)
+        assert torch.allclose(acc.cpu(), y.cpu() + 1.0, rtol=0, atol=1e-5 * float(ref.abs().max()) + 1e-6)
+
+
+@pytest.mark.parametrize("M", [1, 3, 8, 64, 200])
+@pytest.mark.parametrize("N,K", [(509, 96), (1536, 4096), (4096, 1408)])
+def test_linear_bf16(M, N, K):
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(6)
+    x = _rand((M, K), torch.bfloat16, g)
+    w = _rand((N, K), torch.bfloat16, g, 0.05)
+    ref = x.double() @ w.double().T
+    y = kernels.linear_bf16(x.to(DEV), w.to(DEV))
+    err = (y.cpu().double() - ref).abs().max() / ref.abs().max()
+    assert err < 2.0 ** -8, err
+
+
+def _rope_ref(x, pos, cos, sin, rot, interleaved):
+    x = x.double().clone()
+    c, s = cos[pos].double()[:, None, :], sin[pos].double()[:, None, :]
+    if interleaved:
+        a, b = x[..., 0:rot:2].clone(), x[..., 1:rot:2].clone()
+        x[..., 0:rot:2], x[..., 1:rot:2] = a * c - b * s, a * s + b * c
+    else:
+        h = rot // 2
+        a, b = x[..., :h].clone(), x[..., h:rot].clone()
+        x[..., :h], x[..., h:rot] = a * c - b * s, a * s + b * c
+    return x
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,rot,interleaved,norm", [
+    (3, 2, 8, 8, False, False),      # the shape of the reference's rope probe (q (11,3,8), k (11,2,8))
+    (3, 2, 8, 8, True, False),
+    (7, 7, 48, 48, False, True),
+    (6, 2, 16, 16, False, True),
+    (8, 2, 128, 128, False, True),
+    (5, 1, 80, 32, False, True),     # partial rotary
+    (4, 2, 256, 256, True, True),
+])
+def test_qk_norm_rope_kv(dtype, nq, nkv, d, rot, interleaved, norm):
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(7)
+    # positions of the reference's probe (attention_misc_precision_probe.rs:36-40)
+    positions = torch.tensor([0, 7, 2, 31, 9, 16, 3, 63, 4, 12, 5], dtype=torch.int32)
+    T, page, pages, eps = positions.numel(), 4, 9, 1e-5
+    cos, sin = plain.rope_tables(10000.0, rot, 64)
+    qkv = _rand((T, (nq + 2 * nkv) * d), dtype, g)
+    qw = (1 + 0.3 * torch.randn(d, generator=g)) if norm else None
+    kw = (1 + 0.3 * torch.randn(d, generator=g)) if norm else None
+    perm = torch.randperm(pages * page, generator=g)[:T]
+    slots = perm.to(torch.int64)
+    kc = torch.zeros((pages, nkv, page, d), dtype=dtype)
+    vc = torch.zeros_like(kc)
+    q_out = kernels.qk_norm_rope_kv(
+        qkv.to(DEV), qw.to(DEV) if norm else None, kw.to(DEV) if norm else None, eps, cos.to(DEV),
+        sin.to(DEV), rot, interleaved, positions.to(DEV), slots.to(DEV), (kcd := kc.to(DEV)),
+        (vcd := vc.to(DEV)), nq, nkv, d)
+    x = qkv.double().reshape(T, nq + 2 * nkv, d)
+    q, k, v = x[:, :nq], x[:, nq:nq + nkv], x[:, nq + nkv:]
+    if norm:
+        q, k = plain.rms_norm(q, qw.double(), eps), plain.rms_norm(k, kw.double(), eps)
+    q = _rope_ref(q, positions.long(), cos, sin, rot, interleaved)
+    k = _rope_ref(k, positions.long(), cos, sin, rot, interleaved)
+    tol = _tol(dtype)
+    assert (q_out.cpu().double() - q).abs().max() / q.abs().max() < tol
+    kcd, vcd = kcd.cpu().double(), vcd.cpu()
+    for t in range(T):
+        p, o = int(slots[t]) // page, int(slots[t]) % page
+        assert (kcd[p, :, o] - k[t]).abs().max() / k.abs().max() < tol, t
+        assert torch.equal(vcd[p, :, o].double(), v[t]), t
+    # nothing but the named slots was written
+    touched = torch.zeros(pages * page, dtype=torch.bool)
+    touched[slots] = True
+    flat = kcd.permute(0, 2, 1, 3).reshape(pages * page, -1)
+    assert float(flat[~touched].abs().max()) == 0.0
+
+
+def test_rope_invariants():
+    """Pins the plain rotation: position 0 is the identity; pair norms are kept; the inner
+    product of rotated q and k depends on the distance of their positions alone; and the
+    sign convention (a wrong sign or pairing breaks the shift invariance)."""
+    g = torch.Generator().manual_seed(8)
+    d = 16
+    cos, sin = plain.rope_tables(10000.0, d, 128)
+    q = torch.randn(1, 1, d, generator=g, dtype=torch.float64)
+    k = torch.randn(1, 1, d, generator=g, dtype=torch.float64)
+    at = lambda x, p: plain.apply_rope(x, torch.tensor([p]), cos.double(), sin.double())
+    assert torch.allclose(at(q, 0), q)
+    r = at(q, 37)
+    assert torch.allclose(r[..., :8] ** 2 + r[..., 8:] ** 2, q[..., :8] ** 2 + q[..., 8:] ** 2)
+    d1 = (at(q, 9) * at(k, 4)).sum()
+    d2 = (at(q, 59) * at(k, 54)).sum()
+    assert abs(float(d1 - d2)) < 1e-5
+    assert abs(float((at(q, 9) * at(k, 4)).sum() - (at(q, 9) * at(k, 5)).sum())) > 1e-3
+    # first pair, unit vector along a: rotated by +angle (counter-clockwise)
+    e = torch.zeros(1, 1, d, dtype=torch.float64)
+    e[..., 0] = 1.0
+    r = at(e, 1)
+    assert abs(float(r[0, 0, 0]) - math.cos(1.0)) < 1e-6 and abs(float(r[0, 0, 8]) - math.sin(1.0)) < 1e-6
+
+
+def _paged_case(g, dtype, nq, nkv, d, page, seqs, extra_pages=3):
+    """Random K/V of several sequences laid into a paged cache under a shuffled page map.
+    `seqs` = list of (context length, number of query tokens at its end)."""
+    total_pages = sum(-(-c // page) for c, _ in seqs) + extra_pages
+    order = torch.randperm(total_pages, generator=g).tolist()
+    kc = torch.zeros((total_pages, nkv, page, d), dtype=dtype)
+    vc = torch.zeros_like(kc)
+    max_pages = max(-(-c // page) for c, _ in seqs)
+    bt = torch.zeros((len(seqs), max_pages), dtype=torch.int32)
+    ks, vs, qs, tok_seq, positions = [], [], [], [], []
+    for b, (ctx, nq_tok) in enumerate(seqs):
+        k = _rand((ctx, nkv, d), dtype, g)
+        v = _rand((ctx, nkv, d), dtype, g)
+        for lp in range(-(-ctx // page)):
+            phys = order.pop()
+            bt[b, lp] = phys
+            n = min(page, ctx - lp * page)
+            kc[phys, :, :n] = k[lp * page:lp * page + n].transpose(0, 1)
+            vc[phys, :, :n] = v[lp * page:lp * page + n].transpose(0, 1)
+        ks.append(k)
+        vs.append(v)
+        qs.append(_rand((nq_tok, nq, d), dtype, g))
+        tok_seq += [b] * nq_tok
+        positions += list(range(ctx - nq_tok, ctx))
+    return dict(kc=kc, vc=vc, bt=bt, ks=ks, vs=vs, qs=qs,
+                tok_seq=torch.tensor(tok_seq, dtype=torch.int32),
+                positions=torch.tensor(positions, dtype=torch.int32))
+
+
+def _attention_ref(case, seqs, window, scale):
+    outs = []
+    for b, (ctx, n) in enumerate(seqs):
+        k, v = case["ks"][b].double(), case["vs"][b].double()
+        q_full = torch.zeros((ctx, case["qs"][b].shape[1], k.shape[2]), dtype=torch.float64)
+        q_full[ctx - n:] = case["qs"][b].double()
+        o = plain.attention(q_full, k, v, window=window or None, scale=scale)
+        outs.append(o[ctx - n:].reshape(n, -1))
+    return torch.cat(outs)
+
+
+ATTN_CASES = [
+    # nq, nkv, d, page, window, [(context, queries)]
+    (4, 2, 32, 16, 0, [(5, 5), (17, 17), (33, 33)]),
+    (6, 2, 16, 8, 0, [(200, 1), (130, 48), (9, 9), (64, 2)]),
+    (5, 5, 48, 16, 24, [(100, 100), (31, 1), (24, 24), (25, 2)]),
+    (8, 2, 128, 64, 0, [(300, 37), (1, 1), (257, 1)]),
+    (3, 1, 80, 4, 7, [(40, 40), (13, 2)]),
+    (2, 2, 256, 16, 0, [(70, 70)]),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,page,window,seqs", ATTN_CASES)
+def test_attention_generic(dtype, nq, nkv, d, page, window, seqs):
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(9)
+    case = _paged_case(g, dtype, nq, nkv, d, page, seqs)
+    scale = 1.0 / math.sqrt(d)
+    ref = _attention_ref(case, seqs, window, scale)
+    q = torch.cat(case["qs"]).contiguous()
+    out = kernels.attention_generic(q.to(DEV), case["kc"].to(DEV), case["vc"].to(DEV), case["bt"].to(DEV),
+                                    case["tok_seq"].to(DEV), case["positions"].to(DEV), scale, window)
+    err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
+    assert err < _tol(dtype, 2), err
+
+
+def test_attention_pins():
+    """Pins the plain attention: without mask effects (last row) it is softmax(QK^T/sqrt d)V
+    of the library; one token gives v; one group equals multi-head attention."""
+    g = torch.Generator().manual_seed(10)
+    T, nq, nkv, d = 12, 4, 2, 8
+    q = torch.randn(T, nq, d, generator=g, dtype=torch.float64)
+    k = torch.randn(T, nkv, d, generator=g, dtype=torch.float64)
+    v = torch.randn(T, nkv, d, generator=g, dtype=torch.float64)
+    out = plain.attention(q, k, v)
+    lib = torch.nn.functional.scaled_dot_product_attention(
+        q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None], is_causal=True,
+        enable_gqa=True)[0].transpose(0, 1)
+    assert torch.allclose(out, lib, rtol=1e-10, atol=1e-12)
+    assert torch.allclose(plain.attention(q[:1], k[:1], v[:1])[0, 0], v[0, 0])
+    # window w: the query at p sees exactly keys p-w+1..p
+    w = 5
+    outw = plain.attention(q, k, v, window=w)
+    p = 9
+    s = (q[p, 0] @ k[p - w + 1:p + 1, 0].T) / math.sqrt(d)
+    assert torch.allclose(outw[p, 0], torch.softmax(s, -1) @ v[p - w + 1:p + 1, 0])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_far_key_stands_out(dtype):
+    """One far key among hundreds is made to win the softmax by scaling it and the query:
+    a kernel that skips or misplaces it returns a visibly different row."""
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(11)
+    nq, nkv, d, page = 4, 2, 64, 16
+    seqs = [(700, 1)]
+    case = _paged_case(g, dtype, nq, nkv, d, page, seqs)
+    far = 3                                            # position of the key that must win
+    qv = case["qs"][0]
+    kfar = (qv[0, 0].float() / qv[0, 0].float().norm() * 40).to(dtype)
+    case["ks"][0][far, 0] = kfar
+    phys, off = int(case["bt"][0, far // page]), far % page
+    case["kc"][phys, 0, off] = kfar
+    scale = 1.0 / math.sqrt(d)
+    ref = _attention_ref(case, seqs, 0, scale)
+    assert (ref[0, :d] - case["vs"][0][far, 0].double()).abs().max() < 0.05   # head 0 returns v[far]
+    out = kernels.attention_generic(torch.cat(case["qs"]).to(DEV), case["kc"].to(DEV), case["vc"].to(DEV),
+                                    case["bt"].to(DEV), case["tok_seq"].to(DEV), case["positions"].to(DEV),
+                                    scale, 0)
+    err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
+    assert err < _tol(dtype, 2), err

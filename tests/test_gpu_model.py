@@ -1,0 +1,103 @@
+"""The engine against the plain implementation, in float32 and in bfloat16, under every way
+of cutting the work: whole requests; most of a request in one step and its last 32 tokens
+one by one; portions of changing size down to two tokens; and mixed batches of up to four
+live requests with so few pages that pages are used again."""
+import random
+
+import pytest
+import torch
+
+import harness
+import plain_qwen3 as plain
+from configs import TINY
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+LENGTHS = {"A": [5, 17, 33, 100, 128], "B": [1, 9, 64, 130, 200], "W": [3, 24, 25, 77, 150, 61]}
+
+
+def _requests(name):
+    rng = random.Random(100 + ord(name))
+    vocab = TINY[name]["config"]["vocab_size"]
+    return {f"r{i}": harness.random_prompt(rng, n, vocab) for i, n in enumerate(LENGTHS[name])}
+
+
+_plain_cache = {}
+
+
+def _plain_logits(name, model_dir):
+    if name not in _plain_cache:
+        pm = plain.PlainModel(model_dir)
+        _plain_cache[name] = {rid: pm.logits(toks) for rid, toks in _requests(name).items()}
+    return _plain_cache[name]
+
+
+_runner_cache = {}
+
+
+def _runner(name, dtype, model_dir, num_pages):
+    """One loaded model per (config, dtype); a fresh runner (and so a fresh cache) per test."""
+    from xinfer_amd.engine import ModelRunner, load_model
+    key = (name, dtype)
+    if key not in _runner_cache:
+        _runner_cache[key] = load_model(model_dir, dtype, "cuda:0")
+    return ModelRunner(_runner_cache[key], page_size=TINY[name]["page_size"], num_pages=num_pages,
+                       max_requests=4)
+
+
+def _run(name, dtype, model_dirs, steps, what):
+    page = TINY[name]["page_size"]
+    need = harness.tokens_needed(steps, page)
+    runner = _runner(name, dtype, model_dirs[name], need // page)       # exactly enough pages
+    got = harness.replay(runner, steps)
+    for g in range(len(runner.cache.groups)):
+        assert runner.cache.free_pages(g) == need // page               # every page came back
+    ref = _plain_logits(name, model_dirs[name])
+    rel = harness.compare(got, ref, harness.TOL[dtype], f"{name}/{dtype}/{what}")
+    print(f"{name}/{dtype}/{what}: worst error {rel:.2e} of the largest logit")
+    return got
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(TINY))
+def test_whole(name, dtype, model_dirs):
+    got = _run(name, dtype, model_dirs, harness.trace_whole(_requests(name)), "whole")
+    assert len(got) == sum(LENGTHS[name])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(TINY))
+def test_tail_one_by_one(name, dtype, model_dirs):
+    _run(name, dtype, model_dirs, harness.trace_tail_one_by_one(_requests(name)), "tail")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(TINY))
+def test_portions(name, dtype, model_dirs):
+    _run(name, dtype, model_dirs, harness.trace_portions(_requests(name)), "portions")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(TINY))
+@pytest.mark.parametrize("seed", [0, 1])
+def test_mixed(name, dtype, seed, model_dirs):
+    reqs = _requests(name)
+    steps = harness.trace_mixed(reqs, seed)
+    page = TINY[name]["page_size"]
+    # fewer pages than all requests together would need: later requests reuse pages
+    assert harness.tokens_needed(steps, page) < sum(-(-len(t) // page) * page for t in reqs.values())
+    _run(name, dtype, model_dirs, steps, f"mixed{seed}")
+
+
+@pytest.mark.parametrize("name", list(TINY))
+def test_float32_does_not_depend_on_cutting(name, model_dirs):
+    """In float32 every reduction's order is fixed by the position alone, so logits are
+    bit-equal however the tokens were cut and batched."""
+    reqs = _requests(name)
+    a = _run(name, "float32", model_dirs, harness.trace_whole(reqs), "whole")
+    b = _run(name, "float32", model_dirs, harness.trace_mixed(reqs, 7), "mixed7")
+    c = _run(name, "float32", model_dirs, harness.trace_portions(reqs), "portions")
+    for key in a:
+        assert torch.equal(a[key], b[key]), key
+        assert torch.equal(a[key], c[key]), key

@@ -1,0 +1,273 @@
+// Bandwidth-bound kernels: embedding gather, fused residual-add + RMSNorm,
+// fused per-head q/k RMSNorm + rotary embedding + paged KV write, SiLU*mul.
+// All reductions are float32 in an order fixed by the row alone, so a row's
+// result does not depend on what else is in the batch.
+#include "common.h"
+#include <stdarg.h>
+#include <stdio.h>
+
+namespace xi {
+
+static thread_local char g_error[512] = "";
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+// ---------------------------------------------------------------------------------
+// Embedding: out[t, :] = float(table[ids[t], :])                (reference call site:
+// /root/reference/src/models/qwen3.rs:303, candle Embedding::forward)
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                             float* __restrict__ out, int H) {
+  const int t = blockIdx.x;
+  const T* row = table + (size_t)ids[t] * H;
+  float* o = out + (size_t)t * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_float(row[i]);
+}
+
+// ---------------------------------------------------------------------------------
+// Fused residual add + RMSNorm (reference: attention_rs::norm::add_rms_norm at
+// /root/reference/src/models/layers/others.rs:118-123; plain rms_norm at :83).
+//   s = resid[row] (+ y[row]);  if rows == null the sum is written back to resid;
+//   out[r] = s * rsqrt(mean(s^2) + eps) * w, rounded once to the output type.
+// The residual stream is float32 in both precisions.
+// ---------------------------------------------------------------------------------
+template <typename TY, typename TO, int NT>
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TY* __restrict__ y,
+                                   const float* __restrict__ w, float eps, TO* __restrict__ out,
+                                   const int* __restrict__ rows, int H) {
+  __shared__ float scratch[NT / kWave];
+  const int r = blockIdx.x;
+  const int row = rows ? rows[r] : r;
+  float* x = resid + (size_t)row * H;
+  const TY* yr = y ? y + (size_t)row * H : nullptr;
+  TO* o = out + (size_t)r * H;
+  float ss = 0.f;
+  // first pass: sum (written back or kept in the output buffer's place is not possible for
+  // a narrower TO, so the sum is recomputed in the second pass from the same operands).
+  for (int i = threadIdx.x; i < H; i += NT) {
+    float s = x[i];
+    if (yr) s += to_float(yr[i]);
+    ss += s * s;
+  }
+  const float total = block_sum<NT / kWave>(ss, scratch);
+  const float inv = rsqrtf(total / (float)H + eps);
+  for (int i = threadIdx.x; i < H; i += NT) {
+    float s = x[i];
+    if (yr) {
+      s += to_float(yr[i]);
+      if (!rows) x[i] = s;
+    }
+    o[i] = from_float<TO>(s * inv * w[i]);
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// SiLU(gate) * up on a packed [T, 2I] buffer (reference: attention_rs::silu_and_mul at
+// /root/reference/src/models/layers/mlp.rs:627-628; golden formula
+// /root/reference/tests/probes/compare_attention_misc_probe.py:81-86).
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total) {
+  size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; idx < total; idx += stride) {
+    const size_t t = idx / I;
+    const int i = (int)(idx - t * I);
+    const float g = to_float(gu[t * 2 * I + i]);
+    const float u = to_float(gu[t * 2 * I + I + i]);
+    const float s = g / (1.f + __expf(-g));
+    out[idx] = from_float<T>(s * u);
+  }
+}
+template <>
+__global__ void silu_mul_kernel<float>(const float* __restrict__ gu, float* __restrict__ out, int I,
+                                       size_t total) {
+  size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; idx < total; idx += stride) {
+    const size_t t = idx / I;
+    const int i = (int)(idx - t * I);
+    const float g = gu[t * 2 * I + i];
+    const float u = gu[t * 2 * I + I + i];
+    const float s = g / (1.f + expf(-g));  // full-precision exp on the 32-bit path
+    out[idx] = s * u;
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// Per-head q/k RMSNorm + rotary embedding + KV write into the paged cache.
+// One wave per (token, head) over the packed projection row [q heads | k heads | v heads].
+//   q, k: x = rms(x, w) if w given (reference attention.rs:734-741); then the first
+//   `rot` dims are rotated by the token's position (rotary_emb.rs:103; formula
+//   tests/probes/compare_attention_misc_probe.py:33-49):
+//     half layout:        pairs (i, i + rot/2);   interleaved layout: pairs (2i, 2i+1)
+//     o_a = a*cos - b*sin;  o_b = a*sin + b*cos
+//   q goes to q_out [T, nq, d]; k and v go to cache[page, kv_head, offset, :] with
+//   slot = page*page_size + offset (reference slot formula runner.rs:1344-1362).
+//   A negative slot means: do not store (the token's cache belongs to another run).
+// ---------------------------------------------------------------------------------
+template <typename T>
+__global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, const float* __restrict__ qw,
+                                       const float* __restrict__ kw, float eps,
+                                       const float* __restrict__ cos_t,
+                                       const float* __restrict__ sin_t, int rot, int interleaved,
+                                       const int* __restrict__ positions,
+                                       const long long* __restrict__ slots, T* __restrict__ q_out,
+                                       T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                       int page_size, int n_tok, int nq, int nkv, int d) {
+  const int heads = nq + 2 * nkv;
+  const int lane = threadIdx.x & (kWave - 1);
+  const long long wid = (long long)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (wid >= (long long)n_tok * heads) return;
+  const int t = (int)(wid / heads);
+  const int h = (int)(wid - (long long)t * heads);
+  const T* src = qkv + (size_t)t * heads * d + (size_t)h * d;
+
+  T* dst;
+  const float* w = nullptr;
+  bool rotate = true;
+  if (h < nq) {
+    dst = q_out + ((size_t)t * nq + h) * d;
+    w = qw;
+  } else {
+    const long long slot = slots[t];
+    if (slot < 0) return;
+    const long long page = slot / page_size;
+    const int off = (int)(slot - page * page_size);
+    const bool is_k = h < nq + nkv;
+    const int kvh = is_k ? h - nq : h - nq - nkv;
+    T* cache = is_k ? k_cache : v_cache;
+    dst = cache + (((size_t)page * nkv + kvh) * page_size + off) * d;
+    w = is_k ? kw : nullptr;
+    rotate = is_k;
+  }
+  if (!rotate) {  // v: plain copy
+    for (int i = lane; i < d; i += kWave) dst[i] = src[i];
+    return;
+  }
+  float inv = 1.f;
+  if (w) {
+    float ss = 0.f;
+    for (int i = lane; i < d; i += kWave) {
+      const float v = to_float(src[i]);
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    inv = rsqrtf(ss / (float)d + eps);
+  }
+  const int half = rot / 2;
+  const int pos = positions[t];
+  const float* c = cos_t + (size_t)pos * half;
+  const float* s = sin_t + (size_t)pos * half;
+  for (int i = lane; i < half; i += kWave) {
+    const int ia = interleaved ? 2 * i : i;
+    const int ib = interleaved ? 2 * i + 1 : i + half;
+    float a = to_float(src[ia]) * inv;
+    float b = to_float(src[ib]) * inv;
+    if (w) {
+      // the reference rounds the normed value to the activation type before rotating
+      // (two kernels); here it stays in float32 until the single final rounding.
+      a *= w[ia];
+      b *= w[ib];
+    }
+    const float cs = c[i], sn = s[i];
+    dst[ia] = from_float<T>(a * cs - b * sn);
+    dst[ib] = from_float<T>(a * sn + b * cs);
+  }
+  for (int i = rot + lane; i < d; i += kWave) {  // dims beyond the rotary part
+    float v = to_float(src[i]) * inv;
+    if (w) v *= w[i];
+    dst[i] = from_float<T>(v);
+  }
+}
+
+}  // namespace xi
+
+using namespace xi;
+
+extern "C" {
+
+const char* xi_last_error() { return g_error; }
+
+int xi_embed(const void* table, int dtype, const int* ids, float* out, int n_tok, int H,
+             hipStream_t stream) {
+  XI_CHECK(n_tok >= 0 && H > 0, "embed: bad sizes T=%d H=%d", n_tok, H);
+  if (n_tok == 0) return 0;
+  if (dtype == kF32)
+    embed_kernel<float><<<n_tok, 256, 0, stream>>>((const float*)table, ids, out, H);
+  else if (dtype == kBF16)
+    embed_kernel<bf16><<<n_tok, 256, 0, stream>>>((const bf16*)table, ids, out, H);
+  else
+    XI_CHECK(false, "embed: unknown dtype %d", dtype);
+  XI_LAUNCH_CHECK("embed");
+  return 0;
+}
+
+// y may be null (no add).  rows may be null (all n_rows rows in place).
+int xi_add_rmsnorm(float* resid, const void* y, int y_dtype, const float* w, float eps, void* out,
+                   int out_dtype, const int* rows, int n_rows, int H, hipStream_t stream) {
+  XI_CHECK(n_rows >= 0 && H > 0, "add_rmsnorm: bad sizes rows=%d H=%d", n_rows, H);
+  if (n_rows == 0) return 0;
+  constexpr int NT = 256;
+#define XI_NORM(TY, TO)                                                                   \
+  add_rmsnorm_kernel<TY, TO, NT><<<n_rows, NT, 0, stream>>>(resid, (const TY*)y, w, eps, \
+                                                              (TO*)out, rows, H)
+  if (y_dtype == kF32 && out_dtype == kF32) XI_NORM(float, float);
+  else if (y_dtype == kBF16 && out_dtype == kBF16) XI_NORM(bf16, bf16);
+  else if (y_dtype == kF32 && out_dtype == kBF16) XI_NORM(float, bf16);
+  else if (y_dtype == kBF16 && out_dtype == kF32) XI_NORM(bf16, float);
+  else XI_CHECK(false, "add_rmsnorm: unknown dtypes %d %d", y_dtype, out_dtype);
+#undef XI_NORM
+  XI_LAUNCH_CHECK("add_rmsnorm");
+  return 0;
+}
+
+int xi_silu_mul(const void* gate_up, void* out, int dtype, int n_tok, int I, hipStream_t stream) {
+  XI_CHECK(n_tok >= 0 && I > 0, "silu_mul: bad sizes T=%d I=%d", n_tok, I);
+  if (n_tok == 0) return 0;
+  const size_t total = (size_t)n_tok * I;
+  const int nt = 256;
+  size_t blocks = (total + nt - 1) / nt;
+  if (blocks > 65535u * 16u) blocks = 65535u * 16u;
+  if (dtype == kF32)
+    silu_mul_kernel<float><<<(unsigned)blocks, nt, 0, stream>>>((const float*)gate_up, (float*)out, I, total);
+  else if (dtype == kBF16)
+    silu_mul_kernel<bf16><<<(unsigned)blocks, nt, 0, stream>>>((const bf16*)gate_up, (bf16*)out, I, total);
+  else
+    XI_CHECK(false, "silu_mul: unknown dtype %d", dtype);
+  XI_LAUNCH_CHECK("silu_mul");
+  return 0;
+}
+
+int xi_qk_norm_rope_kv(const void* qkv, int dtype, const float* qw, const float* kw, float eps,
+                       const float* cos_t, const float* sin_t, int rot, int interleaved,
+                       const int* positions, const long long* slots, void* q_out, void* k_cache,
+                       void* v_cache, int page_size, int n_tok, int nq, int nkv, int d,
+                       hipStream_t stream) {
+  XI_CHECK(n_tok >= 0 && nq > 0 && nkv > 0 && d > 0 && page_size > 0,
+           "qk_norm_rope_kv: bad sizes T=%d nq=%d nkv=%d d=%d page=%d", n_tok, nq, nkv, d, page_size);
+  XI_CHECK(rot >= 0 && rot <= d && rot % 2 == 0, "qk_norm_rope_kv: rotary_dim %d must be even and <= head_dim %d", rot, d);
+  XI_CHECK((qw == nullptr) == (kw == nullptr), "qk_norm_rope_kv: q and k norm weights must both be given or both absent");
+  if (n_tok == 0) return 0;
+  const long long waves = (long long)n_tok * (nq + 2 * nkv);
+  const int wpb = 4;
+  const long long blocks = (waves + wpb - 1) / wpb;
+  XI_CHECK(blocks < (1ll << 31), "qk_norm_rope_kv: too many tokens");
+#define XI_QK(TT)                                                                               \
+  qk_norm_rope_kv_kernel<TT><<<(unsigned)blocks, wpb * kWave, 0, stream>>>(                     \
+      (const TT*)qkv, qw, kw, eps, cos_t, sin_t, rot, interleaved, positions, slots, (TT*)q_out, \
+      (TT*)k_cache, (TT*)v_cache, page_size, n_tok, nq, nkv, d)
+  if (dtype == kF32) XI_QK(float);
+  else if (dtype == kBF16) XI_QK(bf16);
+  else XI_CHECK(false, "qk_norm_rope_kv: unknown dtype %d", dtype);
+#undef XI_QK
+  XI_LAUNCH_CHECK("qk_norm_rope_kv");
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,3 @@
+from .loading import build_model, load_model, parse_dtype
+from .model import CausalLM
+from .runner import ModelRunner, StepEntry, StepError

@@ -1,0 +1,42 @@
+"""From a model folder (or a typed config and a weight store) to a loaded model."""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..models import family_of, load_config
+from ..weights.store import SafetensorsStore, WeightStore
+from .model import CausalLM
+
+_DTYPES = {"bf16": torch.bfloat16, "bfloat16": torch.bfloat16, "f32": torch.float32,
+           "float32": torch.float32, "fp32": torch.float32}
+
+
+def parse_dtype(name) -> torch.dtype:
+    """The reference takes --dtype f16|bf16|f32 (/root/reference/src/utils/mod.rs:2479-2486);
+    float16 is not built here."""
+    if isinstance(name, torch.dtype):
+        if name not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"dtype {name} is not supported (bfloat16 or float32)")
+        return name
+    try:
+        return _DTYPES[str(name).lower()]
+    except KeyError:
+        raise ValueError(f"dtype {name!r} is not supported (bf16/bfloat16 or f32/float32)") from None
+
+
+def load_model(model_dir: str, dtype, device="cuda:0") -> CausalLM:
+    fam, cfg = load_config(model_dir)
+    store = SafetensorsStore(model_dir)
+    try:
+        return build_model(cfg, store, dtype, device)
+    finally:
+        store.close()
+
+
+def build_model(config, store: WeightStore, dtype, device="cuda:0") -> CausalLM:
+    fam = family_of(config.architecture)
+    model = CausalLM(fam.build_spec(config), parse_dtype(dtype))
+    model.config = config
+    return model.load(store, device)

@@ -1,0 +1,245 @@
+"""Python bindings of the gfx950 kernel library (csrc/kernels/*.hip) through ctypes.
+
+Every function checks on the host that operand shapes, types, devices and layouts match
+what the kernel and its grid assume, and raises `KernelError` otherwise: a kernel is
+never launched on operands it was not written for.  Kernels run on torch's current HIP
+stream.  There is no other implementation behind these functions: if the library
+cannot be built or loaded, importing fails loudly.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from .csrc.build import load_kernels
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+F32, BF16 = 0, 1
+_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        l = load_kernels()
+        l.xi_last_error.restype = ctypes.c_char_p
+        _lib = l
+    return _lib
+
+
+def _code(t: torch.Tensor, what: str) -> int:
+    try:
+        return _CODE[t.dtype]
+    except KeyError:
+        raise KernelError(f"{what}: dtype {t.dtype} is not supported (float32 or bfloat16)") from None
+
+
+def _dev(*tensors: Optional[torch.Tensor]) -> None:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise KernelError("kernel operands must live on the GPU (there is no CPU path)")
+        if not t.is_contiguous():
+            raise KernelError(f"kernel operand of shape {tuple(t.shape)} is not contiguous")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise KernelError("kernel operands live on different devices")
+
+
+def _p(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(t.data_ptr() if t is not None else 0)
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ok(rc: int) -> None:
+    if rc != 0:
+        raise KernelError(lib().xi_last_error().decode())
+
+
+def _want(t: torch.Tensor, dtype: torch.dtype, what: str) -> None:
+    if t.dtype != dtype:
+        raise KernelError(f"{what} must be {dtype}, got {t.dtype}")
+
+
+# ---------------------------------------------------------------------------------------
+def embed(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[t] = float32(table[ids[t]]).  ids: int32 [T], values in [0, rows) (caller checks)."""
+    _dev(table, ids, out)
+    _want(ids, torch.int32, "embed: ids")
+    if table.dim() != 2 or ids.dim() != 1:
+        raise KernelError("embed: table must be [V, H] and ids [T]")
+    T, H = ids.shape[0], table.shape[1]
+    if out is None:
+        out = torch.empty((T, H), dtype=torch.float32, device=table.device)
+    elif out.shape != (T, H) or out.dtype != torch.float32:
+        raise KernelError("embed: out must be float32 [T, H]")
+    _ok(lib().xi_embed(_p(table), _code(table, "embed"), _p(ids), _p(out), T, H, _stream()))
+    return out
+
+
+def add_rmsnorm(resid: torch.Tensor, y: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """s = resid (+ y); out = rms(s) * weight in `out_dtype`.  Without `rows` every row is
+    normed and the sum is written back into resid; with `rows` (int32 indices) only those
+    rows are produced and resid is left alone."""
+    _dev(resid, y, weight, rows, out)
+    _want(resid, torch.float32, "add_rmsnorm: residual stream")
+    _want(weight, torch.float32, "add_rmsnorm: weight")
+    if resid.dim() != 2 or weight.shape != (resid.shape[1],):
+        raise KernelError(f"add_rmsnorm: resid {tuple(resid.shape)} and weight {tuple(weight.shape)} do not match")
+    if y is not None and y.shape != resid.shape:
+        raise KernelError(f"add_rmsnorm: y {tuple(y.shape)} differs from resid {tuple(resid.shape)}")
+    H = resid.shape[1]
+    if rows is not None:
+        _want(rows, torch.int32, "add_rmsnorm: rows")
+        n = rows.shape[0]
+    else:
+        n = resid.shape[0]
+    if out is None:
+        out = torch.empty((n, H), dtype=out_dtype, device=resid.device)
+    elif out.shape != (n, H) or out.dtype != out_dtype:
+        raise KernelError("add_rmsnorm: out has the wrong shape or dtype")
+    _ok(lib().xi_add_rmsnorm(_p(resid), _p(y), _code(y, "add_rmsnorm") if y is not None else F32,
+                             _p(weight), ctypes.c_float(eps), _p(out), _code(out, "add_rmsnorm"),
+                             _p(rows), n, H, _stream()))
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = silu(gate_up[:, :I]) * gate_up[:, I:]"""
+    _dev(gate_up, out)
+    if gate_up.dim() != 2 or gate_up.shape[1] % 2:
+        raise KernelError("silu_mul: input must be [T, 2I]")
+    T, I = gate_up.shape[0], gate_up.shape[1] // 2
+    if out is None:
+        out = torch.empty((T, I), dtype=gate_up.dtype, device=gate_up.device)
+    elif out.shape != (T, I) or out.dtype != gate_up.dtype:
+        raise KernelError("silu_mul: out has the wrong shape or dtype")
+    _ok(lib().xi_silu_mul(_p(gate_up), _p(out), _code(gate_up, "silu_mul"), T, I, _stream()))
+    return out
+
+
+def qk_norm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor],
+                    k_weight: Optional[torch.Tensor], eps: float, cos: torch.Tensor,
+                    sin: torch.Tensor, rotary_dim: int, interleaved: bool,
+                    positions: torch.Tensor, slots: torch.Tensor, k_cache: torch.Tensor,
+                    v_cache: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
+                    q_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Per-head RMSNorm of q and k (if weights are given), rotation by position, q to q_out
+    [T, nq, d], k and v into the paged cache [pages, nkv, page_size, d] at `slots`."""
+    _dev(qkv, q_weight, k_weight, cos, sin, positions, slots, k_cache, v_cache, q_out)
+    nq, nkv, d = num_heads, num_kv_heads, head_dim
+    T = qkv.shape[0]
+    if qkv.dim() != 2 or qkv.shape[1] != (nq + 2 * nkv) * d:
+        raise KernelError(f"qk_norm_rope_kv: qkv {tuple(qkv.shape)} is not [T, {(nq + 2 * nkv) * d}]")
+    _want(positions, torch.int32, "qk_norm_rope_kv: positions")
+    _want(slots, torch.int64, "qk_norm_rope_kv: slots")
+    _want(cos, torch.float32, "qk_norm_rope_kv: cos")
+    _want(sin, torch.float32, "qk_norm_rope_kv: sin")
+    if positions.shape != (T,) or slots.shape != (T,):
+        raise KernelError("qk_norm_rope_kv: positions and slots must be [T]")
+    if cos.dim() != 2 or cos.shape[1] != rotary_dim // 2 or sin.shape != cos.shape:
+        raise KernelError(f"qk_norm_rope_kv: cos/sin {tuple(cos.shape)} are not [positions, {rotary_dim // 2}]")
+    for w in (q_weight, k_weight):
+        if w is not None:
+            _want(w, torch.float32, "qk_norm_rope_kv: norm weight")
+            if w.shape != (d,):
+                raise KernelError("qk_norm_rope_kv: norm weight must be [head_dim]")
+    if (k_cache.dim() != 4 or k_cache.shape[1] != nkv or k_cache.shape[3] != d
+            or v_cache.shape != k_cache.shape or k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype):
+        raise KernelError(f"qk_norm_rope_kv: cache {tuple(k_cache.shape)} {k_cache.dtype} does not match "
+                          f"[pages, {nkv}, page_size, {d}] {qkv.dtype}")
+    if q_out is None:
+        q_out = torch.empty((T, nq, d), dtype=qkv.dtype, device=qkv.device)
+    elif q_out.shape != (T, nq, d) or q_out.dtype != qkv.dtype:
+        raise KernelError("qk_norm_rope_kv: q_out has the wrong shape or dtype")
+    _ok(lib().xi_qk_norm_rope_kv(
+        _p(qkv), _code(qkv, "qk_norm_rope_kv"), _p(q_weight), _p(k_weight), ctypes.c_float(eps),
+        _p(cos), _p(sin), int(rotary_dim), int(bool(interleaved)), _p(positions), _p(slots),
+        _p(q_out), _p(k_cache), _p(v_cache), int(k_cache.shape[2]), T, nq, nkv, d, _stream()))
+    return q_out
+
+
+def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                      block_tables: torch.Tensor, tok_seq: torch.Tensor, positions: torch.Tensor,
+                      scale: float, window: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Causal paged GQA attention for any mix of tokens.  q [T, nq, d]; caches
+    [pages, nkv, page_size, d]; block_tables int32 [B, max_pages]; tok_seq / positions
+    int32 [T] name each token's row of block_tables and its absolute position.
+    window = 0 keeps all keys, w > 0 the last w (the query's own key included)."""
+    _dev(q, k_cache, v_cache, block_tables, tok_seq, positions, out)
+    if q.dim() != 3:
+        raise KernelError("attention: q must be [T, nq, d]")
+    T, nq, d = q.shape
+    if (k_cache.dim() != 4 or k_cache.shape[3] != d or v_cache.shape != k_cache.shape
+            or k_cache.dtype != q.dtype or v_cache.dtype != q.dtype):
+        raise KernelError(f"attention: cache {tuple(k_cache.shape)} {k_cache.dtype} does not match q {tuple(q.shape)} {q.dtype}")
+    nkv, page = k_cache.shape[1], k_cache.shape[2]
+    for t, name in ((block_tables, "block_tables"), (tok_seq, "tok_seq"), (positions, "positions")):
+        _want(t, torch.int32, f"attention: {name}")
+    if block_tables.dim() != 2 or tok_seq.shape != (T,) or positions.shape != (T,):
+        raise KernelError("attention: block_tables must be [B, max_pages], tok_seq and positions [T]")
+    if out is None:
+        out = torch.empty((T, nq * d), dtype=q.dtype, device=q.device)
+    elif out.shape != (T, nq * d) or out.dtype != q.dtype:
+        raise KernelError("attention: out has the wrong shape or dtype")
+    _ok(lib().xi_attention_generic(
+        _p(q), _p(k_cache), _p(v_cache), _code(q, "attention"), _p(block_tables),
+        int(block_tables.shape[1]), _p(tok_seq), _p(positions), _p(out), ctypes.c_float(scale),
+        int(window), int(page), T, nq, nkv, d, _stream()))
+    return out
+
+
+def gemm_tn(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+            out: Optional[torch.Tensor] = None, accumulate: bool = False) -> torch.Tensor:
+    """y = x @ w.T with x [M, K], w [N, K]; float32 accumulation in ascending k.
+    `accumulate` adds the product to `out` instead of overwriting it."""
+    _dev(x, w, out)
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
+        raise KernelError(f"gemm: x {tuple(x.shape)} and w {tuple(w.shape)} do not match")
+    if x.dtype != w.dtype:
+        raise KernelError(f"gemm: x is {x.dtype} but w is {w.dtype}")
+    M, K = x.shape
+    N = w.shape[0]
+    if out is None:
+        if accumulate:
+            raise KernelError("gemm: accumulate needs an output to add to")
+        out = torch.empty((M, N), dtype=out_dtype or x.dtype, device=x.device)
+    elif out.shape != (M, N) or (out_dtype is not None and out.dtype != out_dtype):
+        raise KernelError("gemm: out has the wrong shape or dtype")
+    _ok(lib().xi_gemm_tn(_p(x), _p(w), _p(out), M, N, K, _code(x, "gemm"), _code(out, "gemm"),
+                         int(bool(accumulate)), _stream()))
+    return out
+
+
+def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx, group: int,
+              scale: float, window: int = 0) -> torch.Tensor:
+    """Attention of one step's tokens over the paged cache of `group`; chooses the kernel
+    from the precision and the shape of the batch."""
+    return attention_generic(q, k_cache, v_cache, ctx.block_tables[group], ctx.tok_seq,
+                             ctx.positions, scale, window)
+
+
+def linear_bf16(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """bfloat16 x @ w.T with float32 accumulation.  Many rows: the vendor library
+    (hipBLASLt through torch), which the reference's engine also uses for its matrix
+    products."""
+    _dev(x, w)
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError("linear_bf16: operands must be bfloat16")
+    return torch.nn.functional.linear(x, w)

@@ -1,0 +1,55 @@
+"""Qwen3 dense as data: the typed config turned into a `ModelSpec`.
+
+Layer composition follows /root/reference/src/models/qwen3.rs:108-134
+(input RMSNorm -> attention -> residual add + post-attention RMSNorm -> SwiGLU MLP
+-> residual add), tensor names qwen3.rs:41,54,81,93,217,236-245,261,280.
+"""
+from __future__ import annotations
+
+from ..config.model_config import Qwen3Config
+from ..config.spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+from .registry import ModelFamily, register_architecture
+
+
+def qwen3_spec(cfg: Qwen3Config) -> ModelSpec:
+    rope = PartSpec("rope", dict(
+        head_dim=cfg.head_dim, rotary_dim=cfg.head_dim, theta=cfg.rope_theta,
+        max_positions=cfg.max_position_embeddings, interleaved=False))
+    layers = []
+    for i in range(cfg.num_hidden_layers):
+        prefix = f"model.layers.{i}"
+        mixer = PartSpec("attention", dict(
+            hidden_size=cfg.hidden_size, num_heads=cfg.num_attention_heads,
+            num_kv_heads=cfg.num_key_value_heads, head_dim=cfg.head_dim,
+            bias=cfg.attention_bias, qk_norm=True, qk_norm_eps=cfg.rms_norm_eps,
+            window=cfg.window_of_layer(i), position=rope,
+            scale=float(cfg.head_dim) ** -0.5))
+        ffn = PartSpec("gated_mlp", dict(
+            hidden_size=cfg.hidden_size, intermediate_size=cfg.intermediate_size,
+            activation=cfg.hidden_act))
+        norm = PartSpec("rmsnorm", dict(dim=cfg.hidden_size, eps=cfg.rms_norm_eps))
+        layers.append(LayerSpec(
+            prefix=prefix, block="prenorm", mixer=mixer, feed_forward=ffn,
+            norms={"input_layernorm": norm, "post_attention_layernorm": norm}))
+    return ModelSpec(
+        architecture=cfg.architecture,
+        vocab_size=cfg.vocab_size,
+        hidden_size=cfg.hidden_size,
+        max_positions=cfg.max_position_embeddings,
+        embedding=PartSpec("embedding", dict(
+            name="model.embed_tokens.weight", vocab_size=cfg.vocab_size, dim=cfg.hidden_size)),
+        layers=tuple(layers),
+        schedule=tuple(ScheduleEntry(i) for i in range(cfg.num_hidden_layers)),
+        final_norm=PartSpec("rmsnorm", dict(
+            dim=cfg.hidden_size, eps=cfg.rms_norm_eps, name="model.norm.weight")),
+        head=PartSpec("lm_head", dict(
+            name="model.embed_tokens.weight" if cfg.tie_word_embeddings else "lm_head.weight",
+            tied=cfg.tie_word_embeddings, vocab_size=cfg.vocab_size, dim=cfg.hidden_size)),
+        eos_token_ids=tuple(cfg.eos_token_id or ()),
+    )
+
+
+QWEN3 = ModelFamily("qwen3", Qwen3Config, qwen3_spec)
+# The reference maps all of these names to ModelType::Qwen3 (utils/mod.rs:2357-2365);
+# only the Qwen3 name is registered here because Qwen2 differs (bias, no q/k norm).
+register_architecture("Qwen3ForCausalLM", QWEN3)

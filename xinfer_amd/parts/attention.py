@@ -1,0 +1,91 @@
+"""Paged grouped-query attention as a mixer.
+
+h -> packed q/k/v projection -> per-head RMSNorm of q and k -> rotation by position ->
+keys/values into the paged cache -> causal attention over the cache (all keys, or the
+last `window`) -> output projection.  Reference: Attention::forward_with_kv,
+/root/reference/src/models/layers/attention.rs:796-977 (projection 805-828, q/k norm
+709-748, RoPE 872-879, paged attention 947-958, o_proj 976); q, k, v weights are
+concatenated at load as in attention.rs:376-407.
+"""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+
+from .. import kernels
+from ..config.spec import PartSpec
+from ..weights.store import TensorDecl, WeightStore
+from .base import (KVNeed, LayerCache, Mixer, StepContext, position_encoding_class,
+                   register_mixer)
+from .linear import Linear
+
+
+@register_mixer("attention")
+class PagedAttention(Mixer):
+    def __init__(self, spec: PartSpec, dtype: torch.dtype):
+        super().__init__(spec, dtype)
+        self.hidden = int(spec["hidden_size"])
+        self.nq = int(spec["num_heads"])
+        self.nkv = int(spec["num_kv_heads"])
+        self.d = int(spec["head_dim"])
+        self.bias = bool(spec.get("bias", False))
+        self.qk_norm = bool(spec.get("qk_norm", False))
+        self.qk_norm_eps = float(spec.get("qk_norm_eps", 1e-6))
+        self.window = int(spec.get("window") or 0)
+        self.scale = float(spec.get("scale", self.d ** -0.5))
+        if self.nq % self.nkv:
+            raise ValueError(f"{self.nq} query heads are not a multiple of {self.nkv} kv heads")
+        if self.bias:
+            raise NotImplementedError("attention projections with bias are not built")
+        pos = spec.get("position")
+        self.position = position_encoding_class(pos.kind)(pos, dtype) if pos is not None else None
+        self.qkv: Optional[Linear] = None
+        self.o: Optional[Linear] = None
+        self.q_norm_w = self.k_norm_w = None
+
+    # ---- weights -----------------------------------------------------------
+    @classmethod
+    def declare(cls, spec: PartSpec, prefix: str) -> List[TensorDecl]:
+        h, nq, nkv, d = (int(spec[k]) for k in ("hidden_size", "num_heads", "num_kv_heads", "head_dim"))
+        out = [TensorDecl(f"{prefix}.q_proj.weight", (nq * d, h)),
+               TensorDecl(f"{prefix}.k_proj.weight", (nkv * d, h)),
+               TensorDecl(f"{prefix}.v_proj.weight", (nkv * d, h)),
+               TensorDecl(f"{prefix}.o_proj.weight", (h, nq * d))]
+        if spec.get("qk_norm", False):
+            out += [TensorDecl(f"{prefix}.q_norm.weight", (d,), "norm"),
+                    TensorDecl(f"{prefix}.k_norm.weight", (d,), "norm")]
+        return out
+
+    def load(self, store: WeightStore, prefix: str, device) -> None:
+        def lin(name):
+            t = store.get(name, None, device)
+            return t.to(self.dtype) if (self.dtype == torch.float32 or t.dtype != torch.float32) else t
+        parts = [lin(f"{prefix}.{n}_proj.weight") for n in ("q", "k", "v")]
+        common = torch.float32 if any(p.dtype == torch.float32 for p in parts) else parts[0].dtype
+        self.qkv = Linear(torch.cat([p.to(common) for p in parts], dim=0))
+        self.o = Linear(lin(f"{prefix}.o_proj.weight"))
+        if self.qk_norm:
+            self.q_norm_w = store.get(f"{prefix}.q_norm.weight", torch.float32, device).contiguous()
+            self.k_norm_w = store.get(f"{prefix}.k_norm.weight", torch.float32, device).contiguous()
+        if self.position is not None:
+            self.position.load(store, prefix, device)
+
+    # ---- cache ---------------------------------------------------------------
+    def cache_need(self) -> KVNeed:
+        return KVNeed(self.nkv, self.d, self.window)
+
+    # ---- step ----------------------------------------------------------------
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
+        qkv = self.qkv(x, out_dtype=self.dtype)
+        pos = self.position
+        slots = ctx.slots[cache.group] if cache.write else ctx.no_slots
+        q = kernels.qk_norm_rope_kv(
+            qkv, self.q_norm_w, self.k_norm_w, self.qk_norm_eps,
+            pos.cos if pos is not None else ctx.empty_f32,
+            pos.sin if pos is not None else ctx.empty_f32,
+            pos.rotary_dim if pos is not None else 0,
+            pos.interleaved if pos is not None else False,
+            ctx.positions, slots, cache.k, cache.v, self.nq, self.nkv, self.d)
+        a = kernels.attention(q, cache.k, cache.v, ctx, cache.group, self.scale, self.window)
+        return self.o(a, out_dtype=self.dtype)

@@ -1,0 +1,204 @@
+"""Interfaces of the parts a layer is made of, and the registries that build them.
+
+A part is built from a `PartSpec` (its sizes and constants) and the activation dtype; it
+declares the tensors it needs under a name prefix, loads them from a weight store, and
+runs on the tokens of one step.  A part never learns which model it is in.
+
+  Mixer            forward(x, ctx, cache) -> y        x, y: [T, hidden]
+                   cache_need() -> KVNeed | None      paged keys/values it wants
+                   state_need() -> StateNeed | None   fixed-size per-request state it wants
+  FeedForward      forward(x, ctx) -> y
+  Norm             forward(resid, add, out_dtype, rows=None, out=None) -> normed
+                   resid is the float32 residual stream; `add` (if given) is summed into
+                   it first; with `rows` only those rows are produced and resid is not
+                   changed.
+  PositionEncoding data for the mixer's fused kernel (for "rope": cos/sin tables)
+  Block            forward(stream, ctx, cache) -> stream, the arrangement of the above
+                   around the residual stream.
+
+New kinds register themselves with the decorators below; a `PartSpec.kind` then selects
+them.  Nothing else in the engine has to change.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..config.spec import LayerSpec, PartSpec
+from ..weights.store import TensorDecl, WeightStore
+
+
+# ---- what a layer may ask of the cache ------------------------------------------------
+@dataclass(frozen=True)
+class KVNeed:
+    """Paged keys and values: `window` = 0 keeps every key, w > 0 the last w."""
+    num_kv_heads: int
+    head_dim: int
+    window: int = 0
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """Fixed-size state per live request: one slot of this shape and dtype."""
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class LayerCache:
+    """What one run of a layer gets from the cache.  `write` is False when the run reads
+    the cache that another layer's run owns."""
+    group: int = -1
+    k: Optional[torch.Tensor] = None          # [pages, kv_heads, page_size, head_dim]
+    v: Optional[torch.Tensor] = None
+    state: Optional[torch.Tensor] = None      # [max_requests, *StateNeed.shape]
+    write: bool = True
+
+
+@dataclass
+class StepContext:
+    """Everything about one step's batch that parts may read.  Device tensors unless
+    marked host."""
+    num_tokens: int
+    num_seqs: int
+    dtype: torch.dtype                         # activation dtype
+    device: torch.device
+    positions: torch.Tensor                    # int32 [T]   absolute position of each token
+    tok_seq: torch.Tensor                      # int32 [T]   row of the batch each token is in
+    cu_q: torch.Tensor                         # int32 [B+1] token offsets of the sequences
+    ctx_lens: torch.Tensor                     # int32 [B]   cached length after this step
+    state_slots: torch.Tensor                  # int64 [B]   per-request state slot
+    slots: List[torch.Tensor]                  # per group int64 [T] cache slot of each token
+    block_tables: List[torch.Tensor]           # per group int32 [B, max_pages]
+    cu_q_host: Sequence[int] = ()              # host copies for choosing kernels
+    ctx_lens_host: Sequence[int] = ()
+    max_q_len: int = 0
+    max_ctx_len: int = 0
+    no_slots: Optional[torch.Tensor] = None    # int64 [T] of -1: "store nothing"
+    empty_f32: Optional[torch.Tensor] = None   # float32 [1, 0]: tables of "no rotation"
+
+
+@dataclass
+class Stream:
+    """The residual stream between blocks: `resid` float32 [T, H], and a branch output
+    `pending` that has not been added to it yet (the next norm adds it in the same
+    kernel that norms)."""
+    resid: torch.Tensor
+    pending: Optional[torch.Tensor] = None
+
+
+class Part:
+    def __init__(self, spec: PartSpec, dtype: torch.dtype):
+        self.spec = spec
+        self.dtype = dtype
+
+    @classmethod
+    def declare(cls, spec: PartSpec, prefix: str) -> List[TensorDecl]:
+        return []
+
+    def load(self, store: WeightStore, prefix: str, device) -> None:
+        pass
+
+
+class Mixer(Part):
+    def cache_need(self) -> Optional[KVNeed]:
+        return None
+
+    def state_need(self) -> Optional[StateNeed]:
+        return None
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Norm(Part):
+    def forward(self, resid: torch.Tensor, add: Optional[torch.Tensor], out_dtype: torch.dtype,
+                rows: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    pass
+
+
+class Block:
+    """Arrangement of a layer's parts around the residual stream."""
+
+    def __init__(self, layer: LayerSpec, dtype: torch.dtype):
+        self.layer = layer
+        self.dtype = dtype
+
+    @classmethod
+    def declare(cls, layer: LayerSpec) -> List[TensorDecl]:
+        raise NotImplementedError
+
+    def load(self, store: WeightStore, device) -> None:
+        raise NotImplementedError
+
+    def cache_need(self) -> Optional[KVNeed]:
+        return None
+
+    def state_need(self) -> Optional[StateNeed]:
+        return None
+
+    def forward(self, stream: Stream, ctx: StepContext, cache: LayerCache) -> Stream:
+        raise NotImplementedError
+
+
+# ---- registries -------------------------------------------------------------------------
+MIXERS: Dict[str, type] = {}
+FEED_FORWARDS: Dict[str, type] = {}
+NORMS: Dict[str, type] = {}
+POSITION_ENCODINGS: Dict[str, type] = {}
+BLOCKS: Dict[str, type] = {}
+
+
+def _register(table: Dict[str, type], what: str) -> Callable[[str], Callable[[type], type]]:
+    def named(kind: str) -> Callable[[type], type]:
+        def deco(cls: type) -> type:
+            table[kind] = cls
+            cls.kind = kind
+            return cls
+        return deco
+    return named
+
+
+register_mixer = _register(MIXERS, "mixer")
+register_feed_forward = _register(FEED_FORWARDS, "feed-forward")
+register_norm = _register(NORMS, "norm")
+register_position_encoding = _register(POSITION_ENCODINGS, "position encoding")
+register_block = _register(BLOCKS, "block")
+
+
+def _lookup(table: Dict[str, type], what: str, kind: str) -> type:
+    try:
+        return table[kind]
+    except KeyError:
+        raise KeyError(f"unknown {what} kind {kind!r} (registered: {', '.join(sorted(table))})") from None
+
+
+def mixer_class(kind: str) -> type:
+    return _lookup(MIXERS, "mixer", kind)
+
+
+def feed_forward_class(kind: str) -> type:
+    return _lookup(FEED_FORWARDS, "feed-forward", kind)
+
+
+def norm_class(kind: str) -> type:
+    return _lookup(NORMS, "norm", kind)
+
+
+def position_encoding_class(kind: str) -> type:
+    return _lookup(POSITION_ENCODINGS, "position encoding", kind)
+
+
+def block_class(kind: str) -> type:
+    return _lookup(BLOCKS, "block", kind)

@@ -1,0 +1,65 @@
+"""Block arrangements.
+
+"prenorm": x -> norm -> mixer -> (+x, norm) -> feed-forward -> (+r)
+(reference: Qwen3DecoderLayer::forward, /root/reference/src/models/qwen3.rs:108-134).
+Each residual add is carried out by the norm kernel that follows it: a block hands on
+the stream with its feed-forward output still pending, and the next block's first
+norm (or the model's final norm) adds it.
+"""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+
+from ..config.spec import LayerSpec
+from ..weights.store import TensorDecl, WeightStore
+from .base import (Block, KVNeed, LayerCache, StateNeed, StepContext, Stream,
+                   feed_forward_class, mixer_class, norm_class, register_block)
+
+# tensor-name infixes of a pre-norm decoder layer's parts (HF naming, qwen3.rs:41,54,81,93)
+_MIXER, _FFN = "self_attn", "mlp"
+
+
+@register_block("prenorm")
+class PreNormBlock(Block):
+    NORM_BEFORE_MIXER = "input_layernorm"
+    NORM_BEFORE_FFN = "post_attention_layernorm"
+
+    def __init__(self, layer: LayerSpec, dtype: torch.dtype):
+        super().__init__(layer, dtype)
+        self.mixer = mixer_class(layer.mixer.kind)(layer.mixer, dtype)
+        self.ffn = feed_forward_class(layer.feed_forward.kind)(layer.feed_forward, dtype)
+        n1, n2 = layer.norms[self.NORM_BEFORE_MIXER], layer.norms[self.NORM_BEFORE_FFN]
+        self.norm1 = norm_class(n1.kind)(n1, dtype)
+        self.norm2 = norm_class(n2.kind)(n2, dtype)
+
+    @classmethod
+    def declare(cls, layer: LayerSpec) -> List[TensorDecl]:
+        p = layer.prefix
+        out = mixer_class(layer.mixer.kind).declare(layer.mixer, f"{p}.{_MIXER}")
+        out += feed_forward_class(layer.feed_forward.kind).declare(layer.feed_forward, f"{p}.{_FFN}")
+        for name in (cls.NORM_BEFORE_MIXER, cls.NORM_BEFORE_FFN):
+            n = layer.norms[name]
+            out += norm_class(n.kind).declare(n, f"{p}.{name}")
+        return out
+
+    def load(self, store: WeightStore, device) -> None:
+        p = self.layer.prefix
+        self.mixer.load(store, f"{p}.{_MIXER}", device)
+        self.ffn.load(store, f"{p}.{_FFN}", device)
+        self.norm1.load(store, f"{p}.{self.NORM_BEFORE_MIXER}", device)
+        self.norm2.load(store, f"{p}.{self.NORM_BEFORE_FFN}", device)
+
+    def cache_need(self) -> Optional[KVNeed]:
+        return self.mixer.cache_need()
+
+    def state_need(self) -> Optional[StateNeed]:
+        return self.mixer.state_need()
+
+    def forward(self, stream: Stream, ctx: StepContext, cache: LayerCache) -> Stream:
+        h = self.norm1.forward(stream.resid, stream.pending, self.dtype)
+        a = self.mixer.forward(h, ctx, cache)
+        h2 = self.norm2.forward(stream.resid, a, self.dtype)
+        m = self.ffn.forward(h2, ctx)
+        return Stream(stream.resid, m)

@@ -1,0 +1,38 @@
+"""y = x @ W^T, the matrix product shared by the parts.
+
+The reference routes every dense projection through candle's matmul, i.e. the vendor
+BLAS (/root/reference/src/models/layers/linear.rs:76-124).  Here:
+  float32  : the hand-written fixed-order kernel (`kernels.gemm_tn`) - true 32-bit, and
+             an output element does not depend on the batch it was computed in;
+  bfloat16 : the hand-written skinny kernel for few rows (decode), the vendor library
+             (hipBLASLt through torch) for many rows, as the reference uses a library.
+A weight that the checkpoint stores in 32 bits stays in 32 bits; activations are then
+widened for this product.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .. import kernels
+
+
+class Linear:
+    def __init__(self, weight: torch.Tensor):
+        if weight.dim() != 2:
+            raise ValueError("a linear weight must be [out, in]")
+        self.weight = weight.contiguous()
+        self.out_features, self.in_features = weight.shape
+
+    def __call__(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        w = self.weight
+        out_dtype = out_dtype or x.dtype
+        if w.dtype == torch.float32:
+            xf = x if x.dtype == torch.float32 else x.float()
+            y = kernels.gemm_tn(xf, w, out_dtype=torch.float32)
+            return y if out_dtype == torch.float32 else y.to(out_dtype)
+        if x.dtype != w.dtype:
+            raise kernels.KernelError(f"linear: activations are {x.dtype} but the weight is {w.dtype}")
+        y = kernels.linear_bf16(x, w)
+        return y if out_dtype == y.dtype else y.to(out_dtype)
