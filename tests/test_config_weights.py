@@ -1,0 +1,180 @@
+"""Configuration, registry, weight loading errors, random-weights folders (no GPU)."""
+import json
+import os
+
+import pytest
+import torch
+
+from configs import TINY
+from xinfer_amd.config import ConfigError, Qwen3Config
+from xinfer_amd.engine.model import CausalLM
+from xinfer_amd.models import config_from_dict, family_of, load_config, registered_architectures
+from xinfer_amd.weights import (RandomStore, SafetensorsStore, TensorDecl, WeightError, write_random_model,
+                                write_safetensors)
+
+
+def test_both_tiny_configs_round_trip(tmp_path):
+    for name, t in TINY.items():
+        fam, cfg = config_from_dict(t["config"])
+        assert isinstance(cfg, Qwen3Config)
+        d = tmp_path / name
+        d.mkdir()
+        (d / "config.json").write_text(json.dumps(cfg.to_dict()))
+        fam2, cfg2 = load_config(str(d))
+        assert cfg2 == cfg and fam2 is fam
+        for key in ("hidden_size", "num_attention_heads", "num_key_value_heads", "head_dim", "vocab_size",
+                    "intermediate_size", "num_hidden_layers", "rms_norm_eps", "rope_theta",
+                    "max_position_embeddings", "tie_word_embeddings"):
+            assert getattr(cfg, key) == t["config"][key], key
+
+
+def test_defaults_follow_the_reference():
+    raw = dict(TINY["A"]["config"])
+    for k in ("head_dim", "rope_theta", "tie_word_embeddings"):
+        raw.pop(k)
+    _, cfg = config_from_dict(raw)
+    assert cfg.head_dim == 64 // 4          # hidden / heads (attention.rs:446)
+    assert cfg.rope_theta == 10000.0        # rotary_emb.rs:49
+    assert cfg.tie_word_embeddings is False
+
+
+@pytest.mark.parametrize("change,needle", [
+    (dict(num_key_value_heads=3), "multiple"),
+    (dict(head_dim=15), "even"),
+    (dict(hidden_act="gelu"), "hidden_act"),
+    (dict(rope_scaling={"rope_type": "yarn", "factor": 4.0}), "rope_scaling"),
+    (dict(sliding_window=0), "sliding_window"),
+    (dict(layer_types=["full_attention"]), "layer_types"),
+    (dict(hidden_size="64"), "integer"),
+    (dict(vocab_size=None), "vocab_size"),
+])
+def test_bad_configs_are_refused(change, needle):
+    raw = dict(TINY["A"]["config"], **change)
+    with pytest.raises(ConfigError, match=needle):
+        config_from_dict(raw)
+
+
+def test_missing_required_key():
+    raw = dict(TINY["A"]["config"])
+    raw.pop("num_hidden_layers")
+    with pytest.raises(ConfigError, match="num_hidden_layers"):
+        config_from_dict(raw)
+
+
+def test_registry():
+    assert "Qwen3ForCausalLM" in registered_architectures()
+    with pytest.raises(ConfigError, match="Unsupported architecture"):
+        family_of("NoSuchModelForCausalLM")
+    with pytest.raises(ConfigError, match="exactly one"):
+        config_from_dict(dict(TINY["A"]["config"], architectures=["A", "B"]))
+
+
+def test_window_per_layer():
+    _, cfg = config_from_dict(TINY["W"]["config"])
+    assert [cfg.window_of_layer(i) for i in range(3)] == [24, None, 24]
+    spec = family_of(cfg.architecture).build_spec(cfg)
+    m = CausalLM(spec, torch.float32)
+    assert [(g.window, g.layers) for g in m.cache_groups] == [(24, (0, 2)), (0, (1,))]
+    # without layer_types the window applies to every layer, as the reference passes it on
+    raw = dict(TINY["W"]["config"])
+    raw.pop("layer_types")
+    _, cfg = config_from_dict(raw)
+    assert [cfg.window_of_layer(i) for i in range(3)] == [24, 24, 24]
+
+
+def test_no_size_stands_in_code():
+    """The spec carries every size from the config; two configs give different specs."""
+    specs = []
+    for name in ("A", "B"):
+        fam, cfg = config_from_dict(TINY[name]["config"])
+        specs.append(fam.build_spec(cfg))
+    a, b = specs
+    assert a.layers[0].mixer.params != b.layers[0].mixer.params
+    assert a.head["name"] == "model.embed_tokens.weight" and b.head["name"] == "lm_head.weight"
+
+
+def _decls(name):
+    fam, cfg = config_from_dict(TINY[name]["config"])
+    return CausalLM.declare(fam.build_spec(cfg))
+
+
+def test_random_folder_round_trip(tmp_path):
+    d = write_random_model(str(tmp_path / "m"), TINY["B"]["config"], seed=1, linear_std=0.03, norm_std=0.05)
+    assert sorted(os.listdir(d)) == ["config.json", "model.safetensors"]
+    st = SafetensorsStore(d)
+    decls = _decls("B")
+    st.check(decls)
+    assert {x.name for x in decls} == set(st.names())
+    w = st.get("model.layers.2.mlp.down_proj.weight")
+    assert w.dtype == torch.bfloat16 and tuple(w.shape) == (96, 224)
+    assert abs(float(w.float().std()) - 0.03) < 0.003
+    n = st.get("model.layers.0.self_attn.k_norm.weight").float()
+    assert abs(float(n.mean()) - 1.0) < 0.05
+    # same seed, same values; another seed, other values; a tensor does not depend on the others
+    rs = RandomStore(decls, 1, 0.03, 0.05)
+    assert torch.equal(rs.get("model.layers.2.mlp.down_proj.weight"), w)
+    assert not torch.equal(RandomStore(decls, 2, 0.03, 0.05).get("model.layers.2.mlp.down_proj.weight"), w)
+    one = RandomStore([x for x in decls if x.name == "model.layers.2.mlp.down_proj.weight"], 1, 0.03, 0.05)
+    assert torch.equal(one.get("model.layers.2.mlp.down_proj.weight"), w)
+    # the plain implementation's reader sees the same bytes
+    from safetensors import safe_open
+    with safe_open(os.path.join(d, "model.safetensors"), framework="pt") as f:
+        assert torch.equal(f.get_tensor("model.layers.2.mlp.down_proj.weight"), w)
+
+
+def test_one_error_lists_everything_wrong(tmp_path):
+    d = write_random_model(str(tmp_path / "m"), TINY["A"]["config"], seed=0)
+    st = SafetensorsStore(d)
+    tensors = {n: st.get(n) for n in st.names()}
+    del tensors["model.layers.1.self_attn.q_norm.weight"]
+    del tensors["model.norm.weight"]
+    tensors["model.layers.0.mlp.gate_proj.weight"] = torch.zeros(128, 63, dtype=torch.bfloat16)
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(16)
+    bad = tmp_path / "bad"
+    bad.mkdir()
+    write_safetensors(str(bad / "model.safetensors"), tensors.items())
+    with pytest.raises(WeightError) as e:
+        SafetensorsStore(str(bad)).check(_decls("A"))
+    err = e.value
+    assert err.missing == ["model.layers.1.self_attn.q_norm.weight", "model.norm.weight"]
+    assert err.unexpected == ["model.layers.0.self_attn.rotary_emb.inv_freq"]
+    assert err.wrong_shape == [("model.layers.0.mlp.gate_proj.weight", (128, 63), (128, 64))]
+    text = str(err)
+    for needle in ("missing", "unexpected", "wrong shapes", "q_norm", "inv_freq", "[128, 63]", "[128, 64]"):
+        assert needle in text
+
+
+def test_tied_model_must_not_carry_a_head(tmp_path):
+    d = write_random_model(str(tmp_path / "m"), TINY["A"]["config"], seed=0)
+    st = SafetensorsStore(d)
+    assert "lm_head.weight" not in st.names()
+    tensors = {n: st.get(n) for n in st.names()}
+    tensors["lm_head.weight"] = tensors["model.embed_tokens.weight"].clone()
+    bad = tmp_path / "bad"
+    bad.mkdir()
+    write_safetensors(str(bad / "model.safetensors"), tensors.items())
+    with pytest.raises(WeightError, match="unexpected"):
+        SafetensorsStore(str(bad)).check(_decls("A"))
+
+
+def test_storage_policy(tmp_path):
+    """bfloat16 stays, float16 becomes bfloat16, a tensor stored in 32 bits stays in 32 bits,
+    integer tables become int32."""
+    path = str(tmp_path / "model.safetensors")
+    write_safetensors(path, [("a", torch.ones(3, dtype=torch.bfloat16)), ("b", torch.ones(3, dtype=torch.float16)),
+                             ("c", torch.full((3,), 1.0000001, dtype=torch.float32)),
+                             ("d", torch.arange(3, dtype=torch.int64)), ("e", torch.ones(2, dtype=torch.float64))])
+    st = SafetensorsStore(str(tmp_path))
+    assert st.get("a").dtype == torch.bfloat16
+    assert st.get("b").dtype == torch.bfloat16
+    assert st.get("c").dtype == torch.float32 and float(st.get("c")[0]) == float(torch.tensor(1.0000001))
+    assert st.get("d").dtype == torch.int32
+    assert st.get("e").dtype == torch.bfloat16
+    assert st.get("a", torch.float32).dtype == torch.float32
+
+
+def test_no_weight_files(tmp_path):
+    with pytest.raises(FileNotFoundError, match="No weight files"):
+        SafetensorsStore(str(tmp_path))
+    with pytest.raises(ConfigError, match="config.json"):
+        load_config(str(tmp_path))

@@ -1,0 +1,442 @@
+"""Generation through the entry point, sampling kernels, the replay program, parts alone,
+long decoding, and a toy mixer with state of its own registered from the test."""
+import json
+import os
+import random
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import harness
+import plain_qwen3 as plain
+import plain_sampling
+from configs import TINY
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ---- sampling kernels ---------------------------------------------------------------------
+def _logits(rows, V, seed, coarse=False):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(rows, V, generator=g) * 3
+    if coarse:
+        x = x.to(torch.bfloat16).float()          # many exact ties, as logits of a bfloat16 head have
+    return x
+
+
+@pytest.mark.parametrize("V", [256, 509, 151936])
+def test_argmax_lowest_index_wins_ties(V):
+    from xinfer_amd.sampling import Sampler
+    s = Sampler(DEV)
+    x = _logits(5, V, 1, coarse=True)
+    x[2, 7] = x[2, V - 3] = 50.0
+    out = s.argmax(x.to(DEV)).cpu()
+    assert out.tolist() == [int(torch.nonzero(r == r.max())[0]) for r in x]
+    assert out[2] == 7
+
+
+@pytest.mark.parametrize("coarse", [False, True])
+@pytest.mark.parametrize("V,T,k,p", [
+    (256, 0.8, 0, 1.0), (509, 1.3, 0, 1.0), (300, 0.7, 32, 1.0), (300, 0.7, 0, 0.9),
+    (300, 0.7, 32, 0.95), (2000, 1.0, 5, 0.5), (151936, 0.7, 32, 0.95), (151936, 1.0, 0, 0.8),
+])
+def test_sample_matches_plain(V, T, k, p, coarse):
+    from xinfer_amd.sampling import Sampler, Strategy
+    s = Sampler(DEV)
+    rows = 6
+    x = _logits(rows, V, 2, coarse)
+    us = [0.0, 0.999999, 0.5, 0.123, 0.77, 0.31]
+    got = s.sample(x.to(DEV).clone(), [Strategy(T, k, p)] * rows, us)
+    for r in range(rows):
+        kept = plain_sampling.kept_probabilities(x[r], T, k, p)
+        want = plain_sampling.draw(kept, us[r])
+        if got[r] != want:
+            # float32 sums may put u on the other side of a boundary: then the two tokens are
+            # neighbours among the kept ones and u lies within rounding of their boundary
+            assert kept[got[r]] > 0, (r, got[r], want)
+            cum = torch.cumsum(kept, 0) / kept.sum()
+            lo, hi = sorted((got[r], want))
+            assert float(kept[lo + 1:hi].sum()) == 0.0 and abs(float(cum[lo]) - us[r]) < 1e-5, (r, got[r], want)
+        assert kept[got[r]] > 0
+
+
+def test_sample_frequencies_follow_softmax():
+    from xinfer_amd.sampling import Sampler, Strategy, uniform
+    s = Sampler(DEV)
+    V, n = 256, 4000
+    x = _logits(1, V, 3)[0] * 0.5
+    logits = x[None].repeat(n, 1).to(DEV)
+    toks = s.sample(logits, [Strategy(0.8)] * n, [uniform(7, 0, i) for i in range(n)])
+    freq = torch.bincount(torch.tensor(toks), minlength=V).double() / n
+    want = torch.softmax(x.double() / 0.8, -1)
+    assert float((freq - want).abs().sum()) < 0.25            # total variation of 4000 draws over 256 tokens
+    assert abs(float(freq[want.argmax()]) - float(want.max())) < 0.03
+
+
+def test_per_row_strategies_and_penalties():
+    from xinfer_amd.sampling import Sampler, Strategy
+    s = Sampler(DEV)
+    V = 300
+    x = _logits(3, V, 4)
+    top = int(x[1].argmax())
+    recent = [[], [top, top, 5], [9]]
+    strat = [Strategy(), Strategy(0.0, frequency_penalty=100.0, presence_penalty=1.0), Strategy(0.9, 4, 1.0)]
+    got = s.sample(x.to(DEV).clone(), strat, [0.1, 0.2, 0.3], recent=recent)
+    assert got[0] == int(x[0].argmax())
+    pen = plain_sampling.apply_penalties(x[1], recent[1], 100.0, 1.0)
+    assert got[1] == int(pen.argmax()) != top
+    assert got[2] == plain_sampling.draw(plain_sampling.kept_probabilities(x[2], 0.9, 4, 1.0), 0.3)
+
+
+# ---- generation through the entry point ---------------------------------------------------------
+def _engine(model_dir, name, dtype, **kw):
+    from xinfer_amd import Engine, EngineConfig
+    t = TINY[name]
+    cfg = EngineConfig(weight_path=model_dir, page_size=t["page_size"], seed=5, **kw)
+    return Engine(cfg, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_greedy_generation_tiny_a(dtype, model_dirs):
+    """BASELINE workload of tiny A: prompts of 5, 17 and 33 tokens, 16 greedy tokens each."""
+    from xinfer_amd import SamplingParams
+    rng = random.Random(0)
+    prompts = [harness.random_prompt(rng, n, 256) for n in (5, 17, 33)]
+    eng = _engine(model_dirs["A"], "A", dtype, max_num_seqs=4, num_pages=12, prefill_chunk_size=16)
+    outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=16, ignore_eos=True))
+    pm = plain.PlainModel(model_dirs["A"])
+    for p, o in zip(prompts, outs):
+        assert o.prompt_length == len(p) and o.decoded_length == 16 and o.finish_reason == "length"
+        if dtype == "f32":
+            assert o.token_ids == pm.greedy(p, 16)
+        else:
+            # bfloat16 may pick the other of two nearly equal logits; every token it picks must be
+            # within tolerance of the plain maximum given the same history
+            ids = list(p)
+            for t in o.token_ids:
+                lg = pm.logits(ids)[-1]
+                assert float(lg.max() - lg[t]) <= 2 * harness.TOL["bfloat16"] * float(lg.abs().max())
+                ids.append(t)
+    assert eng.get_available_kv_tokens() == 12 * 16 and eng.runner.cache.live_requests() == 0
+
+
+def test_tiny_b_workload_chunked_and_sampled(model_dirs):
+    """BASELINE workload of tiny B: prompts 1, 9, 64, 130, 200, chunk 48 mixed with decode,
+    temperature 0.8 with a seed, 24 tokens each.  A request's tokens do not depend on what it was
+    batched with: alone and together give the same tokens (float32)."""
+    from xinfer_amd import SamplingParams
+    rng = random.Random(1)
+    prompts = [harness.random_prompt(rng, n, 509) for n in (1, 9, 64, 130, 200)]
+    sps = [SamplingParams(temperature=0.8, max_tokens=24, ignore_eos=True, seed=100 + i) for i in range(5)]
+    eng = _engine(model_dirs["B"], "B", "f32", max_num_seqs=4, num_pages=80, prefill_chunk_size=48,
+                  max_num_batched_tokens=64)
+    together = eng.generate(prompts, sps)
+    assert [o.decoded_length for o in together] == [24] * 5
+    assert len({tuple(o.token_ids) for o in together}) == 5
+    eng2 = _engine(model_dirs["B"], "B", "f32", max_num_seqs=1, num_pages=40, prefill_chunk_size=1000)
+    for i in (4, 0, 2):
+        alone = eng2.generate([prompts[i]], sps[i])[0]             # the same seed, another request id
+        assert alone.token_ids == together[i].token_ids, i
+    # each token is a token the plain model gives non-negligible probability at that point
+    pm = plain.PlainModel(model_dirs["B"])
+    ids = list(prompts[1])
+    for t in together[1].token_ids:
+        pr = torch.softmax(pm.logits(ids)[-1].double() / 0.8, -1)
+        assert float(pr[t]) > 1e-5
+        ids.append(t)
+
+
+def test_preemption_gives_the_same_tokens(model_dirs):
+    """With too few pages for all requests to finish together the youngest is preempted and
+    recomputed; greedy tokens are those of an engine with plenty of pages."""
+    from xinfer_amd import SamplingParams
+    rng = random.Random(2)
+    prompts = [harness.random_prompt(rng, n, 256) for n in (30, 31, 20)]
+    sp = SamplingParams(temperature=0.0, max_tokens=40, ignore_eos=True)
+    roomy = _engine(model_dirs["A"], "A", "f32", max_num_seqs=4, num_pages=40)
+    want = [o.token_ids for o in roomy.generate(prompts, sp)]
+    tight = _engine(model_dirs["A"], "A", "f32", max_num_seqs=4, num_pages=8)
+    got = tight.generate(prompts, sp)
+    assert [o.token_ids for o in got] == want
+    assert tight.num_preemptions > 0 and roomy.num_preemptions == 0
+    assert tight.get_available_kv_tokens() == 8 * 16
+    with pytest.raises(Exception, match="cache pages"):
+        tight.generate([harness.random_prompt(rng, 100, 256)], SamplingParams(max_tokens=60))
+
+
+def test_eos_and_limits(model_dirs):
+    from xinfer_amd import SamplingParams
+    eng = _engine(model_dirs["A"], "A", "f32", max_num_seqs=2, num_pages=16, max_model_len=40)
+    prompt = [1, 2, 3, 4, 5]
+    free_run = eng.generate([prompt], SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))[0]
+    assert free_run.decoded_length == 12
+    eng.eos_token_ids = {free_run.token_ids[4]}
+    cut = eng.generate([prompt], SamplingParams(temperature=0.0, max_tokens=12))[0]
+    first = free_run.token_ids.index(free_run.token_ids[4])
+    assert cut.token_ids == free_run.token_ids[:first] and cut.finish_reason == "eos"
+    eng.eos_token_ids = set()
+    long = eng.generate([prompt], SamplingParams(temperature=0.0, max_tokens=1000, ignore_eos=True))[0]
+    assert long.prompt_length + long.decoded_length == 40          # clipped to max_model_len
+    with pytest.raises(ValueError, match="max_model_len"):
+        eng.generate([[1] * 40], SamplingParams(max_tokens=2))
+
+
+# ---- long decoding and first tokens ----------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_one_by_one(dtype, model_dirs):
+    """A whole sequence up to the model's last position fed one token per step, with a second
+    request decoding beside it, against the plain logits."""
+    from xinfer_amd.engine import ModelRunner, StepEntry, load_model
+    name = "B"
+    rng = random.Random(3)
+    a = harness.random_prompt(rng, 512, 509)
+    b = harness.random_prompt(rng, 300, 509)
+    pm = plain.PlainModel(model_dirs[name])
+    ref = {"a": pm.logits(a), "b": pm.logits(b)}
+    runner = ModelRunner(load_model(model_dirs[name], dtype, DEV), page_size=8, num_pages=64 + 38, max_requests=2)
+    runner.add_request(0)
+    runner.add_request(1)
+    got = {}
+    for i in range(512):
+        entries = [StepEntry(0, [a[i]], [0])]
+        if i < 300:
+            entries.append(StepEntry(1, [b[i]], [0]))
+        lg = runner.step(entries).cpu()
+        got[("a", i)] = lg[0]
+        if i < 300:
+            got[("b", i)] = lg[1]
+    harness.compare(got, ref, harness.TOL[dtype], f"long decoding {dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(TINY))
+def test_first_tokens(name, dtype, model_dirs):
+    """The first positions of a sequence (one key, two keys, ...) alone in a step."""
+    from xinfer_amd.engine import ModelRunner, StepEntry, load_model
+    vocab = TINY[name]["config"]["vocab_size"]
+    toks = [vocab - 1, 0, 7, 7]
+    pm = plain.PlainModel(model_dirs[name])
+    ref = {"x": pm.logits(toks)}
+    runner = ModelRunner(load_model(model_dirs[name], dtype, DEV), TINY[name]["page_size"], 2, 1)
+    runner.add_request(0)
+    got = {("x", i): runner.step([StepEntry(0, [t], [0])]).cpu()[0] for i, t in enumerate(toks)}
+    harness.compare(got, ref, harness.TOL[dtype], f"first tokens {name} {dtype}")
+
+
+def test_step_refuses_bad_input(model_dirs):
+    from xinfer_amd.cache import OutOfPages
+    from xinfer_amd.engine import ModelRunner, StepEntry, StepError, load_model
+    runner = ModelRunner(load_model(model_dirs["A"], "float32", DEV), 16, 2, 2)
+    runner.add_request(0)
+    for entries, needle in [([StepEntry(0, [], [])], "at least one"), ([StepEntry(0, [256], [0])], "vocabulary"),
+                            ([StepEntry(0, [1], [1])], "outside"), ([StepEntry(3, [1], [0])], "not live"),
+                            ([StepEntry(0, [1], []), StepEntry(0, [2], [])], "twice"),
+                            ([StepEntry(0, [1] * 129, [])], "positions")]:
+        with pytest.raises(StepError, match=needle):
+            runner.step(entries)
+    with pytest.raises(OutOfPages):
+        runner.step([StepEntry(0, [1] * 40, [])])
+    assert runner.length(0) == 0 and runner.cache.free_pages(0) == 2
+    runner.cache.check()
+
+
+# ---- the replay program ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(dtype, model_dirs, tmp_path):
+    """bin/trace_run as a user runs it: steps on standard input, `done <step>` lines back,
+    <step>.f32 files with [wanted, vocab] little-endian float32."""
+    name = "A"
+    reqs = {f"r{i}": harness.random_prompt(random.Random(40 + i), n, 256) for i, n in enumerate([33, 70, 5, 64, 100])}
+    steps = harness.trace_mixed(reqs, 3)
+    need = harness.tokens_needed(steps, 64)
+    out = tmp_path / "out"
+    proc = subprocess.Popen(
+        [sys.executable, os.path.join(REPO, "bin", "trace_run"), "--model", model_dirs[name], "--dtype", dtype,
+         "--out", str(out), "--max-tokens", str(need)],
+        stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+    for st in steps:
+        proc.stdin.write(json.dumps(st) + "\n")
+        proc.stdin.flush()
+        assert proc.stdout.readline().strip() == f"done {st['step']}"
+    proc.stdin.close()
+    assert proc.wait(timeout=120) == 0
+    pm = plain.PlainModel(model_dirs[name])
+    ref = {rid: pm.logits(t) for rid, t in reqs.items()}
+    got, fed = {}, {rid: 0 for rid in reqs}
+    for st in steps:
+        wanted = sum(len(e["want"]) for e in st["entries"])
+        arr = np.fromfile(out / f"{st['step']}.f32", dtype="<f4").reshape(wanted, 256)
+        row = 0
+        for e in st["entries"]:
+            for w in e["want"]:
+                got[(e["id"], fed[e["id"]] + w)] = torch.from_numpy(arr[row].copy())
+                row += 1
+            fed[e["id"]] += len(e["tokens"])
+    assert len(got) == sum(len(t) for t in reqs.values())
+    harness.compare(got, ref, harness.TOL[dtype], f"trace_run {dtype}")
+
+
+# ---- parts alone ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_parts_alone(dtype, model_dirs):
+    """Norm, feed-forward and attention mixer of tiny W's layer 0 each against its plain function."""
+    from xinfer_amd.engine import ModelRunner, StepEntry, load_model
+    from xinfer_amd.parts import StepContext
+    name = "W"
+    model = load_model(model_dirs[name], dtype, DEV)
+    pm = plain.PlainModel(model_dirs[name])
+    c, W = pm.config, pm.weights
+    blk = model.blocks[0]
+    g = torch.Generator().manual_seed(12)
+    T, H = 37, c["hidden_size"]
+    tol = 2e-5 if dtype == torch.float32 else 2.0 ** -7
+    x = torch.randn(T, H, generator=g)
+    # norm
+    out = blk.norm1.forward(x.to(DEV).clone(), None, dtype).cpu().float()
+    ref = plain.rms_norm(x, W["model.layers.0.input_layernorm.weight"], c["rms_norm_eps"])
+    assert float((out - ref).abs().max() / ref.abs().max()) < tol
+    # feed-forward
+    xin = x.to(dtype)
+    out = blk.ffn.forward(xin.to(DEV), None).cpu().float()
+    ref = plain.mlp_block(xin.float(), W, "model.layers.0.mlp")
+    assert float((out - ref).abs().max() / ref.abs().max()) < 2 * tol
+    # attention mixer with a window of 24 over 37 tokens, through the runner's own cache plumbing
+    runner = ModelRunner(model, 16, 4, 1)
+    runner.add_request(0)
+    runner.cache.reserve(0, T)
+    ctx = runner._context(runner.cache.build_batch([0], [T]))
+    out = blk.mixer.forward(xin.to(DEV), ctx, runner.layer_caches[0]).cpu().float()
+    cos, sin = plain.rope_tables(float(c["rope_theta"]), c["head_dim"], c["max_position_embeddings"])
+    ref = plain.attention_block(xin.float(), W, "model.layers.0.self_attn", c, torch.arange(T), cos, sin, 24)
+    assert float((out - ref).abs().max() / ref.abs().max()) < 2 * tol
+
+
+# ---- a toy mixer with state of its own, registered from here ----------------------------------------------
+def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
+    """A mixer defined in this test keeps a running sum of its inputs per request in a
+    fixed-size state slot (no pages).  A new architecture using it in one layer, beside a
+    normal attention layer, is registered, written as a random model folder, loaded and
+    stepped in portions and mixed batches, without a change to the framework's files."""
+    from dataclasses import dataclass
+    from xinfer_amd.config.spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+    from xinfer_amd.engine import ModelRunner, StepEntry, load_model
+    from xinfer_amd.models import ModelFamily, register_architecture
+    from xinfer_amd.parts import Mixer, StateNeed, register_mixer
+    from xinfer_amd.weights import TensorDecl, write_random_model
+
+    @register_mixer("running_mean")
+    class RunningMean(Mixer):
+        """y[t] = W @ mean(x[0..t]) of the request: the state is (sum, count)."""
+
+        def __init__(self, spec, dtype):
+            super().__init__(spec, dtype)
+            self.h = int(spec["hidden_size"])
+
+        @classmethod
+        def declare(cls, spec, prefix):
+            return [TensorDecl(f"{prefix}.mix.weight", (int(spec["hidden_size"]),) * 2)]
+
+        def load(self, store, prefix, device):
+            self.w = store.get(f"{prefix}.mix.weight", torch.float32, device)
+
+        def state_need(self):
+            return StateNeed((self.h + 1,), torch.float32)
+
+        def forward(self, x, ctx, cache):
+            out = torch.empty((ctx.num_tokens, self.h), dtype=torch.float32, device=x.device)
+            for b in range(ctx.num_seqs):
+                lo, hi = ctx.cu_q_host[b], ctx.cu_q_host[b + 1]
+                slot = int(ctx.state_slots[b])
+                first_pos = ctx.ctx_lens_host[b] - (hi - lo)
+                if first_pos == 0:
+                    cache.state[slot].zero_()                       # a slot used before starts clean
+                st = cache.state[slot]
+                sums = st[:self.h] + torch.cumsum(x[lo:hi].float(), 0)
+                counts = st[self.h] + torch.arange(1, hi - lo + 1, device=x.device)
+                out[lo:hi] = (sums / counts[:, None]) @ self.w.T
+                st[:self.h] = sums[-1]
+                st[self.h] = counts[-1]
+            return out.to(self.dtype)
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        vocab_size: int
+        hidden_size: int
+        architecture: str = "ToyStateForCausalLM"
+
+        @classmethod
+        def from_dict(cls, raw, where="config.json"):
+            return cls(int(raw["vocab_size"]), int(raw["hidden_size"]))
+
+        def to_dict(self):
+            return {"architectures": [self.architecture], "vocab_size": self.vocab_size,
+                    "hidden_size": self.hidden_size}
+
+    def toy_spec(cfg):
+        h = cfg.hidden_size
+        norm = PartSpec("rmsnorm", dict(dim=h, eps=1e-5))
+        ffn = PartSpec("gated_mlp", dict(hidden_size=h, intermediate_size=2 * h, activation="silu"))
+        rope = PartSpec("rope", dict(head_dim=16, rotary_dim=16, theta=10000.0, max_positions=256))
+        attn = PartSpec("attention", dict(hidden_size=h, num_heads=2, num_kv_heads=1, head_dim=16, qk_norm=False,
+                                          window=None, position=rope, scale=0.25))
+        layers = (
+            LayerSpec("model.layers.0", "prenorm", PartSpec("running_mean", dict(hidden_size=h)), ffn,
+                      {"input_layernorm": norm, "post_attention_layernorm": norm}),
+            LayerSpec("model.layers.1", "prenorm", attn, ffn,
+                      {"input_layernorm": norm, "post_attention_layernorm": norm}))
+        return ModelSpec(
+            architecture=cfg.architecture, vocab_size=cfg.vocab_size, hidden_size=h, max_positions=256,
+            embedding=PartSpec("embedding", dict(name="model.embed_tokens.weight", vocab_size=cfg.vocab_size, dim=h)),
+            # layer 1 runs twice; its second run reads the keys and values its first run stored
+            layers=layers, schedule=(ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(1, cache_of=1)),
+            final_norm=PartSpec("rmsnorm", dict(dim=h, eps=1e-5, name="model.norm.weight")),
+            head=PartSpec("lm_head", dict(name="lm_head.weight", tied=False, vocab_size=cfg.vocab_size, dim=h)))
+
+    register_architecture("ToyStateForCausalLM", ModelFamily("toy", ToyConfig, toy_spec))
+    d = write_random_model(str(tmp_path / "toy"), {"architectures": ["ToyStateForCausalLM"], "vocab_size": 97,
+                                                   "hidden_size": 32}, seed=3, linear_std=0.1)
+    model = load_model(d, "float32", DEV)
+    assert set(model.state_needs) == {0} and set(model.kv_needs) == {1}
+
+    def run(steps):
+        runner = ModelRunner(model, page_size=8, num_pages=12, max_requests=2)
+        return harness.replay(runner, steps)
+
+    # the same model written out plainly, whole sequences
+    W = plain.read_weights(d)
+    cos, sin = plain.rope_tables(10000.0, 16, 256)
+
+    def mlp(x, i):
+        return plain.mlp_block(x, W, f"model.layers.{i}.mlp")
+
+    def toy_logits(ids):
+        T = len(ids)
+        x = W["model.embed_tokens.weight"][torch.tensor(ids)]
+        h = plain.rms_norm(x, W["model.layers.0.input_layernorm.weight"], 1e-5)
+        mean = torch.cumsum(h, 0) / torch.arange(1, T + 1)[:, None]
+        r = x + mean @ W["model.layers.0.self_attn.mix.weight"].T
+        x = r + mlp(plain.rms_norm(r, W["model.layers.0.post_attention_layernorm.weight"], 1e-5), 0)
+        kv = None
+        for _ in range(2):
+            h = plain.rms_norm(x, W["model.layers.1.input_layernorm.weight"], 1e-5)
+            pos = torch.arange(T)
+            q = plain.apply_rope((h @ W["model.layers.1.self_attn.q_proj.weight"].T).reshape(T, 2, 16), pos, cos, sin)
+            if kv is None:
+                k = plain.apply_rope((h @ W["model.layers.1.self_attn.k_proj.weight"].T).reshape(T, 1, 16), pos, cos, sin)
+                kv = (k, (h @ W["model.layers.1.self_attn.v_proj.weight"].T).reshape(T, 1, 16))
+            a = plain.attention(q, kv[0], kv[1], scale=0.25).reshape(T, 32)
+            r = x + a @ W["model.layers.1.self_attn.o_proj.weight"].T
+            x = r + mlp(plain.rms_norm(r, W["model.layers.1.post_attention_layernorm.weight"], 1e-5), 1)
+        return plain.rms_norm(x, W["model.norm.weight"], 1e-5) @ W["lm_head.weight"].T
+
+    rng = random.Random(9)
+    reqs = {f"q{i}": harness.random_prompt(rng, n, 97) for i, n in enumerate([19, 40, 7, 33])}
+    ref = {rid: toy_logits(t) for rid, t in reqs.items()}
+    for what, steps in (("whole", harness.trace_whole(reqs)), ("mixed", harness.trace_mixed(reqs, 1, max_live=2)),
+                        ("portions", harness.trace_portions(reqs))):
+        harness.compare(run(steps), ref, harness.TOL["float32"], f"toy {what}")

@@ -62,16 +62,6 @@ def test_add_rmsnorm(out_dtype, y_dtype, T, H, eps):
     assert torch.equal(out2.cpu(), out.cpu()[rows.long()])
 
 
-def test_rmsnorm_matches_library_and_scale_invariance():
-    """Pins the plain formula: equals torch's rms_norm; rms(c*x) = rms(x) as eps -> 0."""
-    g = torch.Generator().manual_seed(3)
-    x = torch.randn(5, 48, generator=g, dtype=torch.float64)
-    w = torch.randn(48, generator=g, dtype=torch.float64)
-    lib = torch.nn.functional.rms_norm(x, (48,), w, 1e-6)
-    assert torch.allclose(plain.rms_norm(x, w, 1e-6), lib, rtol=1e-12, atol=1e-12)
-    assert torch.allclose(plain.rms_norm(7.0 * x, w, 0.0), plain.rms_norm(x, w, 0.0), rtol=1e-12)
-
-
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T,I", [(13, 48), (5, 1001), (2, 12288)])
 def test_silu_mul(dtype, T, I):
@@ -183,30 +173,6 @@ def test_qk_norm_rope_kv(dtype, nq, nkv, d, rot, interleaved, norm):
     assert float(flat[~touched].abs().max()) == 0.0
 
 
-def test_rope_invariants():
-    """Pins the plain rotation: position 0 is the identity; pair norms are kept; the inner
-    product of rotated q and k depends on the distance of their positions alone; and the
-    sign convention (a wrong sign or pairing breaks the shift invariance)."""
-    g = torch.Generator().manual_seed(8)
-    d = 16
-    cos, sin = plain.rope_tables(10000.0, d, 128)
-    q = torch.randn(1, 1, d, generator=g, dtype=torch.float64)
-    k = torch.randn(1, 1, d, generator=g, dtype=torch.float64)
-    at = lambda x, p: plain.apply_rope(x, torch.tensor([p]), cos.double(), sin.double())
-    assert torch.allclose(at(q, 0), q)
-    r = at(q, 37)
-    assert torch.allclose(r[..., :8] ** 2 + r[..., 8:] ** 2, q[..., :8] ** 2 + q[..., 8:] ** 2)
-    d1 = (at(q, 9) * at(k, 4)).sum()
-    d2 = (at(q, 59) * at(k, 54)).sum()
-    assert abs(float(d1 - d2)) < 1e-5
-    assert abs(float((at(q, 9) * at(k, 4)).sum() - (at(q, 9) * at(k, 5)).sum())) > 1e-3
-    # first pair, unit vector along a: rotated by +angle (counter-clockwise)
-    e = torch.zeros(1, 1, d, dtype=torch.float64)
-    e[..., 0] = 1.0
-    r = at(e, 1)
-    assert abs(float(r[0, 0, 0]) - math.cos(1.0)) < 1e-6 and abs(float(r[0, 0, 8]) - math.sin(1.0)) < 1e-6
-
-
 def _paged_case(g, dtype, nq, nkv, d, page, seqs, extra_pages=3):
     """Random K/V of several sequences laid into a paged cache under a shuffled page map.
     `seqs` = list of (context length, number of query tokens at its end)."""
@@ -271,28 +237,6 @@ def test_attention_generic(dtype, nq, nkv, d, page, window, seqs):
                                     case["tok_seq"].to(DEV), case["positions"].to(DEV), scale, window)
     err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
     assert err < _tol(dtype, 2), err
-
-
-def test_attention_pins():
-    """Pins the plain attention: without mask effects (last row) it is softmax(QK^T/sqrt d)V
-    of the library; one token gives v; one group equals multi-head attention."""
-    g = torch.Generator().manual_seed(10)
-    T, nq, nkv, d = 12, 4, 2, 8
-    q = torch.randn(T, nq, d, generator=g, dtype=torch.float64)
-    k = torch.randn(T, nkv, d, generator=g, dtype=torch.float64)
-    v = torch.randn(T, nkv, d, generator=g, dtype=torch.float64)
-    out = plain.attention(q, k, v)
-    lib = torch.nn.functional.scaled_dot_product_attention(
-        q.transpose(0, 1)[None], k.transpose(0, 1)[None], v.transpose(0, 1)[None], is_causal=True,
-        enable_gqa=True)[0].transpose(0, 1)
-    assert torch.allclose(out, lib, rtol=1e-10, atol=1e-12)
-    assert torch.allclose(plain.attention(q[:1], k[:1], v[:1])[0, 0], v[0, 0])
-    # window w: the query at p sees exactly keys p-w+1..p
-    w = 5
-    outw = plain.attention(q, k, v, window=w)
-    p = 9
-    s = (q[p, 0] @ k[p - w + 1:p + 1, 0].T) / math.sqrt(d)
-    assert torch.allclose(outw[p, 0], torch.softmax(s, -1) @ v[p - w + 1:p + 1, 0])
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

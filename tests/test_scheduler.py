@@ -1,0 +1,151 @@
+"""The scheduler's decisions (no GPU): admission, token budget, portions, decode beside
+prefill, finishing and freeing, and what happens when pages run out."""
+import random
+
+import pytest
+
+from xinfer_amd.cache import CacheGroup, PagedCacheManager
+from xinfer_amd.engine.scheduler import RequestTooLarge, Scheduler, SchedulerError
+
+
+def make(num_pages=64, page=16, max_seqs=4, budget=64, chunk=32, window_pages=None):
+    groups = [CacheGroup(page, num_pages)]
+    if window_pages:
+        groups.append(CacheGroup(page, window_pages, window=20))
+    cm = PagedCacheManager(groups, max_requests=max_seqs)
+    return cm, Scheduler(cm, max_seqs, budget, chunk)
+
+
+def drive(s, cm, reqs, max_steps=10000, on_step=None):
+    """Runs the schedule/commit/append loop with made-up tokens until everything finished.
+    reqs: id -> (prompt_len, max_new).  Returns per request the list of (start, count)."""
+    total = {rid: p for rid, (p, _) in reqs.items()}
+    new = {rid: 0 for rid in reqs}
+    seen = {rid: [] for rid in reqs}
+    steps = 0
+    while not s.idle():
+        plan, pre = s.schedule()
+        assert plan, "nothing planned although requests remain"
+        for rid in pre:
+            seen[rid].append("preempted")
+        assert sum(e.count for e in plan) <= s.max_batched_tokens
+        assert len({e.request for e in plan}) == len(plan) <= s.max_num_seqs
+        for e in plan:
+            assert 1 <= e.count <= s.chunk_size
+            assert e.start == s.computed(e.request)
+            assert e.sample == (e.start + e.count == total[e.request])
+            seen[e.request].append((e.start, e.count))
+        if on_step:
+            on_step(plan)
+        s.commit()
+        cm.check()
+        for e in plan:
+            if e.sample:
+                new[e.request] += 1
+                if new[e.request] >= reqs[e.request][1]:
+                    s.finish(e.request)
+                else:
+                    total[e.request] += 1
+                    s.append_token(e.request)
+        steps += 1
+        assert steps < max_steps
+    return seen, steps
+
+
+def test_portions_budget_and_mixing():
+    cm, s = make(budget=40, chunk=32)
+    s.add(0, 70, 3)
+    s.add(1, 10, 5)
+    plan, _ = s.schedule()
+    # request 0 gets a portion of 32; request 1's whole prompt (10) no longer fits the 8 left
+    assert [(e.request, e.start, e.count, e.sample) for e in plan] == [(0, 0, 32, False), (1, 0, 8, False)]
+    s.commit()
+    plan, _ = s.schedule()
+    assert [(e.request, e.start, e.count, e.sample) for e in plan] == [(0, 32, 32, False), (1, 8, 2, True)]
+    s.commit()
+    s.append_token(1)
+    plan, _ = s.schedule()
+    # a decode token of request 1 is planned first, beside the last portion of request 0
+    assert [(e.request, e.start, e.count, e.sample) for e in plan] == [(1, 10, 1, True), (0, 64, 6, True)]
+
+
+def test_every_token_is_processed_exactly_once():
+    cm, s = make(num_pages=64, budget=48, chunk=20)
+    reqs = {0: (70, 4), 1: (1, 9), 2: (33, 1), 3: (20, 6), 4: (47, 3), 5: (5, 5)}
+    for rid, (p, n) in reqs.items():
+        s.add(rid, p, n)
+    seen, _ = drive(s, cm, reqs)
+    for rid, (p, n) in reqs.items():
+        spans = [x for x in seen[rid] if x != "preempted"]
+        pos = 0
+        for start, count in spans:
+            assert start == pos
+            pos += count
+        assert pos == p + n - 1            # the last sampled token is never fed
+    assert cm.free_pages(0) == 64 and cm.live_requests() == 0
+
+
+def test_max_num_seqs_limits_admission():
+    cm, s = make(max_seqs=2, budget=1000, chunk=1000)
+    for rid in range(5):
+        s.add(rid, 8, 2)
+    plan, _ = s.schedule()
+    assert [e.request for e in plan] == [0, 1] and s.num_waiting() == 3
+
+
+def test_request_that_can_never_fit_is_refused():
+    cm, s = make(num_pages=4, page=16)
+    with pytest.raises(RequestTooLarge, match="cache pages"):
+        s.add(0, 60, 8)                    # 68 tokens need 5 pages
+    s.add(1, 60, 4)                        # 64 tokens fit exactly
+    with pytest.raises(SchedulerError, match="exists"):
+        s.add(1, 3, 3)
+    with pytest.raises(SchedulerError):
+        s.add(2, 0, 3)
+
+
+def test_admission_waits_for_pages():
+    cm, s = make(num_pages=6, page=16, budget=1000, chunk=1000)
+    s.add(0, 64, 16)                       # 4 pages now, a fifth later
+    s.add(1, 48, 4)                        # needs 3 pages: only 2 are left
+    plan, _ = s.schedule()
+    assert [e.request for e in plan] == [0] and s.num_waiting() == 1
+    s.commit()
+    s.finish(0)
+    plan, _ = s.schedule()
+    assert [e.request for e in plan] == [1] and cm.free_pages(0) == 3
+
+
+def test_out_of_pages_preempts_the_youngest_and_recomputes():
+    """Two requests fill the pool; when the older one needs another page the younger one is
+    preempted, waits at the head of the queue, and is later recomputed from its first token
+    (prompt and generated tokens alike)."""
+    cm, s = make(num_pages=4, page=16, budget=1000, chunk=1000)
+    reqs = {0: (30, 10), 1: (31, 20)}
+    for rid, (p, n) in reqs.items():
+        s.add(rid, p, n)
+    seen, _ = drive(s, cm, reqs)
+    assert "preempted" in seen[1] and "preempted" not in seen[0]
+    i = seen[1].index("preempted")
+    before, after = seen[1][:i], seen[1][i + 1:]
+    assert before[0] == (0, 31) and all(c == 1 for _, c in before[1:])
+    assert after[0][0] == 0 and after[0][1] == 31 + len(before) - 1 + 1   # all known tokens again
+    assert cm.free_pages(0) == 4
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_random_workloads_finish_and_free_everything(seed):
+    rng = random.Random(seed)
+    cm, s = make(num_pages=rng.choice([12, 20, 40]), page=rng.choice([4, 8, 16]), max_seqs=rng.choice([2, 4]),
+                 budget=rng.choice([16, 33, 64]), chunk=rng.choice([5, 16, 48]), window_pages=rng.choice([None, 40]))
+    cap = cm.groups[0].num_pages * cm.groups[0].page_size
+    reqs = {}
+    for rid in range(12):
+        p = rng.randrange(1, cap // 2)
+        n = rng.randrange(1, max(2, min(30, cap - p)))
+        reqs[rid] = (p, n)
+        s.add(rid, p, n)
+    seen, steps = drive(s, cm, reqs)
+    assert cm.live_requests() == 0
+    for g, grp in enumerate(cm.groups):
+        assert cm.free_pages(g) == grp.num_pages

@@ -60,3 +60,47 @@ int xi_cm_check(CacheManager* cm, char* why, int cap) {
 const char* xi_cm_last_error(CacheManager* cm) { return cm->last_error().c_str(); }
 
 }  // extern "C"
+
+// ---- scheduler -----------------------------------------------------------------------
+#include "scheduler.h"
+
+using xi::Scheduler;
+
+extern "C" {
+
+Scheduler* xi_sched_create(CacheManager* cm, int max_num_seqs, int max_batched_tokens, int chunk_size) {
+  return cm ? new Scheduler(cm, max_num_seqs, max_batched_tokens, chunk_size) : nullptr;
+}
+void xi_sched_destroy(Scheduler* s) { delete s; }
+int xi_sched_add(Scheduler* s, int64_t id, int64_t prompt_len, int64_t max_new_tokens) {
+  return s->add(id, prompt_len, max_new_tokens);
+}
+// Plans a step.  Writes up to cap entries and up to pre_cap preempted ids; returns the
+// number of entries (or -1 if cap is too small), *n_preempted the number of preempted.
+int xi_sched_schedule(Scheduler* s, int64_t* ids, int64_t* starts, int32_t* counts, int32_t* sample,
+                      int cap, int64_t* preempted, int pre_cap, int32_t* n_preempted) {
+  std::vector<int64_t> pre;
+  const auto& plan = s->schedule(&pre);
+  *n_preempted = (int32_t)pre.size();
+  for (int i = 0; i < (int)pre.size() && i < pre_cap; ++i) preempted[i] = pre[i];
+  if ((int)plan.size() > cap) return -1;
+  for (size_t i = 0; i < plan.size(); ++i) {
+    ids[i] = plan[i].id;
+    starts[i] = plan[i].start;
+    counts[i] = plan[i].count;
+    sample[i] = plan[i].sample;
+  }
+  return (int)plan.size();
+}
+void xi_sched_commit(Scheduler* s) { s->commit(); }
+int xi_sched_append_token(Scheduler* s, int64_t id) { return s->append_token(id); }
+int xi_sched_finish(Scheduler* s, int64_t id) { return s->finish(id); }
+int xi_sched_num_waiting(Scheduler* s) { return s->num_waiting(); }
+int xi_sched_num_running(Scheduler* s) { return s->num_running(); }
+int64_t xi_sched_computed(Scheduler* s, int64_t id) {
+  const xi::SchedRequest* r = s->find(id);
+  return r ? r->computed : -1;
+}
+const char* xi_sched_last_error(Scheduler* s) { return s->last_error().c_str(); }
+
+}  // extern "C"

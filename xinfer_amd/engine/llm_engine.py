@@ -1,0 +1,218 @@
+"""The engine: admits requests, runs the schedule-step-sample loop, returns outputs.
+
+Reference: LLMEngine (/root/reference/src/core/engine.rs): admission and the clipping of
+max_tokens 628-806, the loop prepare_step -> run_forward -> finish_step 1034-1151 and
+1363-1629, blocking generation generate_sync 1864-2011; finishing rules in
+Scheduler::postprocess (/root/reference/src/core/scheduler.rs:592-661): end-of-sequence
+token unless ignore_eos, max_tokens reached, max_model_len reached.  The end-of-sequence
+token is not part of the output, as in the reference.
+"""
+from __future__ import annotations
+
+import os
+import time
+from dataclasses import dataclass, field
+from typing import Dict, Iterable, List, Optional, Sequence, Union
+
+import torch
+
+from ..config.engine_config import EngineConfig, GenerationConfig, GenerationOutput, Message, SamplingParams
+from ..sampling import Sampler, Strategy, resolve_strategy, uniform
+from .loading import load_model, parse_dtype
+from .runner import ModelRunner, StepEntry
+from .scheduler import RequestTooLarge, Scheduler
+from .tokenizer import load_tokenizer
+
+DEFAULT_MAX_TOKENS = 16384      # /root/reference/src/core/engine.rs:650-678
+
+
+def _now_ms() -> int:
+    return int(time.time() * 1000)
+
+
+@dataclass
+class _Request:
+    rid: int
+    tokens: List[int]                  # prompt and generated tokens
+    prompt_len: int
+    max_tokens: int
+    params: SamplingParams
+    strategy: Strategy
+    seed: int
+    stream: int = 0                    # which stream of random numbers of that seed
+    prompt_start: int = 0
+    decode_start: int = 0
+    decode_finish: int = 0
+    finish_reason: str = ""
+    preemptions: int = 0
+
+    @property
+    def generated(self) -> List[int]:
+        return self.tokens[self.prompt_len:]
+
+
+class LLMEngine:
+    def __init__(self, econfig: EngineConfig, dtype="bf16"):
+        self.econfig = econfig
+        self.dtype = parse_dtype(dtype)
+        model_dir = econfig.model_dir()
+        self.model = load_model(model_dir, self.dtype, econfig.device)
+        spec = self.model.spec
+        self.max_model_len = min(econfig.max_model_len or spec.max_positions, spec.max_positions)
+        self.tokenizer = load_tokenizer(model_dir, spec.vocab_size)
+        self.eos_token_ids = set(spec.eos_token_ids) | set(self.tokenizer.eos_token_ids())
+        self.generation_cfg = econfig.generation_cfg or _read_generation_config(model_dir)
+        self.seed = econfig.seed if econfig.seed is not None else int.from_bytes(os.urandom(4), "little")
+        page = econfig.page_size
+        num_pages = econfig.num_pages or self._plan_pages(page)
+        self.runner = ModelRunner(self.model, page, num_pages, econfig.max_num_seqs)
+        budget = econfig.max_num_batched_tokens or max(econfig.prefill_chunk_size, econfig.max_num_seqs)
+        self.scheduler = Scheduler(self.runner.cache, econfig.max_num_seqs, budget,
+                                   econfig.prefill_chunk_size)
+        self.sampler = Sampler(self.model.device)
+        self._requests: Dict[int, _Request] = {}
+        self._finished: Dict[int, _Request] = {}
+        self._next_id = 0
+        self.steps = 0
+        self.num_preemptions = 0
+
+    # ---- memory -------------------------------------------------------------------
+    def _plan_pages(self, page: int) -> int:
+        """Pages per group from a share of the memory that is free after loading the
+        weights (the reference's kv_fraction, 0.6 by default on GPUs,
+        /root/reference/src/utils/kvcache_allocator.rs:336-346), capped by what
+        max_num_seqs requests of max_model_len tokens can use."""
+        free, _ = torch.cuda.mem_get_info(self.model.device)
+        frac = self.econfig.kv_fraction if self.econfig.kv_fraction is not None else 0.6
+        per_token = 0
+        esize = torch.tensor([], dtype=self.dtype).element_size()
+        for kv in self.model.kv_needs.values():
+            per_token += 2 * kv.num_kv_heads * kv.head_dim * esize
+        per_page = max(1, per_token * page)
+        by_memory = int(free * frac) // per_page
+        by_use = self.econfig.max_num_seqs * (-(-self.max_model_len // page))
+        return max(1, min(by_memory, by_use))
+
+    def get_available_kv_tokens(self) -> int:
+        return min(self.runner.cache.free_pages(g) for g in range(len(self.runner.cache.groups))) \
+            * self.econfig.page_size
+
+    # ---- admission --------------------------------------------------------------------
+    def add_request(self, prompt: Sequence[int], params: Optional[SamplingParams] = None) -> int:
+        """Admits a tokenised prompt; returns the request's id."""
+        params = params or SamplingParams()
+        prompt = [int(t) for t in prompt]
+        if not prompt:
+            raise ValueError("a prompt needs at least one token")
+        if len(prompt) > self.max_model_len - 1:          # engine.rs:639-647
+            raise ValueError(f"prompt of {len(prompt)} tokens exceeds max_model_len {self.max_model_len}")
+        vocab = self.model.spec.vocab_size
+        if min(prompt) < 0 or max(prompt) >= vocab:
+            raise ValueError(f"a prompt token is outside the vocabulary of {vocab}")
+        max_tokens = params.max_tokens or self.econfig.max_tokens or DEFAULT_MAX_TOKENS
+        max_tokens = max(1, min(max_tokens, self.max_model_len - len(prompt)))   # engine.rs:650-678
+        rid = self._next_id
+        self._next_id += 1
+        self.scheduler.add(rid, len(prompt), max_tokens)
+        # a request with a seed of its own draws from that seed's first stream whatever its
+        # id; otherwise from the engine's seed and a stream of its own
+        seed, stream = (params.seed, 0) if params.seed is not None else (self.seed, rid)
+        self._requests[rid] = _Request(
+            rid, prompt, len(prompt), max_tokens, params,
+            resolve_strategy(params, self.generation_cfg), seed, stream, prompt_start=_now_ms())
+        return rid
+
+    # ---- the loop ------------------------------------------------------------------------
+    def step(self) -> List[int]:
+        """One iteration: plan, run the batch, sample, finish.  Returns the ids that finished."""
+        plan, preempted = self.scheduler.schedule()
+        for rid in preempted:
+            self._requests[rid].preemptions += 1
+            self.num_preemptions += 1
+        if not plan:
+            if not self.scheduler.idle():
+                raise RuntimeError("the scheduler planned nothing although requests are waiting")
+            return []
+        entries, sampled = [], []
+        for e in plan:
+            r = self._requests[e.request]
+            toks = r.tokens[e.start:e.start + e.count]
+            entries.append(StepEntry(e.request, toks, [e.count - 1] if e.sample else []))
+            if e.sample:
+                sampled.append(r)
+        logits = self.runner.step(entries, reserved=True)
+        self.scheduler.commit()
+        self.steps += 1
+        done: List[int] = []
+        if sampled:
+            tokens = self.sampler.sample(
+                logits, [r.strategy for r in sampled],
+                [uniform(r.seed, r.stream, len(r.generated)) for r in sampled],
+                recent=[r.generated for r in sampled])
+            now = _now_ms()
+            for r, tok in zip(sampled, tokens):
+                if not r.generated:
+                    r.decode_start = now
+                reason = ""
+                if tok in self.eos_token_ids and not r.params.ignore_eos:
+                    reason = "eos"
+                else:
+                    r.tokens.append(int(tok))
+                    if len(r.generated) >= r.max_tokens:
+                        reason = "length"
+                    elif len(r.tokens) >= self.max_model_len:
+                        reason = "max_model_len"
+                    else:
+                        self.scheduler.append_token(r.rid)
+                if reason:
+                    r.finish_reason = reason
+                    r.decode_finish = now
+                    self.scheduler.finish(r.rid)
+                    self._finished[r.rid] = self._requests.pop(r.rid)
+                    done.append(r.rid)
+        return done
+
+    def run_until_done(self) -> None:
+        while not self.scheduler.idle():
+            self.step()
+
+    # ---- outputs ---------------------------------------------------------------------------
+    def _output(self, r: _Request) -> GenerationOutput:
+        gen = r.generated
+        return GenerationOutput(
+            seq_id=r.rid, prompt_length=r.prompt_len, prompt_start_time=r.prompt_start,
+            decode_start_time=r.decode_start, decode_finish_time=r.decode_finish,
+            decoded_length=len(gen), decode_output=self.tokenizer.decode(gen), token_ids=list(gen),
+            finish_reason=r.finish_reason)
+
+    def generate(self, prompts: Sequence[Union[str, Sequence[int]]],
+                 params: Union[SamplingParams, Sequence[SamplingParams], None] = None) -> List[GenerationOutput]:
+        """Prompts as text (tokenised with the model's tokenizer) or as token ids."""
+        if params is None or isinstance(params, SamplingParams):
+            params = [params or SamplingParams()] * len(prompts)
+        if len(params) != len(prompts):
+            raise ValueError("one SamplingParams per prompt is needed")
+        rids = []
+        for p, sp in zip(prompts, params):
+            ids = self.tokenizer.encode(p) if isinstance(p, str) else list(p)
+            rids.append(self.add_request(ids, sp))
+        self.run_until_done()
+        return [self._output(self._finished.pop(rid)) for rid in rids]
+
+    def generate_sync(self, params: Sequence[SamplingParams],
+                      message_list: Sequence[Sequence[Message]]) -> List[GenerationOutput]:
+        """The reference's blocking chat entry point (xinfer.pyi:199-205): every message list
+        is rendered with the chat template and completed."""
+        prompts = [self.tokenizer.apply_chat_template(list(m)) for m in message_list]
+        return self.generate(prompts, list(params))
+
+
+def _read_generation_config(model_dir: str) -> Optional[GenerationConfig]:
+    import json
+    path = os.path.join(model_dir, "generation_config.json")
+    if not os.path.isfile(path):
+        return None
+    with open(path, "r", encoding="utf-8") as f:
+        raw = json.load(f)
+    return GenerationConfig(raw.get("temperature"), raw.get("top_p"), raw.get("top_k"),
+                            raw.get("frequency_penalty"), raw.get("presence_penalty"))

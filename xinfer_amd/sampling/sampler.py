@@ -1,0 +1,136 @@
+"""Choice of the sampling strategy per request and the draw itself.
+
+Strategies and their precedence follow the reference: temperature below 1e-7 or absent
+means greedy (/root/reference/src/utils/logits_processor.rs:48-65); a request's own
+parameters come before the model's generation defaults, and with neither the default is
+top-k 32, top-p 0.95, temperature 0.7 (/root/reference/src/core/runner.rs:1803-1854).
+The reference picks one strategy per batch from its first sequence and draws from one
+shared generator; here every request has its own strategy and its own stream of random
+numbers (seed, request, number of tokens drawn so far), so a request's tokens do not
+depend on what it was batched with.
+"""
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+from typing import List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from .. import kernels
+from ..config.engine_config import GenerationConfig, SamplingParams
+
+PENALTY_CONTEXT = 128      # last generated tokens that penalties look at (runner.rs:1887-1912)
+_MASK = (1 << 64) - 1
+
+
+@dataclass(frozen=True)
+class Strategy:
+    temperature: float = 0.0    # 0: greedy
+    top_k: int = 0              # 0: no limit
+    top_p: float = 1.0          # 1: no limit
+    frequency_penalty: float = 0.0
+    presence_penalty: float = 0.0
+
+    @property
+    def greedy(self) -> bool:
+        return self.temperature < 1e-7
+
+
+def get_strategy(temperature: Optional[float], top_k: Optional[int], top_p: Optional[float]) -> Strategy:
+    """LogitsProcessor::get_strategy (logits_processor.rs:48-65)."""
+    if temperature is None or temperature < 1e-7:
+        return Strategy()
+    k = int(top_k) if (top_k is not None and top_k > 0) else 0
+    p = float(top_p) if top_p is not None else 1.0
+    return Strategy(float(temperature), k, p)
+
+
+def resolve_strategy(params: SamplingParams, defaults: Optional[GenerationConfig]) -> Strategy:
+    """Precedence of runner.rs:1803-1854."""
+    freq = params.frequency_penalty if params.frequency_penalty is not None else \
+        (defaults.frequency_penalty if defaults else None)
+    pres = params.presence_penalty if params.presence_penalty is not None else \
+        (defaults.presence_penalty if defaults else None)
+    has_user = (params.temperature is not None or (params.top_k is not None and params.top_k > 0)
+                or (params.top_p is not None and 0.0 < params.top_p < 1.0))
+    if params.temperature is not None and params.temperature == 0.0:
+        s = Strategy()
+    elif has_user:
+        s = get_strategy(params.temperature, params.top_k, params.top_p)
+    elif defaults is not None and defaults.temperature is not None and (
+            defaults.top_k is not None or defaults.top_p is not None):
+        s = get_strategy(defaults.temperature, defaults.top_k, defaults.top_p)
+    else:
+        s = Strategy(0.7, 32, 0.95)
+    return Strategy(s.temperature, s.top_k, s.top_p, float(freq or 0.0), float(pres or 0.0))
+
+
+def uniform(seed: int, request: int, draw: int) -> float:
+    """The draw-th uniform number in [0, 1) of a request's stream: splitmix64 of the three
+    counters, 24 bits kept so that the float32 value is exact."""
+    x = (seed * 0x9E3779B97F4A7C15 + request * 0xBF58476D1CE4E5B9 + draw * 0x94D049BB133111EB + 0x2545F4914F6CDD1D) & _MASK
+    for _ in range(2):
+        x = (x + 0x9E3779B97F4A7C15) & _MASK
+        z = x
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _MASK
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _MASK
+        x = z ^ (z >> 31)
+    return (x >> 40) / float(1 << 24)
+
+
+class Sampler:
+    """Draws one token per row of float32 logits on the GPU."""
+
+    def __init__(self, device):
+        self.device = torch.device(device)
+        lib = kernels.lib()
+        self._lib = lib
+
+    def argmax(self, logits: torch.Tensor) -> torch.Tensor:
+        kernels._dev(logits)
+        kernels._want(logits, torch.float32, "argmax: logits")
+        out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
+        kernels._ok(self._lib.xi_argmax(kernels._p(logits), logits.shape[0], logits.shape[1],
+                                        kernels._p(out), kernels._stream()))
+        return out
+
+    def sample(self, logits: torch.Tensor, strategies: Sequence[Strategy], uniforms: Sequence[float],
+               recent: Optional[Sequence[Sequence[int]]] = None) -> List[int]:
+        """logits float32 [R, V] (changed in place when penalties apply); one strategy and
+        one uniform number per row; `recent[r]` = the row's last generated tokens, for the
+        penalties.  Returns R token ids."""
+        kernels._dev(logits)
+        kernels._want(logits, torch.float32, "sample: logits")
+        R, V = logits.shape
+        if R != len(strategies) or R != len(uniforms):
+            raise kernels.KernelError("sample: one strategy and one uniform number per row are needed")
+        if R == 0:
+            return []
+        dev = logits.device
+        if recent is not None and any((s.frequency_penalty or s.presence_penalty) and len(rc) > 1
+                                      for s, rc in zip(strategies, recent)):
+            n = PENALTY_CONTEXT
+            rec = np.full((R, n), -1, dtype=np.int32)
+            fr = np.zeros(R, dtype=np.float32)
+            pr = np.zeros(R, dtype=np.float32)
+            for r, (s, rc) in enumerate(zip(strategies, recent)):
+                rc = list(rc)[-n:]
+                if len(rc) > 1:                      # logits_processor.rs:395
+                    rec[r, :len(rc)] = rc
+                    fr[r], pr[r] = s.frequency_penalty, s.presence_penalty
+            rec_d, fr_d, pr_d = (torch.from_numpy(a).to(dev) for a in (rec, fr, pr))
+            kernels._ok(self._lib.xi_apply_penalties(kernels._p(logits), R, V, kernels._p(rec_d), n,
+                                                     kernels._p(fr_d), kernels._p(pr_d), kernels._stream()))
+        if all(s.greedy for s in strategies):
+            return self.argmax(logits).tolist()
+        t = torch.tensor([s.temperature for s in strategies], dtype=torch.float32, device=dev)
+        k = torch.tensor([s.top_k for s in strategies], dtype=torch.int32, device=dev)
+        p = torch.tensor([s.top_p for s in strategies], dtype=torch.float32, device=dev)
+        u = torch.tensor(list(uniforms), dtype=torch.float32, device=dev)
+        probs = torch.empty_like(logits)
+        out = torch.empty((R,), dtype=torch.int32, device=dev)
+        kernels._ok(self._lib.xi_sample(kernels._p(logits), R, V, kernels._p(t), kernels._p(k), kernels._p(p),
+                                        kernels._p(u), kernels._p(probs), kernels._p(out), kernels._stream()))
+        return out.tolist()
