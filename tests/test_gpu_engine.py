@@ -165,8 +165,10 @@ def test_preemption_gives_the_same_tokens(model_dirs):
     assert [o.token_ids for o in got] == want
     assert tight.num_preemptions > 0 and roomy.num_preemptions == 0
     assert tight.get_available_kv_tokens() == 8 * 16
+    # a request that could never fit, even alone, is refused when it is added
+    small = _engine(model_dirs["A"], "A", "f32", max_num_seqs=2, num_pages=4)
     with pytest.raises(Exception, match="cache pages"):
-        tight.generate([harness.random_prompt(rng, 100, 256)], SamplingParams(max_tokens=60))
+        small.generate([harness.random_prompt(rng, 60, 256)], SamplingParams(max_tokens=30))
 
 
 def test_eos_and_limits(model_dirs):

@@ -58,6 +58,7 @@ def _bind(lib):
         "xi_cm_block_table": (i, [vp, i64, i, _I32P, i]),
         "xi_cm_check": (i, [vp, ctypes.c_char_p, i]),
         "xi_cm_last_error": (ctypes.c_char_p, [vp]),
+        "xi_cm_max_table_len": (i, [vp, i, _I64P]),
         "xi_cm_build_batch": (i, [vp, i, _I64P, _I32P, _I32P, _I32P, _I32P, _I32P, _I32P,
                                   _I64P, _I32P, i, i]),
     }
@@ -179,13 +180,11 @@ class PagedCacheManager:
         B = len(rids)
         T = int(sum(n_tokens))
         G = len(self.groups)
-        if max_pages is None:
-            max_pages = 1
-            for g, grp in enumerate(self.groups):
-                for rid, n in zip(rids, n_tokens):
-                    need = -(-(self.length(rid) + n) // grp.page_size)
-                    max_pages = max(max_pages, need)
         ids = np.asarray(rids, dtype=np.int64)
+        if max_pages is None:
+            max_pages = self._lib.xi_cm_max_table_len(self._h, B, ids.ctypes.data_as(_I64P))
+            if max_pages < 0:
+                raise CacheError("cannot build the batch: a request is not live")
         nt = np.asarray(n_tokens, dtype=np.int32)
         out = BatchArrays(
             num_tokens=T, num_seqs=B, max_pages=int(max_pages),

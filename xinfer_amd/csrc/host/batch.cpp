@@ -11,6 +11,17 @@ using xi::RequestPages;
 
 extern "C" {
 
+// The longest block table among the given requests, over all groups (at least 1).
+int xi_cm_max_table_len(CacheManager* cm, int B, const int64_t* ids) {
+  size_t longest = 1;
+  for (int b = 0; b < B; ++b) {
+    const RequestPages* r = cm->find(ids[b]);
+    if (!r) return -1;
+    for (const auto& t : r->tables) longest = t.size() > longest ? t.size() : longest;
+  }
+  return (int)longest;
+}
+
 // Fills, for B entries with T tokens in total:
 //   positions[T], tok_seq[T], cu_q[B+1], ctx_lens[B], state_slots[B]
 //   slots[G][T]                     cache slot of each new token per group

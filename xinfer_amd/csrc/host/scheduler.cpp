@@ -119,7 +119,10 @@ void Scheduler::commit() {
   for (const SchedEntry& e : plan_) {
     auto it = requests_.find(e.id);
     if (it == requests_.end() || !it->second.running) continue;
-    cm_->commit(e.id, e.count);
+    if (cm_->commit(e.id, e.count) < 0) {
+      error_ = cm_->last_error();
+      continue;
+    }
     it->second.computed += e.count;
   }
   plan_.clear();

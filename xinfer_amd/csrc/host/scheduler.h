@@ -52,7 +52,7 @@ class Scheduler {
   // Plans one step and reserves its pages.  Ids preempted while planning are appended to
   // `preempted`.
   const std::vector<SchedEntry>& schedule(std::vector<int64_t>* preempted);
-  // The planned step ran: its tokens are in the cache.
+  // The planned step ran: its tokens are in the cache (recorded in the cache manager too).
   void commit();
   // A sampled token joins the request's known tokens.  -1 if unknown or beyond max_len.
   int append_token(int64_t id);

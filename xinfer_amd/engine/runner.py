@@ -86,8 +86,9 @@ class ModelRunner:
     # ---- the step -----------------------------------------------------------------
     def step(self, entries: Sequence[StepEntry], reserved: bool = False) -> torch.Tensor:
         """Runs the entries' tokens as one batch.  Returns float32 [wanted, vocab] in the
-        order of the entries and of each entry's `want`.  With `reserved` the caller has
-        reserved the pages already (the scheduler does)."""
+        order of the entries and of each entry's `want`.  With `reserved` the caller (the
+        scheduler) has reserved the pages already and also records afterwards that the
+        tokens are in the cache; without it this call does both."""
         spec = self.model.spec
         if not entries:
             return torch.empty((0, spec.vocab_size), dtype=torch.float32, device=self.device)
@@ -119,20 +120,16 @@ class ModelRunner:
         if ids_host.min() < 0 or ids_host.max() >= spec.vocab_size:
             raise StepError(f"a token id is outside the vocabulary of {spec.vocab_size}")
         if not reserved:
-            done = []
-            try:
-                for rid, n in zip(rids, counts):
-                    self.cache.reserve(rid, n)
-                    done.append(rid)
-            except OutOfPages:
-                raise
+            for rid, n in zip(rids, counts):
+                self.cache.reserve(rid, n)      # OutOfPages leaves every request's length as it was
         arrays = self.cache.build_batch(rids, counts)
         ctx = self._context(arrays)
         ids = torch.from_numpy(ids_host.astype(np.int32)).to(self.device)
         want_rows = torch.tensor(rows, dtype=torch.int32, device=self.device)
         logits = self.model.forward(ids, ctx, self.layer_caches, want_rows)
-        for rid, n in zip(rids, counts):
-            self.cache.commit(rid, n)
+        if not reserved:
+            for rid, n in zip(rids, counts):
+                self.cache.commit(rid, n)
         return logits
 
     def _context(self, a: BatchArrays) -> StepContext:
