@@ -1,0 +1,186 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine at Qwen3-8B layer sizes on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line.  `value` is decoded tokens per second at batch 8 and the context
+length the configuration names (the last timed step ends at that length); a "step" is one
+decode step through the engine's own step function (mixed-batch path, paged cache,
+kernels) followed by greedy sampling on the GPU.  Beside it: the prefill of one
+2,048-token prompt, the decode step's bandwidth roofline, and decode at batch 1 and 64.
+
+Data is synthetic: weights are seeded random values of the architecture's shapes made
+on the GPU, token ids are seeded uniform, and the cache contents the decode steps read
+are random values (decode timing does not depend on what the cache holds).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+# MI355X published peaks
+HBM_GBPS = 8000.0
+PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "fp32": 157.3}
+
+QWEN3_8B = dict(
+    architectures=["Qwen3ForCausalLM"], hidden_size=4096, intermediate_size=12288,
+    num_hidden_layers=36, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+    vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False,
+    max_position_embeddings=40960, hidden_act="silu")
+FULL_LAYERS = QWEN3_8B["num_hidden_layers"]
+CONTEXT = 4096
+PREFILL_TOKENS = 2048
+
+
+def weight_bytes(cfg, esize=2):
+    h, i, nq, nkv, d, v, L = (cfg.hidden_size, cfg.intermediate_size, cfg.num_attention_heads,
+                              cfg.num_key_value_heads, cfg.head_dim, cfg.vocab_size, cfg.num_hidden_layers)
+    per_layer = (nq + 2 * nkv) * d * h + h * nq * d + 2 * i * h + h * i
+    return (L * per_layer + v * h) * esize          # every linear weight once, and the head
+
+
+def kv_bytes_per_token(cfg, esize=2):
+    return 2 * cfg.num_key_value_heads * cfg.head_dim * esize * cfg.num_hidden_layers
+
+
+def prefill_flops(cfg, T):
+    h, i, nq, nkv, d, v, L = (cfg.hidden_size, cfg.intermediate_size, cfg.num_attention_heads,
+                              cfg.num_key_value_heads, cfg.head_dim, cfg.vocab_size, cfg.num_hidden_layers)
+    per_layer = (nq + 2 * nkv) * d * h + h * nq * d + 2 * i * h + h * i
+    linear = 2.0 * T * L * per_layer + 2.0 * v * h          # the head runs on one row
+    attn = L * 4.0 * nq * d * (T * (T + 1) / 2.0)           # causal QK^T and PV
+    return linear + attn
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS,
+                    help="fewer layers than the configuration has (reported in config)")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--skip-points", action="store_true", help="only the default decode run")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+    from xinfer_amd.engine import ModelRunner, StepEntry, build_model
+    from xinfer_amd.models import config_from_dict
+    from xinfer_amd.sampling import Sampler
+    from xinfer_amd.weights.random_init import random_store_for
+
+    dev = "cuda:0"
+    raw = dict(QWEN3_8B, num_hidden_layers=args.layers)
+    _, cfg = config_from_dict(raw)
+    store = random_store_for(cfg, seed=0, linear_std=0.02, norm_std=0.1)
+    t0 = time.time()
+    model = build_model(cfg, store, "bf16", dev)
+    torch.cuda.synchronize()
+    print(f"[bench] model of {args.layers} layers built in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
+
+    page = 64
+    max_batch = 8 if args.skip_points else 64
+    max_batch = max(max_batch, args.batch)
+    num_pages = max_batch * (CONTEXT // page) + PREFILL_TOKENS // page + 8
+    runner = ModelRunner(model, page_size=page, num_pages=num_pages, max_requests=max_batch + 1)
+    g = torch.Generator(device=dev)
+    g.manual_seed(1)
+    for lc in runner.layer_caches.values():          # random cache contents for the decode runs
+        lc.k.copy_(torch.randn(lc.k.shape, generator=g, device=dev, dtype=torch.float32).to(lc.k.dtype))
+        lc.v.copy_(torch.randn(lc.v.shape, generator=g, device=dev, dtype=torch.float32).to(lc.v.dtype))
+    sampler = Sampler(dev)
+    cpu_gen = torch.Generator().manual_seed(2)
+
+    def sync():
+        torch.cuda.synchronize()
+
+    def decode_run(batch, steps, warmup):
+        """`batch` requests whose caches already hold CONTEXT - steps - warmup tokens decode
+        steps + warmup tokens, so that the last timed step ends at CONTEXT."""
+        start = CONTEXT - steps - warmup
+        rids = list(range(100, 100 + batch))
+        for rid in rids:
+            runner.add_request(rid)
+            runner.cache.reserve(rid, start)
+            runner.cache.commit(rid, start)
+        toks = torch.randint(0, cfg.vocab_size, (batch,), generator=cpu_gen).tolist()
+
+        def one(toks):
+            logits = runner.step([StepEntry(r, [t], [0]) for r, t in zip(rids, toks)])
+            return sampler.argmax(logits).tolist()
+
+        for _ in range(warmup):
+            toks = one(toks)
+        sync()
+        t = time.perf_counter()
+        for _ in range(steps):
+            toks = one(toks)
+        sync()
+        dt = time.perf_counter() - t
+        for rid in rids:
+            runner.release(rid)
+        return dt / steps
+
+    def prefill_run(reps=3):
+        ids = torch.randint(0, cfg.vocab_size, (PREFILL_TOKENS,), generator=cpu_gen).tolist()
+        best = None
+        for _ in range(reps + 1):                  # the first run warms up
+            runner.add_request(7)
+            sync()
+            t = time.perf_counter()
+            logits = runner.step([StepEntry(7, ids, [PREFILL_TOKENS - 1])])
+            sampler.argmax(logits).tolist()
+            sync()
+            dt = time.perf_counter() - t
+            runner.release(7)
+            best = dt if best is None else min(best, dt)
+        return best
+
+    sec = decode_run(args.batch, args.steps, args.warmup)
+    wb, kvb = weight_bytes(cfg), kv_bytes_per_token(cfg)
+    # mean cache length over the timed steps (it grows by one each step, ending at CONTEXT)
+    mean_ctx = CONTEXT - (args.steps - 1) / 2.0
+    step_bytes = wb + args.batch * mean_ctx * kvb
+    achieved = step_bytes / sec / 1e9
+    out = {
+        "metric": "decode tok/s at batch 8, Qwen3-8B bf16", "value": round(args.batch / sec, 2),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic: seeded random weights, uniform random token ids, random cache contents",
+        "config": {
+            "model": "Qwen3-8B layer sizes", "global_batch": args.batch, "seq_len": CONTEXT,
+            "parallelism": "single GPU", "layers": args.layers, "layers_of_model": FULL_LAYERS,
+            "hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size,
+            "num_attention_heads": cfg.num_attention_heads, "num_key_value_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size, "rope_theta": cfg.rope_theta,
+            "rms_norm_eps": cfg.rms_norm_eps, "tie_word_embeddings": cfg.tie_word_embeddings,
+            "page_size": page, "prefill_tokens": PREFILL_TOKENS, "kv_dtype": "bf16"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_GBPS, 4)},
+    }
+    print(f"[bench] decode b{args.batch}: {sec * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
+    psec = prefill_run()
+    flops = prefill_flops(cfg, PREFILL_TOKENS)
+    out["prefill"] = {"value": round(PREFILL_TOKENS / psec, 1), "tokens": PREFILL_TOKENS,
+                      "ms": round(psec * 1e3, 3),
+                      "frac": round(flops / psec / (PEAK_TFLOPS["bf16"] * 1e12), 4)}
+    print(f"[bench] prefill {PREFILL_TOKENS}: {psec * 1e3:.2f} ms", file=sys.stderr, flush=True)
+    if not args.skip_points:
+        points = {}
+        for b in (1, 64):
+            s = decode_run(b, max(8, args.steps // 2), max(2, args.warmup // 2))
+            points[f"decode_b{b}"] = round(b / s, 2)
+            print(f"[bench] decode b{b}: {s * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
+        out["points"] = points
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -166,6 +166,13 @@ def test_qk_norm_rope_kv(dtype, nq, nkv, d, rot, interleaved, norm):
         p, o = int(slots[t]) // page, int(slots[t]) % page
         assert (kcd[p, :, o] - k[t]).abs().max() / k.abs().max() < tol, t
         assert torch.equal(vcd[p, :, o].double(), v[t]), t
+    # the transposed V pool [pages, nkv, d, page] holds the same values
+    vt = torch.zeros((pages, nkv, d, page), dtype=dtype, device=DEV)
+    kernels.qk_norm_rope_kv(
+        qkv.to(DEV), qw.to(DEV) if norm else None, kw.to(DEV) if norm else None, eps, cos.to(DEV),
+        sin.to(DEV), rot, interleaved, positions.to(DEV), slots.to(DEV), kc.to(DEV), vt, nq, nkv, d,
+        v_transposed=True)
+    assert torch.equal(vt.cpu().transpose(2, 3), vcd)
     # nothing but the named slots was written
     touched = torch.zeros(pages * page, dtype=torch.bool)
     touched[slots] = True
@@ -262,3 +269,102 @@ def test_attention_far_key_stands_out(dtype):
                                     scale, 0)
     err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
     assert err < _tol(dtype, 2), err
+
+
+# ---- the matrix-core attention kernels (bfloat16, V transposed in the cache) -------------------
+def _mfma_inputs(case):
+    return (torch.cat(case["qs"]).contiguous().to(DEV), case["kc"].to(DEV),
+            case["vc"].transpose(2, 3).contiguous().to(DEV), case["bt"].to(DEV))
+
+
+def _cu_ctx(seqs):
+    cu = [0]
+    for _, n in seqs:
+        cu.append(cu[-1] + n)
+    return (torch.tensor(cu, dtype=torch.int32), torch.tensor([c for c, _ in seqs], dtype=torch.int32))
+
+
+PREFILL_CASES = ATTN_CASES + [
+    (8, 2, 128, 64, 0, [(2048, 300), (129, 129), (640, 2)]),     # a cached prefix before the portion
+    (4, 1, 64, 16, 100, [(500, 260), (99, 99), (101, 3)]),       # window crossing block borders
+    (6, 3, 96, 8, 0, [(257, 257)]),
+    (2, 1, 16, 8, 5, [(40, 40), (6, 1)]),
+    (16, 1, 32, 32, 0, [(77, 33)]),                               # group of 16
+]
+
+
+@pytest.mark.parametrize("nq,nkv,d,page,window,seqs", PREFILL_CASES)
+def test_attention_prefill_mfma(nq, nkv, d, page, window, seqs):
+    from xinfer_amd import kernels
+    if page % 8:
+        pytest.skip("the matrix-core kernels need pages of a multiple of 8 tokens")
+    g = torch.Generator().manual_seed(21)
+    case = _paged_case(g, torch.bfloat16, nq, nkv, d, page, seqs)
+    scale = 1.0 / math.sqrt(d)
+    ref = _attention_ref(case, seqs, window, scale)
+    q, kc, vt, bt = _mfma_inputs(case)
+    cu, ctx = _cu_ctx(seqs)
+    qb = kernels.prefill_block(d)
+    tiles = torch.tensor([(b, q0) for b, (_, n) in enumerate(seqs) for q0 in range(0, n, qb)], dtype=torch.int32)
+    out = kernels.attention_prefill_bf16(q, kc, vt, bt, tiles.to(DEV), cu.to(DEV), ctx.to(DEV), scale, window)
+    err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
+    assert err < _tol(torch.bfloat16, 2), err
+    # the generic kernel reads the transposed pool too
+    out2 = kernels.attention_generic(q, kc, vt, bt, case["tok_seq"].to(DEV), case["positions"].to(DEV), scale,
+                                     window, v_transposed=True)
+    err = (out2.cpu().double() - ref).abs().max() / ref.abs().max()
+    assert err < _tol(torch.bfloat16, 2), err
+
+
+DECODE_CASES = [
+    (4, 2, 32, 16, 0, [(5, 1), (17, 1), (33, 1), (1, 1)]),
+    (6, 2, 16, 8, 0, [(200, 1), (130, 1), (513, 1)]),
+    (5, 5, 48, 16, 24, [(100, 1), (24, 1), (25, 1), (7, 1)]),
+    (32, 8, 128, 64, 0, [(4096, 1), (1, 1), (257, 1), (256, 1), (1025, 1)]),
+    (8, 2, 128, 64, 300, [(2000, 1), (299, 1), (301, 1), (600, 1)]),
+    (16, 1, 64, 8, 0, [(700, 1)]),
+    (2, 2, 256, 16, 0, [(70, 1), (300, 1)]),
+]
+
+
+@pytest.mark.parametrize("nq,nkv,d,page,window,seqs", DECODE_CASES)
+def test_attention_decode_mfma(nq, nkv, d, page, window, seqs):
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(22)
+    case = _paged_case(g, torch.bfloat16, nq, nkv, d, page, seqs)
+    scale = 1.0 / math.sqrt(d)
+    ref = _attention_ref(case, seqs, window, scale)
+    q, kc, vt, bt = _mfma_inputs(case)
+    _, ctx = _cu_ctx(seqs)
+    out = kernels.attention_decode_bf16(q, kc, vt, bt, ctx.to(DEV), int(ctx.max()), scale, window)
+    err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
+    assert err < _tol(torch.bfloat16, 2), err
+
+
+def test_attention_mfma_far_key_and_page_edges():
+    """One key is made to win the softmax, placed in turn at a page's first and last offset,
+    at the first key, and just before the query: decode and prefill kernels must return its
+    value row; a kernel that drops or misplaces a key returns something else."""
+    from xinfer_amd import kernels
+    nq, nkv, d, page = 8, 2, 128, 64
+    scale = 1.0 / math.sqrt(d)
+    for far in (0, 63, 64, 127, 511, 512, 1150, 1198):
+        g = torch.Generator().manual_seed(23)
+        seqs = [(1200, 1)]
+        case = _paged_case(g, torch.bfloat16, nq, nkv, d, page, seqs)
+        qv = case["qs"][0]
+        for kvh in range(nkv):
+            kfar = (qv[0, kvh * 4].float() / qv[0, kvh * 4].float().norm() * 60).to(torch.bfloat16)
+            case["ks"][0][far, kvh] = kfar
+            phys, off = int(case["bt"][0, far // page]), far % page
+            case["kc"][phys, kvh, off] = kfar
+        ref = _attention_ref(case, seqs, 0, scale)
+        assert (ref[0, :d] - case["vs"][0][far, 0].double()).abs().max() < 0.05
+        q, kc, vt, bt = _mfma_inputs(case)
+        _, ctx = _cu_ctx(seqs)
+        out = kernels.attention_decode_bf16(q, kc, vt, bt, ctx.to(DEV), 1200, scale, 0)
+        assert (out.cpu().double() - ref).abs().max() / ref.abs().max() < _tol(torch.bfloat16, 2), far
+        cu = torch.tensor([0, 1], dtype=torch.int32)
+        tiles = torch.tensor([[0, 0]], dtype=torch.int32)
+        out = kernels.attention_prefill_bf16(q, kc, vt, bt, tiles.to(DEV), cu.to(DEV), ctx.to(DEV), scale, 0)
+        assert (out.cpu().double() - ref).abs().max() / ref.abs().max() < _tol(torch.bfloat16, 2), far

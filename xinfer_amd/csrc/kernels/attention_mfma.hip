@@ -1,0 +1,407 @@
+// bfloat16 paged causal GQA attention on the gfx950 matrix cores, for prefill and decode.
+//
+// Both kernels are built on one wave-level step: 32 keys against NQT tiles of 16 query
+// columns, with v_mfma_f32_16x16x32_bf16 and no transposes through LDS:
+//
+//   S^T[key, q] = K[key, :] . Q[q, :]          A = K rows      B = Q^T
+//   O^T[d, q]  += V^T[d, key] * P^T[key, q]    A = V^T rows    B = P^T
+//
+// A-operand lane l holds row l%16 and 8 contiguous elements of the contraction index
+// (group l/16); B-operand lane l holds column l%16 and the same 8 elements; the 16x16
+// result has lane l holding column l%16, rows 4*(l/16)..+3.  So a lane's S^T results are
+// 4 consecutive keys of its own query column, which is exactly a B operand of the second
+// product once rounded to bfloat16 - provided the V^T operand pairs the same keys with the
+// same slots.  Row m of the two K tiles of a step is therefore key 8*(m/4) + m%4 (tile 0)
+// and that + 4 (tile 1): lane group j then holds keys 8j..8j+7, one 16-byte load from V^T.
+//
+// The cache keeps K as [page, kv_head, offset, d] and V transposed as
+// [page, kv_head, d, offset], so both operands are read from global memory in the layout
+// the matrix cores want.  Softmax runs in float32 (exp2 with log2(e) folded into the
+// scale); all per-query state (running max, sum, correction) lives in the lanes of that
+// query's column.
+//
+// Reference: PagedAttention::forward, /root/reference/src/models/layers/attention.rs:947-958
+// (varlen prefill over cu_seqlens with a cached prefix; decode with split-K, workspace
+// /root/reference/src/utils/kvcache_allocator.rs:662-673); golden formula
+// /root/reference/tests/probes/compare_flashinfer_probe.py:51-73.
+#include "common.h"
+
+namespace xi {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+__device__ __forceinline__ bf16x8 load8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
+__device__ __forceinline__ bf16x8 zero8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.f;
+  return z;
+}
+
+struct PagedKV {
+  const bf16* k;    // [pages, nkv, page, d]
+  const bf16* vt;   // [pages, nkv, d, page]
+  const int* bt;    // this sequence's block table
+  int page, nkv, d, kvh;
+};
+
+// Per-wave attention state for NQT column tiles and up to DT*16 output dims.
+template <int KC, int DT, int NQT>
+struct WaveAttn {
+  bf16x8 qb[NQT][KC];   // Q^T operands
+  f32x4 acc[DT][NQT];   // O^T accumulators
+  float m[NQT], l[NQT]; // running max (log2 domain) and per-lane partial sums
+  int qpos[NQT];        // position of this lane's query column (-1: no query)
+  int qlo[NQT];         // first key the query sees
+
+  __device__ __forceinline__ void init() {
+#pragma unroll
+    for (int ct = 0; ct < NQT; ++ct) {
+      m[ct] = -INFINITY;
+      l[ct] = 0.f;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) acc[dt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+  }
+
+  // q_row: pointer to this lane's query row (d elements) per column tile, or null.
+  __device__ __forceinline__ void load_q(const bf16* const* q_rows, int d, int j) {
+#pragma unroll
+    for (int ct = 0; ct < NQT; ++ct)
+#pragma unroll
+      for (int c = 0; c < KC; ++c) {
+        const int off = 32 * c + 8 * j;
+        qb[ct][c] = (q_rows[ct] && off < d) ? load8(q_rows[ct] + off) : zero8();
+      }
+  }
+
+  // Keys k_base .. k_base+31 (k_base a multiple of 32).  k_last: last key of the sequence
+  // that exists in the cache (addresses are clamped to it).  masked: some key of the step
+  // may be hidden from some query (else the mask arithmetic is skipped).
+  __device__ __forceinline__ void step(const PagedKV& kv, int k_base, int k_last, float scale_log2,
+                                       bool masked, int r, int j) {
+    const int d = kv.d;
+    // ---- K operands: tile 0 row r <-> key k_base + 8*(r/4) + r%4, tile 1 that + 4
+    int kgrp = k_base + 8 * (r >> 2);
+    if (kgrp > k_last) kgrp = k_last & ~7;
+    const int kpage = kv.bt[kgrp / kv.page];
+    const bf16* kp = kv.k + (((size_t)kpage * kv.nkv + kv.kvh) * kv.page + (kgrp % kv.page) + (r & 3)) * d;
+    bf16x8 ka[2][KC];
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+      const int off = 32 * c + 8 * j;
+      if (off < d) {
+        ka[0][c] = load8(kp + off);
+        ka[1][c] = load8(kp + 4 * d + off);
+      } else {
+        ka[0][c] = zero8();
+        ka[1][c] = zero8();
+      }
+    }
+    // ---- V^T operands: row 16*dt + r, keys k_base + 8j .. +7
+    int vgrp = k_base + 8 * j;
+    if (vgrp > k_last) vgrp = k_last & ~7;
+    const int vpage = kv.bt[vgrp / kv.page];
+    const bf16* vp = kv.vt + (((size_t)vpage * kv.nkv + kv.kvh) * d + r) * kv.page + (vgrp % kv.page);
+    bf16x8 va[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) va[dt] = (16 * dt < d) ? load8(vp + (size_t)16 * dt * kv.page) : zero8();
+
+    bf16x8 pb[NQT];
+#pragma unroll
+    for (int ct = 0; ct < NQT; ++ct) {
+      f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < KC; ++c) {
+        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[0][c], qb[ct][c], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[1][c], qb[ct][c], s1, 0, 0, 0);
+      }
+      float s[8];
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        s[v] = s0[v] * scale_log2;
+        s[4 + v] = s1[v] * scale_log2;
+      }
+      if (masked) {
+        const int key0 = k_base + 8 * j;
+#pragma unroll
+        for (int v = 0; v < 8; ++v) {
+          const int key = key0 + v;
+          if (key > qpos[ct] || key < qlo[ct]) s[v] = -INFINITY;
+        }
+      }
+      float mx = s[0];
+#pragma unroll
+      for (int v = 1; v < 8; ++v) mx = fmaxf(mx, s[v]);
+      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      const float m_new = fmaxf(m[ct], mx);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float corr = __builtin_amdgcn_exp2f(m[ct] - m_safe);
+      float psum = 0.f;
+#pragma unroll
+      for (int v = 0; v < 8; ++v) {
+        const float p = __builtin_amdgcn_exp2f(s[v] - m_safe);
+        psum += p;
+        pb[ct][v] = (__bf16)p;
+      }
+      l[ct] = l[ct] * corr + psum;
+      m[ct] = m_new;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        acc[dt][ct][0] *= corr;
+        acc[dt][ct][1] *= corr;
+        acc[dt][ct][2] *= corr;
+        acc[dt][ct][3] *= corr;
+      }
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int ct = 0; ct < NQT; ++ct)
+        acc[dt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt], pb[ct], acc[dt][ct], 0, 0, 0);
+  }
+
+  // Sum of a column's per-lane partial sums over the four lane groups.
+  __device__ __forceinline__ float total_l(int ct) const {
+    float t = l[ct] + __shfl_xor(l[ct], 16, kWave);
+    return t + __shfl_xor(t, 32, kWave);
+  }
+};
+
+// =====================================================================================
+// Prefill (and mixed batches): one workgroup of 4 waves per (query block, query head);
+// each wave owns NQT*16 consecutive query tokens and walks the keys they can see.
+//   tiles[i] = {sequence, first query token of the block within the sequence's portion}
+// =====================================================================================
+template <int KC, int DT, int NQT>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ vt_cache,
+    const int* __restrict__ block_tables, int max_pages, const int* __restrict__ tiles,
+    const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, bf16* __restrict__ out,
+    float scale_log2, int window, int page, int nq, int nkv, int d) {
+  constexpr int QW = 16 * NQT;  // queries per wave
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, j = lane >> 4;
+  const int seq = tiles[2 * blockIdx.x], q0_blk = tiles[2 * blockIdx.x + 1];
+  const int head = blockIdx.y;
+  const int q_begin = cu_q[seq], q_len = cu_q[seq + 1] - q_begin;
+  const int ctx = ctx_lens[seq];
+  const int q0 = q0_blk + wave * QW;  // first query of this wave within the portion
+  if (q0 >= q_len) return;
+  const int pos0 = ctx - q_len;  // position of the portion's first token
+
+  PagedKV kv{k_cache, vt_cache, block_tables + (size_t)seq * max_pages, page, nkv, d, head / (nq / nkv)};
+  WaveAttn<KC, DT, NQT> w;
+  w.init();
+  const bf16* q_rows[NQT];
+#pragma unroll
+  for (int ct = 0; ct < NQT; ++ct) {
+    const int qi = q0 + 16 * ct + r;
+    const bool ok = qi < q_len;
+    w.qpos[ct] = ok ? pos0 + qi : -1;
+    w.qlo[ct] = (ok && window > 0 && w.qpos[ct] - window + 1 > 0) ? w.qpos[ct] - window + 1 : 0;
+    q_rows[ct] = ok ? q + ((size_t)(q_begin + qi) * nq + head) * d : nullptr;
+  }
+  w.load_q(q_rows, d, j);
+  // range of keys this wave's queries see (wave-uniform)
+  const int n_q = min(QW, q_len - q0);
+  const int first_pos = pos0 + q0, last_pos = pos0 + q0 + n_q - 1;
+  const int lo_first = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
+  const int k_begin = lo_first & ~31;
+  for (int kb = k_begin; kb <= last_pos; kb += 32) {
+    // a step needs the mask unless every key is at or before every query and inside every window
+    const int lo_last = (window > 0 && last_pos - window + 1 > 0) ? last_pos - window + 1 : 0;
+    const bool masked = (kb + 31 > first_pos) || (kb < lo_last);
+    w.step(kv, kb, ctx - 1, scale_log2, masked, r, j);
+  }
+#pragma unroll
+  for (int ct = 0; ct < NQT; ++ct) {
+    const float lt = w.total_l(ct);
+    const int qi = q0 + 16 * ct + r;
+    if (qi >= q_len) continue;
+    const float inv = 1.f / lt;
+    bf16* o = out + ((size_t)(q_begin + qi) * nq + head) * d;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      if (16 * dt >= d) break;
+      bf16* op = o + 16 * dt + 4 * j;
+      const f32x4 a = w.acc[dt][ct];
+      op[0] = __float2bfloat16(a[0] * inv);
+      op[1] = __float2bfloat16(a[1] * inv);
+      op[2] = __float2bfloat16(a[2] * inv);
+      op[3] = __float2bfloat16(a[3] * inv);
+    }
+  }
+}
+
+// =====================================================================================
+// Decode: every sequence has one query token.  Workgroup (split, kv head, sequence): the
+// query heads of the kv group are the columns of one tile; the workgroup's four waves
+// take alternate 32-key steps of its chunk of `keys_per_wg` keys and merge through LDS.
+// Partial results (O * 2^-m normalised sums and m, l) go to a workspace, combined by the
+// second kernel in split order.
+// =====================================================================================
+template <int KC, int DT>
+__global__ __launch_bounds__(256) void attn_decode_split_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ vt_cache,
+    const int* __restrict__ block_tables, int max_pages, const int* __restrict__ ctx_lens,
+    float* __restrict__ part_o, float* __restrict__ part_ml, int max_splits, float scale_log2, int window,
+    int page, int nq, int nkv, int d, int keys_per_wg) {
+  extern __shared__ float lds[];  // [4 waves][g][d] + [4][g][2]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, j = lane >> 4;
+  const int split = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
+  const int g = nq / nkv;
+  const int ctx = ctx_lens[seq];
+  const int pos = ctx - 1;
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int k_begin = (lo & ~31) + split * keys_per_wg;
+  if (k_begin > pos) return;  // no keys for this split (the combine kernel knows)
+  const int k_end = min(pos + 1, k_begin + keys_per_wg);  // exclusive
+
+  PagedKV kv{k_cache, vt_cache, block_tables + (size_t)seq * max_pages, page, nkv, d, kvh};
+  WaveAttn<KC, DT, 1> w;
+  w.init();
+  const bool col = r < g;
+  w.qpos[0] = col ? pos : -1;
+  w.qlo[0] = lo;
+  const bf16* q_rows[1] = {col ? q + ((size_t)seq * nq + kvh * g + r) * d : nullptr};
+  w.load_q(q_rows, d, j);
+  for (int kb = k_begin + 32 * wave; kb < k_end; kb += 128) {
+    const bool masked = (kb + 31 > pos) || (kb < lo);
+    w.step(kv, kb, pos, scale_log2, masked, r, j);
+  }
+  const float lt = w.total_l(0);
+  float* lds_o = lds;                    // [4][g][d]
+  float* lds_ml = lds + 4 * g * d;       // [4][g][2]
+  if (col) {
+    if (j == 0) {
+      lds_ml[(wave * g + r) * 2] = w.m[0];
+      lds_ml[(wave * g + r) * 2 + 1] = lt;
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      if (16 * dt >= d) break;
+      float* o = lds_o + ((size_t)wave * g + r) * d + 16 * dt + 4 * j;
+      o[0] = w.acc[dt][0][0];
+      o[1] = w.acc[dt][0][1];
+      o[2] = w.acc[dt][0][2];
+      o[3] = w.acc[dt][0][3];
+    }
+  }
+  __syncthreads();
+  // merge the four waves, in wave order, and store the partial of (seq, head, split)
+  for (int idx = threadIdx.x; idx < g * d; idx += blockDim.x) {
+    const int h = idx / d, i = idx - h * d;
+    float mm = -INFINITY;
+#pragma unroll
+    for (int wv = 0; wv < 4; ++wv) mm = fmaxf(mm, lds_ml[(wv * g + h) * 2]);
+    float o = 0.f, ll = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < 4; ++wv) {
+      const float mw = lds_ml[(wv * g + h) * 2];
+      const float f = (mw == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mw - mm);
+      o += lds_o[((size_t)wv * g + h) * d + i] * f;
+      ll += lds_ml[(wv * g + h) * 2 + 1] * f;
+    }
+    const size_t pidx = ((size_t)seq * nq + kvh * g + h) * max_splits + split;
+    part_o[pidx * d + i] = o;
+    if (i == 0) {
+      part_ml[pidx * 2] = mm;
+      part_ml[pidx * 2 + 1] = ll;
+    }
+  }
+}
+
+__global__ void attn_decode_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                           const int* __restrict__ ctx_lens, bf16* __restrict__ out,
+                                           int max_splits, int window, int nq, int d, int keys_per_wg) {
+  const int head = blockIdx.x, seq = blockIdx.y;
+  const int pos = ctx_lens[seq] - 1;
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int n_splits = (pos - (lo & ~31)) / keys_per_wg + 1;
+  const size_t base = ((size_t)seq * nq + head) * max_splits;
+  float mm = -INFINITY;
+  for (int s = 0; s < n_splits; ++s) mm = fmaxf(mm, part_ml[(base + s) * 2]);
+  float ll = 0.f;
+  for (int s = 0; s < n_splits; ++s) ll += part_ml[(base + s) * 2 + 1] * __builtin_amdgcn_exp2f(part_ml[(base + s) * 2] - mm);
+  const float inv = 1.f / ll;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+    float o = 0.f;
+    for (int s = 0; s < n_splits; ++s) o += part_o[(base + s) * d + i] * __builtin_amdgcn_exp2f(part_ml[(base + s) * 2] - mm);
+    out[((size_t)seq * nq + head) * d + i] = __float2bfloat16(o * inv);
+  }
+}
+
+}  // namespace xi
+
+using namespace xi;
+
+extern "C" {
+
+// Sizes the MFMA kernels take: head_dim a multiple of 16 up to 256, page size a multiple of 8,
+// at most 16 query heads per kv head (decode).  Returns 1 if supported.
+int xi_attention_mfma_supported(int nq, int nkv, int d, int page) {
+  return (d % 16 == 0 && d >= 16 && d <= 256 && page % 8 == 0 && nq % nkv == 0) ? 1 : 0;
+}
+
+int xi_attention_prefill_bf16(const void* q, const void* k_cache, const void* vt_cache, const int* block_tables,
+                              int max_pages, const int* tiles, int n_tiles, const int* cu_q,
+                              const int* ctx_lens, void* out, float scale, int window, int page, int nq,
+                              int nkv, int d, hipStream_t stream) {
+  XI_CHECK(xi_attention_mfma_supported(nq, nkv, d, page), "attention_prefill: unsupported sizes nq=%d nkv=%d d=%d page=%d",
+           nq, nkv, d, page);
+  XI_CHECK(nq <= 65535, "attention_prefill: too many heads");
+  if (n_tiles == 0) return 0;
+  dim3 grid(n_tiles, nq);
+  const float sl = scale * kLog2e;
+#define XI_PF(KC, DT, NQT)                                                                           \
+  attn_prefill_kernel<KC, DT, NQT><<<grid, 256, 0, stream>>>(                                        \
+      (const bf16*)q, (const bf16*)k_cache, (const bf16*)vt_cache, block_tables, max_pages, tiles, cu_q, \
+      ctx_lens, (bf16*)out, sl, window, page, nq, nkv, d)
+  if (d <= 64) XI_PF(2, 4, 2);
+  else if (d <= 128) XI_PF(4, 8, 2);
+  else XI_PF(8, 16, 1);
+#undef XI_PF
+  XI_LAUNCH_CHECK("attention_prefill");
+  return 0;
+}
+
+// Queries per block of the prefill kernel for a head size (the host builds `tiles` with it).
+int xi_attention_prefill_block(int d) { return d <= 128 ? 128 : 64; }
+
+int xi_attention_decode_bf16(const void* q, const void* k_cache, const void* vt_cache, const int* block_tables,
+                             int max_pages, const int* ctx_lens, void* out, float* part_o, float* part_ml,
+                             int max_splits, int keys_per_wg, float scale, int window, int page, int n_seq,
+                             int nq, int nkv, int d, hipStream_t stream) {
+  XI_CHECK(xi_attention_mfma_supported(nq, nkv, d, page), "attention_decode: unsupported sizes nq=%d nkv=%d d=%d page=%d",
+           nq, nkv, d, page);
+  const int g = nq / nkv;
+  XI_CHECK(g <= 16, "attention_decode: %d query heads per kv head exceed 16", g);
+  XI_CHECK(keys_per_wg > 0 && keys_per_wg % 128 == 0, "attention_decode: keys_per_wg %d must be a multiple of 128", keys_per_wg);
+  XI_CHECK(max_splits > 0 && nkv <= 65535 && n_seq <= 65535, "attention_decode: bad grid");
+  const size_t lds = (size_t)(4 * g * d + 4 * g * 2) * sizeof(float);
+  XI_CHECK(lds <= 64 * 1024, "attention_decode: group %d x head_dim %d needs too much LDS", g, d);
+  if (n_seq == 0) return 0;
+  dim3 grid(max_splits, nkv, n_seq);
+  const float sl = scale * kLog2e;
+#define XI_DC(KC, DT)                                                                              \
+  attn_decode_split_kernel<KC, DT><<<grid, 256, lds, stream>>>(                                    \
+      (const bf16*)q, (const bf16*)k_cache, (const bf16*)vt_cache, block_tables, max_pages, ctx_lens, \
+      part_o, part_ml, max_splits, sl, window, page, nq, nkv, d, keys_per_wg)
+  if (d <= 64) XI_DC(2, 4);
+  else if (d <= 128) XI_DC(4, 8);
+  else XI_DC(8, 16);
+#undef XI_DC
+  XI_LAUNCH_CHECK("attention_decode_split");
+  attn_decode_combine_kernel<<<dim3(nq, n_seq), 64, 0, stream>>>(part_o, part_ml, ctx_lens, (bf16*)out,
+                                                                  max_splits, window, nq, d, keys_per_wg);
+  XI_LAUNCH_CHECK("attention_decode_combine");
+  return 0;
+}
+
+}  // extern "C"

@@ -108,7 +108,8 @@ __global__ void silu_mul_kernel<float>(const float* __restrict__ gu, float* __re
 //     half layout:        pairs (i, i + rot/2);   interleaved layout: pairs (2i, 2i+1)
 //     o_a = a*cos - b*sin;  o_b = a*sin + b*cos
 //   q goes to q_out [T, nq, d]; k and v go to cache[page, kv_head, offset, :] with
-//   slot = page*page_size + offset (reference slot formula runner.rs:1344-1362).
+//   slot = page*page_size + offset (reference slot formula runner.rs:1344-1362); with
+//   v_transposed the V pool is [page, kv_head, d, offset] (what the MFMA attention reads).
 //   A negative slot means: do not store (the token's cache belongs to another run).
 // ---------------------------------------------------------------------------------
 template <typename T>
@@ -119,7 +120,7 @@ __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, const float* _
                                        const int* __restrict__ positions,
                                        const long long* __restrict__ slots, T* __restrict__ q_out,
                                        T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                       int page_size, int n_tok, int nq, int nkv, int d) {
+                                       int page_size, int n_tok, int nq, int nkv, int d, int v_transposed) {
   const int heads = nq + 2 * nkv;
   const int lane = threadIdx.x & (kWave - 1);
   const long long wid = (long long)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
@@ -141,6 +142,11 @@ __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, const float* _
     const int off = (int)(slot - page * page_size);
     const bool is_k = h < nq + nkv;
     const int kvh = is_k ? h - nq : h - nq - nkv;
+    if (!is_k && v_transposed) {  // V kept as [page, kv_head, d, offset]
+      T* vt = v_cache + ((size_t)page * nkv + kvh) * d * page_size + off;
+      for (int i = lane; i < d; i += kWave) vt[(size_t)i * page_size] = src[i];
+      return;
+    }
     T* cache = is_k ? k_cache : v_cache;
     dst = cache + (((size_t)page * nkv + kvh) * page_size + off) * d;
     w = is_k ? kw : nullptr;
@@ -247,7 +253,7 @@ int xi_silu_mul(const void* gate_up, void* out, int dtype, int n_tok, int I, hip
 int xi_qk_norm_rope_kv(const void* qkv, int dtype, const float* qw, const float* kw, float eps,
                        const float* cos_t, const float* sin_t, int rot, int interleaved,
                        const int* positions, const long long* slots, void* q_out, void* k_cache,
-                       void* v_cache, int page_size, int n_tok, int nq, int nkv, int d,
+                       void* v_cache, int page_size, int n_tok, int nq, int nkv, int d, int v_transposed,
                        hipStream_t stream) {
   XI_CHECK(n_tok >= 0 && nq > 0 && nkv > 0 && d > 0 && page_size > 0,
            "qk_norm_rope_kv: bad sizes T=%d nq=%d nkv=%d d=%d page=%d", n_tok, nq, nkv, d, page_size);
@@ -261,7 +267,7 @@ int xi_qk_norm_rope_kv(const void* qkv, int dtype, const float* qw, const float*
 #define XI_QK(TT)                                                                               \
   qk_norm_rope_kv_kernel<TT><<<(unsigned)blocks, wpb * kWave, 0, stream>>>(                     \
       (const TT*)qkv, qw, kw, eps, cos_t, sin_t, rot, interleaved, positions, slots, (TT*)q_out, \
-      (TT*)k_cache, (TT*)v_cache, page_size, n_tok, nq, nkv, d)
+      (TT*)k_cache, (TT*)v_cache, page_size, n_tok, nq, nkv, d, v_transposed)
   if (dtype == kF32) XI_QK(float);
   else if (dtype == kBF16) XI_QK(bf16);
   else XI_CHECK(false, "qk_norm_rope_kv: unknown dtype %d", dtype);

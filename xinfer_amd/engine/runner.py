@@ -59,10 +59,11 @@ class ModelRunner:
         for layer, kv in model.kv_needs.items():
             g = model.group_of_layer[layer]
             shape = (groups[g].num_pages, kv.num_kv_heads, self.page_size, kv.head_dim)
+            v_shape = (shape[0], shape[1], shape[3], shape[2]) if kv.v_transposed else shape
             self.layer_caches[layer] = LayerCache(
                 group=g,
                 k=torch.zeros(shape, dtype=model.dtype, device=self.device),
-                v=torch.zeros(shape, dtype=model.dtype, device=self.device))
+                v=torch.zeros(v_shape, dtype=model.dtype, device=self.device))
         for layer, st in model.state_needs.items():
             arena = torch.zeros((self.max_requests, *st.shape), dtype=st.dtype, device=self.device)
             if layer in self.layer_caches:

@@ -139,9 +139,10 @@ def qk_norm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor],
                     sin: torch.Tensor, rotary_dim: int, interleaved: bool,
                     positions: torch.Tensor, slots: torch.Tensor, k_cache: torch.Tensor,
                     v_cache: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
-                    q_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    q_out: Optional[torch.Tensor] = None, v_transposed: bool = False) -> torch.Tensor:
     """Per-head RMSNorm of q and k (if weights are given), rotation by position, q to q_out
-    [T, nq, d], k and v into the paged cache [pages, nkv, page_size, d] at `slots`."""
+    [T, nq, d], k and v into the paged cache [pages, nkv, page_size, d] at `slots`; with
+    `v_transposed` the V pool is [pages, nkv, d, page_size]."""
     _dev(qkv, q_weight, k_weight, cos, sin, positions, slots, k_cache, v_cache, q_out)
     nq, nkv, d = num_heads, num_kv_heads, head_dim
     T = qkv.shape[0]
@@ -160,10 +161,7 @@ def qk_norm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor],
             _want(w, torch.float32, "qk_norm_rope_kv: norm weight")
             if w.shape != (d,):
                 raise KernelError("qk_norm_rope_kv: norm weight must be [head_dim]")
-    if (k_cache.dim() != 4 or k_cache.shape[1] != nkv or k_cache.shape[3] != d
-            or v_cache.shape != k_cache.shape or k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype):
-        raise KernelError(f"qk_norm_rope_kv: cache {tuple(k_cache.shape)} {k_cache.dtype} does not match "
-                          f"[pages, {nkv}, page_size, {d}] {qkv.dtype}")
+    _check_cache(k_cache, v_cache, nkv, d, qkv.dtype, v_transposed, "qk_norm_rope_kv")
     if q_out is None:
         q_out = torch.empty((T, nq, d), dtype=qkv.dtype, device=qkv.device)
     elif q_out.shape != (T, nq, d) or q_out.dtype != qkv.dtype:
@@ -171,13 +169,26 @@ def qk_norm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor],
     _ok(lib().xi_qk_norm_rope_kv(
         _p(qkv), _code(qkv, "qk_norm_rope_kv"), _p(q_weight), _p(k_weight), ctypes.c_float(eps),
         _p(cos), _p(sin), int(rotary_dim), int(bool(interleaved)), _p(positions), _p(slots),
-        _p(q_out), _p(k_cache), _p(v_cache), int(k_cache.shape[2]), T, nq, nkv, d, _stream()))
+        _p(q_out), _p(k_cache), _p(v_cache), int(k_cache.shape[2]), T, nq, nkv, d,
+        int(bool(v_transposed)), _stream()))
     return q_out
+
+
+def _check_cache(k_cache, v_cache, nkv, d, dtype, v_transposed, what):
+    """K pool [pages, nkv, page, d]; V pool the same, or [pages, nkv, d, page] if transposed."""
+    if k_cache.dim() != 4 or k_cache.shape[1] != nkv or k_cache.shape[3] != d or k_cache.dtype != dtype:
+        raise KernelError(f"{what}: K pool {tuple(k_cache.shape)} {k_cache.dtype} does not match "
+                          f"[pages, {nkv}, page_size, {d}] {dtype}")
+    pages, _, page, _ = k_cache.shape
+    want = (pages, nkv, d, page) if v_transposed else (pages, nkv, page, d)
+    if tuple(v_cache.shape) != want or v_cache.dtype != dtype:
+        raise KernelError(f"{what}: V pool {tuple(v_cache.shape)} {v_cache.dtype} does not match {want} {dtype}")
 
 
 def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       block_tables: torch.Tensor, tok_seq: torch.Tensor, positions: torch.Tensor,
-                      scale: float, window: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      scale: float, window: int = 0, out: Optional[torch.Tensor] = None,
+                      v_transposed: bool = False) -> torch.Tensor:
     """Causal paged GQA attention for any mix of tokens.  q [T, nq, d]; caches
     [pages, nkv, page_size, d]; block_tables int32 [B, max_pages]; tok_seq / positions
     int32 [T] name each token's row of block_tables and its absolute position.
@@ -186,10 +197,10 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     if q.dim() != 3:
         raise KernelError("attention: q must be [T, nq, d]")
     T, nq, d = q.shape
-    if (k_cache.dim() != 4 or k_cache.shape[3] != d or v_cache.shape != k_cache.shape
-            or k_cache.dtype != q.dtype or v_cache.dtype != q.dtype):
-        raise KernelError(f"attention: cache {tuple(k_cache.shape)} {k_cache.dtype} does not match q {tuple(q.shape)} {q.dtype}")
+    if k_cache.dim() != 4:
+        raise KernelError("attention: the K pool must be [pages, nkv, page_size, d]")
     nkv, page = k_cache.shape[1], k_cache.shape[2]
+    _check_cache(k_cache, v_cache, nkv, d, q.dtype, v_transposed, "attention")
     for t, name in ((block_tables, "block_tables"), (tok_seq, "tok_seq"), (positions, "positions")):
         _want(t, torch.int32, f"attention: {name}")
     if block_tables.dim() != 2 or tok_seq.shape != (T,) or positions.shape != (T,):
@@ -201,7 +212,7 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     _ok(lib().xi_attention_generic(
         _p(q), _p(k_cache), _p(v_cache), _code(q, "attention"), _p(block_tables),
         int(block_tables.shape[1]), _p(tok_seq), _p(positions), _p(out), ctypes.c_float(scale),
-        int(window), int(page), T, nq, nkv, d, _stream()))
+        int(window), int(page), T, nq, nkv, d, int(bool(v_transposed)), _stream()))
     return out
 
 
@@ -227,12 +238,88 @@ def gemm_tn(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] =
     return out
 
 
+DECODE_KEYS_PER_WORKGROUP = 256
+
+
+def mfma_attention_supported(nq: int, nkv: int, d: int, page: int) -> bool:
+    return bool(lib().xi_attention_mfma_supported(nq, nkv, d, page))
+
+
+def attention_prefill_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, scale, window=0, out=None):
+    """MFMA attention for any mix of portions.  tiles int32 [n, 2] = (sequence, first query
+    token of a block of `prefill_block(d)` tokens within the sequence's portion)."""
+    _dev(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, out)
+    T, nq, d = q.shape
+    nkv, page = k_cache.shape[1], k_cache.shape[2]
+    _want(q, torch.bfloat16, "attention_prefill: q")
+    _check_cache(k_cache, vt_cache, nkv, d, torch.bfloat16, True, "attention_prefill")
+    for t, name in ((block_tables, "block_tables"), (tiles, "tiles"), (cu_q, "cu_q"), (ctx_lens, "ctx_lens")):
+        _want(t, torch.int32, f"attention_prefill: {name}")
+    B = ctx_lens.shape[0]
+    if block_tables.shape[0] != B or cu_q.shape != (B + 1,) or tiles.dim() != 2 or tiles.shape[1] != 2:
+        raise KernelError("attention_prefill: block_tables [B, pages], cu_q [B+1], ctx_lens [B], tiles [n, 2] expected")
+    if out is None:
+        out = torch.empty((T, nq * d), dtype=q.dtype, device=q.device)
+    _ok(lib().xi_attention_prefill_bf16(
+        _p(q), _p(k_cache), _p(vt_cache), _p(block_tables), int(block_tables.shape[1]), _p(tiles),
+        int(tiles.shape[0]), _p(cu_q), _p(ctx_lens), _p(out), ctypes.c_float(scale), int(window), int(page),
+        nq, nkv, d, _stream()))
+    return out
+
+
+def prefill_block(d: int) -> int:
+    return int(lib().xi_attention_prefill_block(int(d)))
+
+
+def attention_decode_bf16(q, k_cache, vt_cache, block_tables, ctx_lens, max_ctx_len, scale, window=0, out=None):
+    """Split-K MFMA attention for a batch in which every sequence has one token (q [B, nq, d])."""
+    _dev(q, k_cache, vt_cache, block_tables, ctx_lens, out)
+    B, nq, d = q.shape
+    nkv, page = k_cache.shape[1], k_cache.shape[2]
+    _want(q, torch.bfloat16, "attention_decode: q")
+    _check_cache(k_cache, vt_cache, nkv, d, torch.bfloat16, True, "attention_decode")
+    _want(block_tables, torch.int32, "attention_decode: block_tables")
+    _want(ctx_lens, torch.int32, "attention_decode: ctx_lens")
+    if block_tables.shape[0] != B or ctx_lens.shape != (B,):
+        raise KernelError("attention_decode: one block table row and one context length per sequence")
+    span = min(int(max_ctx_len), int(window) + 31) if window > 0 else int(max_ctx_len)
+    kpw = DECODE_KEYS_PER_WORKGROUP
+    max_splits = span // kpw + 1
+    part_o = torch.empty((B, nq, max_splits, d), dtype=torch.float32, device=q.device)
+    part_ml = torch.empty((B, nq, max_splits, 2), dtype=torch.float32, device=q.device)
+    if out is None:
+        out = torch.empty((B, nq * d), dtype=q.dtype, device=q.device)
+    _ok(lib().xi_attention_decode_bf16(
+        _p(q), _p(k_cache), _p(vt_cache), _p(block_tables), int(block_tables.shape[1]), _p(ctx_lens), _p(out),
+        _p(part_o), _p(part_ml), max_splits, kpw, ctypes.c_float(scale), int(window), int(page), B, nq, nkv, d,
+        _stream()))
+    return out
+
+
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx, group: int,
-              scale: float, window: int = 0) -> torch.Tensor:
+              scale: float, window: int = 0, v_transposed: bool = False) -> torch.Tensor:
     """Attention of one step's tokens over the paged cache of `group`; chooses the kernel
-    from the precision and the shape of the batch."""
-    return attention_generic(q, k_cache, v_cache, ctx.block_tables[group], ctx.tok_seq,
-                             ctx.positions, scale, window)
+    from the precision and the shape of the batch: float32, or sizes the matrix-core
+    kernels do not take, go to the generic kernel; bfloat16 batches of single tokens to
+    the split-K decode kernel; everything else to the prefill kernel."""
+    T, nq, d = q.shape
+    nkv, page = k_cache.shape[1], k_cache.shape[2]
+    bt = ctx.block_tables[group]
+    if q.dtype == torch.bfloat16 and v_transposed and mfma_attention_supported(nq, nkv, d, page):
+        g = nq // nkv
+        if ctx.max_q_len == 1 and g <= 16 and (4 * g * d + 8 * g) * 4 <= 64 * 1024:
+            return attention_decode_bf16(q, k_cache, v_cache, bt, ctx.ctx_lens, ctx.max_ctx_len, scale, window)
+        qb = prefill_block(d)
+        key = ("attention_tiles", qb)
+        tiles = ctx.scratch.get(key)
+        if tiles is None:
+            rows = [(b, q0) for b in range(ctx.num_seqs)
+                    for q0 in range(0, ctx.cu_q_host[b + 1] - ctx.cu_q_host[b], qb)]
+            tiles = torch.tensor(rows, dtype=torch.int32, device=q.device).reshape(-1, 2)
+            ctx.scratch[key] = tiles
+        return attention_prefill_bf16(q, k_cache, v_cache, bt, tiles, ctx.cu_q, ctx.ctx_lens, scale, window)
+    return attention_generic(q, k_cache, v_cache, bt, ctx.tok_seq, ctx.positions, scale, window,
+                             v_transposed=v_transposed)
 
 
 def linear_bf16(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:

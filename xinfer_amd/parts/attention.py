@@ -73,19 +73,21 @@ class PagedAttention(Mixer):
 
     # ---- cache ---------------------------------------------------------------
     def cache_need(self) -> KVNeed:
-        return KVNeed(self.nkv, self.d, self.window)
+        # the matrix-core kernels of the bfloat16 path read V transposed
+        return KVNeed(self.nkv, self.d, self.window, v_transposed=self.dtype == torch.bfloat16)
 
     # ---- step ----------------------------------------------------------------
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
         qkv = self.qkv(x, out_dtype=self.dtype)
         pos = self.position
         slots = ctx.slots[cache.group] if cache.write else ctx.no_slots
+        vt = self.dtype == torch.bfloat16
         q = kernels.qk_norm_rope_kv(
             qkv, self.q_norm_w, self.k_norm_w, self.qk_norm_eps,
             pos.cos if pos is not None else ctx.empty_f32,
             pos.sin if pos is not None else ctx.empty_f32,
             pos.rotary_dim if pos is not None else 0,
             pos.interleaved if pos is not None else False,
-            ctx.positions, slots, cache.k, cache.v, self.nq, self.nkv, self.d)
-        a = kernels.attention(q, cache.k, cache.v, ctx, cache.group, self.scale, self.window)
+            ctx.positions, slots, cache.k, cache.v, self.nq, self.nkv, self.d, v_transposed=vt)
+        a = kernels.attention(q, cache.k, cache.v, ctx, cache.group, self.scale, self.window, v_transposed=vt)
         return self.o(a, out_dtype=self.dtype)

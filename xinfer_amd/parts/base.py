@@ -33,10 +33,13 @@ from ..weights.store import TensorDecl, WeightStore
 # ---- what a layer may ask of the cache ------------------------------------------------
 @dataclass(frozen=True)
 class KVNeed:
-    """Paged keys and values: `window` = 0 keeps every key, w > 0 the last w."""
+    """Paged keys and values: `window` = 0 keeps every key, w > 0 the last w.  The K pool
+    is [pages, kv_heads, page_size, head_dim]; the V pool the same, or with `v_transposed`
+    [pages, kv_heads, head_dim, page_size]."""
     num_kv_heads: int
     head_dim: int
     window: int = 0
+    v_transposed: bool = False
 
 
 @dataclass(frozen=True)
@@ -78,6 +81,7 @@ class StepContext:
     max_ctx_len: int = 0
     no_slots: Optional[torch.Tensor] = None    # int64 [T] of -1: "store nothing"
     empty_f32: Optional[torch.Tensor] = None   # float32 [1, 0]: tables of "no rotation"
+    scratch: Dict[Any, Any] = field(default_factory=dict)   # per-step data that kernels derive once
 
 
 @dataclass
