@@ -63,6 +63,8 @@ def main() -> int:
                     help="fewer layers than the configuration has (reported in config)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--skip-points", action="store_true", help="only the default decode run")
+    ap.add_argument("--only", choices=["all", "decode", "prefill"], default="all",
+                    help="run one phase only (for profiling); the JSON line then lacks the other")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -84,7 +86,7 @@ def main() -> int:
     print(f"[bench] model of {args.layers} layers built in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
 
     page = 64
-    max_batch = 8 if args.skip_points else 64
+    max_batch = 8 if (args.skip_points or args.only != "all") else 64
     max_batch = max(max_batch, args.batch)
     num_pages = max_batch * (CONTEXT // page) + PREFILL_TOKENS // page + 8
     runner = ModelRunner(model, page_size=page, num_pages=num_pages, max_requests=max_batch + 1)
@@ -141,6 +143,10 @@ def main() -> int:
             best = dt if best is None else min(best, dt)
         return best
 
+    if args.only == "prefill":
+        psec = prefill_run()
+        print(json.dumps({"prefill_ms": round(psec * 1e3, 3), "layers": args.layers}), flush=True)
+        return 0
     sec = decode_run(args.batch, args.steps, args.warmup)
     wb, kvb = weight_bytes(cfg), kv_bytes_per_token(cfg)
     # mean cache length over the timed steps (it grows by one each step, ending at CONTEXT)
@@ -165,6 +171,9 @@ def main() -> int:
                      "frac": round(achieved / HBM_GBPS, 4)},
     }
     print(f"[bench] decode b{args.batch}: {sec * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
+    if args.only == "decode":
+        print(json.dumps(out), flush=True)
+        return 0
     psec = prefill_run()
     flops = prefill_flops(cfg, PREFILL_TOKENS)
     out["prefill"] = {"value": round(PREFILL_TOKENS / psec, 1), "tokens": PREFILL_TOKENS,
