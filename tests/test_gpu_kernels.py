@@ -112,6 +112,63 @@ def test_linear_bf16(M, N, K):
     assert err < 2.0 ** -8, err
 
 
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("M", [1, 5, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(509, 96), (77, 136), (1536, 4096), (4096, 1408), (16, 8)])
+def test_linear_skinny(M, N, K, out_dtype):
+    """The streaming matrix-core product for few rows: widths that are no multiple of the 16-row
+    tile or the 32-wide k step, every tile shape it can choose, and a row alone bit-equal to the
+    same row inside a batch."""
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(7)
+    x = _rand((M, K), torch.bfloat16, g)
+    w = _rand((N, K), torch.bfloat16, g, 0.05)
+    ref = x.double() @ w.double().T
+    tol = 2.0 ** -8 if out_dtype == torch.bfloat16 else 1e-5
+    outs = []
+    for variant in (0, 1, 2, 3, 4):
+        y = kernels.linear_skinny(x.to(DEV), w.to(DEV), out_dtype, variant=variant)
+        assert y.dtype == out_dtype and y.shape == (M, N)
+        err = (y.cpu().double() - ref).abs().max() / ref.abs().max()
+        assert err < tol, (variant, err)
+        outs.append(y.cpu())
+    # with the same split of K over waves (variant 4: eight waves) a row alone is bit-equal to
+    # the same row inside the batch; the default choice may split K differently for few rows,
+    # which changes the order of the float32 sums and nothing else
+    r = M // 2
+    y1 = kernels.linear_skinny(x[r:r + 1].contiguous().to(DEV), w.to(DEV), out_dtype, variant=4)
+    assert torch.equal(y1.cpu()[0], outs[4][r])
+    y0 = kernels.linear_skinny(x[r:r + 1].contiguous().to(DEV), w.to(DEV), out_dtype)
+    assert float((y0.cpu()[0].double() - ref[r]).abs().max() / ref.abs().max()) < tol
+
+
+@pytest.mark.parametrize("M", [1, 8, 20, 64])
+@pytest.mark.parametrize("I,K", [(224, 96), (176, 80), (1001, 136), (12288, 4096)])
+def test_linear_skinny_gated(M, I, K):
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(8)
+    x = _rand((M, K), torch.bfloat16, g)
+    w = _rand((2 * I, K), torch.bfloat16, g, 0.1)
+    gu = x.double() @ w.double().T
+    ref = plain.swiglu(gu[:, :I], gu[:, I:])
+    y = kernels.linear_skinny(x.to(DEV), w.to(DEV), gated=True)
+    assert y.shape == (M, I)
+    err = (y.cpu().double() - ref).abs().max() / ref.abs().max()
+    assert err < 2.0 ** -8, err
+
+
+def test_linear_skinny_refuses():
+    from xinfer_amd import kernels
+    x = torch.zeros((65, 64), dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros((32, 64), dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(kernels.KernelError, match="<= 64"):
+        kernels.linear_skinny(x, w)
+    with pytest.raises(kernels.KernelError, match="multiple of 8"):
+        kernels.linear_skinny(x[:4, :60].contiguous(), w[:, :60].contiguous())
+    with pytest.raises(kernels.KernelError, match="bfloat16"):
+        kernels.linear_skinny(x[:4].float(), w.float())
+
+
 def _rope_ref(x, pos, cos, sin, rot, interleaved):
     x = x.double().clone()
     c, s = cos[pos].double()[:, None, :], sin[pos].double()[:, None, :]

@@ -317,22 +317,43 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(
   }
 }
 
-__global__ void attn_decode_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                           const int* __restrict__ ctx_lens, bf16* __restrict__ out,
-                                           int max_splits, int window, int nq, int d, int keys_per_wg) {
-  const int head = blockIdx.x, seq = blockIdx.y;
+// One wave per (head, sequence).  Lanes first share out the splits to find the common
+// maximum and each split's weight, then every lane sums its output dims over the splits in
+// split order.
+__global__ __launch_bounds__(64) void attn_decode_combine_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ ctx_lens,
+    bf16* __restrict__ out, int max_splits, int window, int nq, int d, int keys_per_wg) {
+  extern __shared__ float f_s[];  // [max_splits] weight of each split
+  const int head = blockIdx.x, seq = blockIdx.y, lane = threadIdx.x;
   const int pos = ctx_lens[seq] - 1;
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int n_splits = (pos - (lo & ~31)) / keys_per_wg + 1;
   const size_t base = ((size_t)seq * nq + head) * max_splits;
   float mm = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) mm = fmaxf(mm, part_ml[(base + s) * 2]);
+  for (int s = lane; s < n_splits; s += kWave) mm = fmaxf(mm, part_ml[(base + s) * 2]);
+  mm = wave_max(mm);
   float ll = 0.f;
-  for (int s = 0; s < n_splits; ++s) ll += part_ml[(base + s) * 2 + 1] * __builtin_amdgcn_exp2f(part_ml[(base + s) * 2] - mm);
+  for (int s = lane; s < n_splits; s += kWave) {
+    const float f = __builtin_amdgcn_exp2f(part_ml[(base + s) * 2] - mm);
+    f_s[s] = f;
+    ll += part_ml[(base + s) * 2 + 1] * f;
+  }
+  ll = wave_sum(ll);
+  __syncthreads();
   const float inv = 1.f / ll;
-  for (int i = threadIdx.x; i < d; i += blockDim.x) {
+  for (int i = lane; i < d; i += kWave) {
+    const float* po = part_o + base * d + i;
     float o = 0.f;
-    for (int s = 0; s < n_splits; ++s) o += part_o[(base + s) * d + i] * __builtin_amdgcn_exp2f(part_ml[(base + s) * 2] - mm);
+    int s = 0;
+    for (; s + 4 <= n_splits; s += 4) {
+      const float a0 = po[(size_t)s * d], a1 = po[(size_t)(s + 1) * d], a2 = po[(size_t)(s + 2) * d],
+                  a3 = po[(size_t)(s + 3) * d];
+      o += a0 * f_s[s];
+      o += a1 * f_s[s + 1];
+      o += a2 * f_s[s + 2];
+      o += a3 * f_s[s + 3];
+    }
+    for (; s < n_splits; ++s) o += po[(size_t)s * d] * f_s[s];
     out[((size_t)seq * nq + head) * d + i] = __float2bfloat16(o * inv);
   }
 }
@@ -384,6 +405,7 @@ int xi_attention_decode_bf16(const void* q, const void* k_cache, const void* vt_
   XI_CHECK(g <= 16, "attention_decode: %d query heads per kv head exceed 16", g);
   XI_CHECK(keys_per_wg > 0 && keys_per_wg % 128 == 0, "attention_decode: keys_per_wg %d must be a multiple of 128", keys_per_wg);
   XI_CHECK(max_splits > 0 && nkv <= 65535 && n_seq <= 65535, "attention_decode: bad grid");
+  XI_CHECK((size_t)max_splits * sizeof(float) <= 48 * 1024, "attention_decode: %d splits are too many", max_splits);
   const size_t lds = (size_t)(4 * g * d + 4 * g * 2) * sizeof(float);
   XI_CHECK(lds <= 64 * 1024, "attention_decode: group %d x head_dim %d needs too much LDS", g, d);
   if (n_seq == 0) return 0;
@@ -398,7 +420,7 @@ int xi_attention_decode_bf16(const void* q, const void* k_cache, const void* vt_
   else XI_DC(8, 16);
 #undef XI_DC
   XI_LAUNCH_CHECK("attention_decode_split");
-  attn_decode_combine_kernel<<<dim3(nq, n_seq), 64, 0, stream>>>(part_o, part_ml, ctx_lens, (bf16*)out,
+  attn_decode_combine_kernel<<<dim3(nq, n_seq), 64, max_splits * sizeof(float), stream>>>(part_o, part_ml, ctx_lens, (bf16*)out,
                                                                   max_splits, window, nq, d, keys_per_wg);
   XI_LAUNCH_CHECK("attention_decode_combine");
   return 0;

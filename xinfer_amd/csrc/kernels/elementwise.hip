@@ -66,6 +66,72 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TY* __restri
   }
 }
 
+// The same, for widths that are a multiple of 4 up to 4 * NT * MAXV: every thread keeps its
+// part of the row in registers, so the row is read once and all loads are in flight
+// together (one row of a decode step is otherwise a chain of dependent memory round trips).
+struct alignas(8) bf16x4_t { bf16 v[4]; };
+__device__ __forceinline__ float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 load4(const bf16* p) {
+  const bf16x4_t t = *reinterpret_cast<const bf16x4_t*>(p);
+  return float4{to_float(t.v[0]), to_float(t.v[1]), to_float(t.v[2]), to_float(t.v[3])};
+}
+__device__ __forceinline__ void store4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void store4(bf16* p, float4 v) {
+  bf16x4_t t;
+  t.v[0] = from_float<bf16>(v.x);
+  t.v[1] = from_float<bf16>(v.y);
+  t.v[2] = from_float<bf16>(v.z);
+  t.v[3] = from_float<bf16>(v.w);
+  *reinterpret_cast<bf16x4_t*>(p) = t;
+}
+
+template <typename TY, typename TO, int NT, int MAXV>
+__global__ __launch_bounds__(NT) void add_rmsnorm_vec_kernel(float* __restrict__ resid, const TY* __restrict__ y,
+                                                             const float* __restrict__ w, float eps,
+                                                             TO* __restrict__ out, const int* __restrict__ rows,
+                                                             int H) {
+  __shared__ float scratch[NT / kWave];
+  const int r = blockIdx.x;
+  const int row = rows ? rows[r] : r;
+  float* x = resid + (size_t)row * H;
+  const TY* yr = y ? y + (size_t)row * H : nullptr;
+  TO* o = out + (size_t)r * H;
+  const int nvec = H / 4;
+  float4 s[MAXV], wv[MAXV];
+#pragma unroll
+  for (int v = 0; v < MAXV; ++v) {
+    const int i = v * NT + threadIdx.x;
+    if (i < nvec) {
+      s[v] = load4(x + 4 * i);
+      wv[v] = load4(w + 4 * i);
+      if (yr) {
+        const float4 yy = load4(yr + 4 * i);
+        s[v].x += yy.x;
+        s[v].y += yy.y;
+        s[v].z += yy.z;
+        s[v].w += yy.w;
+      }
+    } else {
+      s[v] = float4{0.f, 0.f, 0.f, 0.f};
+      wv[v] = s[v];
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int v = 0; v < MAXV; ++v) ss += (s[v].x * s[v].x + s[v].y * s[v].y) + (s[v].z * s[v].z + s[v].w * s[v].w);
+  const float total = block_sum<NT / kWave>(ss, scratch);
+  const float inv = rsqrtf(total / (float)H + eps);
+#pragma unroll
+  for (int v = 0; v < MAXV; ++v) {
+    const int i = v * NT + threadIdx.x;
+    if (i < nvec) {
+      if (yr && !rows) store4(x + 4 * i, s[v]);
+      store4(o + 4 * i, float4{s[v].x * inv * wv[v].x, s[v].y * inv * wv[v].y, s[v].z * inv * wv[v].z,
+                               s[v].w * inv * wv[v].w});
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------------
 // SiLU(gate) * up on a packed [T, 2I] buffer (reference: attention_rs::silu_and_mul at
 // /root/reference/src/models/layers/mlp.rs:627-628; golden formula
@@ -96,6 +162,27 @@ __global__ void silu_mul_kernel<float>(const float* __restrict__ gu, float* __re
     const float u = gu[t * 2 * I + I + i];
     const float s = g / (1.f + expf(-g));  // full-precision exp on the 32-bit path
     out[idx] = s * u;
+  }
+}
+
+// bfloat16 with I a multiple of 8: 16-byte loads and stores.
+struct alignas(16) bf16x8_t { bf16 v[8]; };
+__global__ void silu_mul_vec8_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out, int I, size_t total8) {
+  const int per_row = I / 8;
+  size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; idx < total8; idx += stride) {
+    const size_t t = idx / per_row;
+    const int c = (int)(idx - t * per_row);
+    const bf16x8_t g = *reinterpret_cast<const bf16x8_t*>(gu + t * 2 * I + 8 * c);
+    const bf16x8_t u = *reinterpret_cast<const bf16x8_t*>(gu + t * 2 * I + I + 8 * c);
+    bf16x8_t o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float gf = to_float(g.v[e]);
+      o.v[e] = from_float<bf16>(gf / (1.f + __expf(-gf)) * to_float(u.v[e]));
+    }
+    *reinterpret_cast<bf16x8_t*>(out + t * I + 8 * c) = o;
   }
 }
 
@@ -219,10 +306,17 @@ int xi_add_rmsnorm(float* resid, const void* y, int y_dtype, const float* w, flo
                    int out_dtype, const int* rows, int n_rows, int H, hipStream_t stream) {
   XI_CHECK(n_rows >= 0 && H > 0, "add_rmsnorm: bad sizes rows=%d H=%d", n_rows, H);
   if (n_rows == 0) return 0;
-  constexpr int NT = 256;
-#define XI_NORM(TY, TO)                                                                   \
-  add_rmsnorm_kernel<TY, TO, NT><<<n_rows, NT, 0, stream>>>(resid, (const TY*)y, w, eps, \
-                                                              (TO*)out, rows, H)
+  constexpr int NT = 256, MAXV = 8;
+  const bool vec = H % 4 == 0 && H <= 4 * NT * MAXV && ((uintptr_t)resid | (uintptr_t)y | (uintptr_t)w | (uintptr_t)out) % 16 == 0;
+#define XI_NORM(TY, TO)                                                                            \
+  do {                                                                                             \
+    if (vec)                                                                                       \
+      add_rmsnorm_vec_kernel<TY, TO, NT, MAXV><<<n_rows, NT, 0, stream>>>(resid, (const TY*)y, w, eps, \
+                                                                          (TO*)out, rows, H);      \
+    else                                                                                           \
+      add_rmsnorm_kernel<TY, TO, NT><<<n_rows, NT, 0, stream>>>(resid, (const TY*)y, w, eps,       \
+                                                                (TO*)out, rows, H);                \
+  } while (0)
   if (y_dtype == kF32 && out_dtype == kF32) XI_NORM(float, float);
   else if (y_dtype == kBF16 && out_dtype == kBF16) XI_NORM(bf16, bf16);
   else if (y_dtype == kF32 && out_dtype == kBF16) XI_NORM(float, bf16);
@@ -242,7 +336,12 @@ int xi_silu_mul(const void* gate_up, void* out, int dtype, int n_tok, int I, hip
   if (blocks > 65535u * 16u) blocks = 65535u * 16u;
   if (dtype == kF32)
     silu_mul_kernel<float><<<(unsigned)blocks, nt, 0, stream>>>((const float*)gate_up, (float*)out, I, total);
-  else if (dtype == kBF16)
+  else if (dtype == kBF16 && I % 8 == 0 && ((uintptr_t)gate_up | (uintptr_t)out) % 16 == 0) {
+    const size_t total8 = total / 8;
+    size_t b8 = (total8 + nt - 1) / nt;
+    if (b8 > 65535u * 16u) b8 = 65535u * 16u;
+    silu_mul_vec8_kernel<<<(unsigned)b8, nt, 0, stream>>>((const bf16*)gate_up, (bf16*)out, I, total8);
+  } else if (dtype == kBF16)
     silu_mul_kernel<bf16><<<(unsigned)blocks, nt, 0, stream>>>((const bf16*)gate_up, (bf16*)out, I, total);
   else
     XI_CHECK(false, "silu_mul: unknown dtype %d", dtype);

@@ -322,11 +322,47 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx
                              v_transposed=v_transposed)
 
 
-def linear_bf16(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-    """bfloat16 x @ w.T with float32 accumulation.  Many rows: the vendor library
-    (hipBLASLt through torch), which the reference's engine also uses for its matrix
-    products."""
+SKINNY_MAX_ROWS = 64      # most rows the streaming kernel takes
+SKINNY_ROWS = 8           # up to this many rows it is faster than the vendor library (measured)
+SKINNY_GATED_ROWS = 16    # the same for the fused gate/up/silu form, which also saves a kernel
+
+
+def linear_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+                  gated: bool = False, out: Optional[torch.Tensor] = None, variant: int = 0) -> torch.Tensor:
+    """bfloat16 x [M, K] @ w [N, K]^T for M <= 64 rows with the streaming matrix-core kernel.
+    `gated`: w is [2N, K] = [gate; up] and the result is silu(x @ gate^T) * (x @ up^T), [M, N]."""
+    _dev(x, w, out)
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError("linear_skinny: operands must be bfloat16")
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
+        raise KernelError(f"linear_skinny: x {tuple(x.shape)} and w {tuple(w.shape)} do not match")
+    M, K = x.shape
+    N = w.shape[0]
+    if gated:
+        if N % 2:
+            raise KernelError("linear_skinny: a gated weight must be [2N, K]")
+        N //= 2
+    if M > SKINNY_MAX_ROWS or K % 8:
+        raise KernelError(f"linear_skinny: M={M} must be <= {SKINNY_MAX_ROWS} and K={K} a multiple of 8")
+    out_dtype = out_dtype or torch.bfloat16
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype, device=x.device)
+    elif out.shape != (M, N) or out.dtype != out_dtype:
+        raise KernelError("linear_skinny: out has the wrong shape or dtype")
+    _ok(lib().xi_linear_skinny(_p(x), _p(w), _p(out), M, N, K, _code(out, "linear_skinny"), int(bool(gated)),
+                               int(variant), _stream()))
+    return out
+
+
+def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """bfloat16 x @ w.T with float32 accumulation.  Few rows (decode): the hand-written
+    streaming kernel.  Many rows: the vendor library (hipBLASLt through torch), which the
+    reference's engine also uses for its matrix products."""
     _dev(x, w)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError("linear_bf16: operands must be bfloat16")
-    return torch.nn.functional.linear(x, w)
+    out_dtype = out_dtype or torch.bfloat16
+    if 0 < x.shape[0] <= SKINNY_ROWS and x.shape[1] % 8 == 0:
+        return linear_skinny(x, w, out_dtype)
+    y = torch.nn.functional.linear(x, w)
+    return y if y.dtype == out_dtype else y.to(out_dtype)

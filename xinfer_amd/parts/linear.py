@@ -34,5 +34,4 @@ class Linear:
             return y if out_dtype == torch.float32 else y.to(out_dtype)
         if x.dtype != w.dtype:
             raise kernels.KernelError(f"linear: activations are {x.dtype} but the weight is {w.dtype}")
-        y = kernels.linear_bf16(x, w)
-        return y if out_dtype == y.dtype else y.to(out_dtype)
+        return kernels.linear_bf16(x, w, out_dtype)

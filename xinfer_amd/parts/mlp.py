@@ -45,6 +45,10 @@ class GatedMLP(FeedForward):
         self.down = Linear(lin(f"{prefix}.down_proj.weight"))
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
-        gu = self.gate_up(x, out_dtype=self.dtype)
-        m = kernels.silu_mul(gu)
+        w = self.gate_up.weight
+        if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+                and 0 < x.shape[0] <= kernels.SKINNY_GATED_ROWS and x.shape[1] % 8 == 0):
+            m = kernels.linear_skinny(x, w, gated=True)        # gate, up and silu*mul in one pass
+        else:
+            m = kernels.silu_mul(self.gate_up(x, out_dtype=self.dtype))
         return self.down(m, out_dtype=self.dtype)
