@@ -247,6 +247,60 @@ def test_step_refuses_bad_input(model_dirs):
     runner.cache.check()
 
 
+# ---- decode steps recorded as HIP graphs ---------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,n_req", [("B", 3), ("W", 12)])
+def test_decode_graph_replays_equal_launch_by_launch(name, n_req, dtype, model_dirs):
+    """Decode steps replayed from a recorded graph give, bit for bit, the logits of the same
+    steps launched kernel by kernel: over many replays, with prompt portions of other requests
+    run between them (the program's own launch-by-launch work), with requests that end and
+    join (so the batch size, and with it the graph, changes), and with pages used again.
+    Twelve requests make the matrix products go through the vendor library inside the graph."""
+    from xinfer_amd.engine import ModelRunner, StepEntry, load_model
+    t = TINY[name]
+    vocab, page = t["config"]["vocab_size"], t["page_size"]
+    model = load_model(model_dirs[name], dtype, DEV)
+    rng = random.Random(77)
+    prompts = {i: harness.random_prompt(rng, rng.randrange(3, 60), vocab) for i in range(n_req + 2)}
+    feed = {i: harness.random_prompt(rng, 40, vocab) for i in prompts}
+
+    def run(use_graphs):
+        runner = ModelRunner(model, page, 16 * (n_req + 2), n_req + 2, use_graphs=use_graphs)
+        out = []
+        live = list(range(n_req))
+        for i in live:
+            runner.add_request(i)
+            runner.step([StepEntry(i, prompts[i], [])])
+        for step in range(36):
+            if step == 9:                            # one ends; its pages go back
+                runner.release(live.pop(1))
+            if step == 14:                           # another joins: a prompt portion between replays
+                j = n_req
+                runner.add_request(j)
+                out.append(runner.step([StepEntry(j, prompts[j][:2], [1])]).cpu())
+                out.append(runner.step([StepEntry(j, prompts[j][2:], [0])]).cpu())
+                live.append(j)
+            entries = [StepEntry(i, [feed[i][step]], [0] if (i + step) % 5 else []) for i in live]
+            out.append(runner.step(entries).cpu())
+        runner.cache.check()
+        return out, runner.graph_replays
+
+    want, n0 = run(False)
+    got, n1 = run(True)
+    assert n0 == 0 and n1 == 36
+    assert len(want) == len(got)
+    for k, (a, b) in enumerate(zip(want, got)):
+        assert a.shape == b.shape and torch.equal(a, b), f"step {k} differs between graph and launches"
+
+
+def test_model_with_a_part_that_reads_the_host_is_not_recorded(model_dirs):
+    from xinfer_amd.engine import ModelRunner, load_model
+    model = load_model(model_dirs["A"], "bfloat16", DEV)
+    assert model.graph_safe and ModelRunner(model, 16, 4, 2).use_graphs
+    model.blocks[0].mixer.graph_safe = False
+    assert not model.graph_safe and not ModelRunner(model, 16, 4, 2).use_graphs
+
+
 # ---- the replay program ---------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_program(dtype, model_dirs, tmp_path):
@@ -311,7 +365,7 @@ def test_parts_alone(dtype, model_dirs):
     runner = ModelRunner(model, 16, 4, 1)
     runner.add_request(0)
     runner.cache.reserve(0, T)
-    ctx = runner._context(runner.cache.build_batch([0], [T]))
+    ctx = runner._context(runner.cache.build_batch([0], [T]), np.zeros(T, np.int32), np.zeros(0, np.int32))[0]
     out = blk.mixer.forward(xin.to(DEV), ctx, runner.layer_caches[0]).cpu().float()
     cos, sin = plain.rope_tables(float(c["rope_theta"]), c["head_dim"], c["max_position_embeddings"])
     ref = plain.attention_block(xin.float(), W, "model.layers.0.self_attn", c, torch.arange(T), cos, sin, 24)

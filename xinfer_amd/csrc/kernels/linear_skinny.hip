@@ -162,11 +162,17 @@ int xi_linear_skinny(const void* x, const void* w, void* y, int M, int N, int K,
   const int mt = (M + 15) / 16;
   const int tiles = (N + 15) / 16;  // 16-row tiles of the output
   // Wide outputs keep two row tiles per workgroup (x operands are reused); narrow ones one
-  // tile and sixteen waves so that every compute unit still has work.
+  // tile and sixteen waves so that every compute unit still has work.  The number of waves
+  // fixes the order of the float32 sums, so it is chosen from N alone and a row's result
+  // does not depend on how many rows came with it (the gated form with more than 32 rows
+  // is the exception: sixteen waves of two tiles do not fit in LDS there).
   int rt = (variant == 1) ? 1 : (variant == 2) ? 2 : (tiles >= 2048 ? 2 : 1);
-  int nw = (variant == 3) ? 16 : (variant == 4) ? 8 : ((gated ? tiles : tiles / rt) < 512 && mt <= 2 ? 16 : 8);
   if (gated) rt = 2;
-  if (nw == 16 && rt * mt > 4) nw = 8;
+  int nw = (variant == 3) ? 16 : (variant == 4) ? 8 : ((gated ? tiles : tiles / rt) < 512 ? 16 : 8);
+  if (nw == 16 && rt * mt > 4) {
+    if (rt == 2 && !gated && variant != 2) rt = 1;
+    else nw = 8;
+  }
 #define XI_SK(MT, RT, NW, U, G, TO) launch_skinny<MT, RT, NW, U, G, TO>(x, w, y, M, N, K, stream)
 #define XI_SK_TO(MT, RT, NW, U, G)                         \
   do {                                                     \

@@ -65,7 +65,8 @@ class LLMEngine:
         self.seed = econfig.seed if econfig.seed is not None else int.from_bytes(os.urandom(4), "little")
         page = econfig.page_size
         num_pages = econfig.num_pages or self._plan_pages(page)
-        self.runner = ModelRunner(self.model, page, num_pages, econfig.max_num_seqs)
+        self.runner = ModelRunner(self.model, page, num_pages, econfig.max_num_seqs,
+                                  use_graphs=not econfig.disable_cuda_graph)
         budget = econfig.max_num_batched_tokens or max(econfig.prefill_chunk_size, econfig.max_num_seqs)
         self.scheduler = Scheduler(self.runner.cache, econfig.max_num_seqs, budget,
                                    econfig.prefill_chunk_size)

@@ -43,6 +43,11 @@ class CausalLM:
                 raise ValueError(f"schedule entry reads the cache of unknown layer {e.cache_of}")
         self._plan_cache()
 
+    @property
+    def graph_safe(self) -> bool:
+        """Every part can be recorded into a HIP graph (see `Part.graph_safe`)."""
+        return all(p.graph_safe for p in (self.embedding, self.final_norm, self.head, *self.blocks))
+
     # ---- weights -------------------------------------------------------------
     @classmethod
     def declare(cls, spec: ModelSpec) -> List[TensorDecl]:

@@ -16,7 +16,7 @@ sequence; this one mixes them and leaves sampling to the caller.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, List, Optional, Sequence, Tuple
+from typing import Any, Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -37,9 +37,60 @@ class StepError(ValueError):
     pass
 
 
+class _Staging:
+    """Pinned host buffers through which a step's index arrays reach the device: one copy
+    for the 32-bit arrays and one for the 64-bit ones."""
+
+    def __init__(self, device):
+        self.device = device
+        self._pin = {torch.int32: None, torch.int64: None}
+        self._done: Optional[torch.cuda.Event] = None
+
+    def upload(self, parts: Sequence[np.ndarray], dtype: torch.dtype,
+               dst: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, List[int]]:
+        """Concatenates `parts` into one device tensor (into `dst` if given) and returns it
+        with the offset of every part."""
+        offsets, n = [], 0
+        for p in parts:
+            offsets.append(n)
+            n += int(p.size)
+        pin = self._pin[dtype]
+        if pin is None or pin.numel() < n:
+            pin = torch.empty((max(1024, 1 << (n - 1).bit_length()),), dtype=dtype, pin_memory=True)
+            self._pin[dtype] = pin
+        if self._done is not None:
+            self._done.synchronize()        # the previous step's copy has left the buffer
+        host = pin.numpy()
+        for off, p in zip(offsets, parts):
+            host[off:off + p.size] = p.reshape(-1)
+        if dst is None:
+            dst = torch.empty((n,), dtype=dtype, device=self.device)
+        elif dst.numel() != n or dst.dtype != dtype:
+            raise ValueError("staging: the fixed device buffer does not fit this step's arrays")
+        dst.copy_(pin[:n], non_blocking=True)
+        return dst, offsets
+
+    def mark(self) -> None:
+        self._done = torch.cuda.Event()
+        self._done.record()
+
+
+@dataclass
+class _DecodeGraph:
+    graph: Any
+    dev32: torch.Tensor
+    dev64: torch.Tensor
+    logits: torch.Tensor            # [B, vocab], rewritten by every replay
+    want: torch.Tensor              # int32 [B]: this step's wanted rows (first R valid)
+    keep: Tuple[Any, ...] = ()      # everything else the recorded kernels read: it must stay
+                                    # allocated for as long as the graph may be replayed
+
+
 class ModelRunner:
-    def __init__(self, model: CausalLM, page_size: int, num_pages, max_requests: int):
-        """`num_pages`: pages of every group's pool, or a list with one count per group."""
+    def __init__(self, model: CausalLM, page_size: int, num_pages, max_requests: int,
+                 use_graphs: bool = True, graph_max_batch: int = 64):
+        """`num_pages`: pages of every group's pool, or a list with one count per group.
+        `use_graphs`: record decode steps of up to `graph_max_batch` requests as HIP graphs."""
         if not torch.cuda.is_available():
             raise RuntimeError("xinfer_amd runs on an AMD GPU only: no HIP device is visible")
         self.model = model
@@ -71,6 +122,14 @@ class ModelRunner:
             else:
                 self.layer_caches[layer] = LayerCache(state=arena)
         self._empty_f32 = torch.empty((1, 0), dtype=torch.float32, device=self.device)
+        self._staging = _Staging(self.device)
+        self.use_graphs = bool(use_graphs) and model.graph_safe
+        self.graph_max_batch = int(graph_max_batch)
+        self._graphs: Dict[Tuple[int, int], _DecodeGraph] = {}
+        self._graph_pool = None
+        # widest block table a request can have: the fixed width of a recorded step's tables
+        self._max_table = max(1, -(-model.spec.max_positions // self.page_size))
+        self.graph_replays = 0
 
     # ---- requests ---------------------------------------------------------------
     def add_request(self, rid: int) -> int:
@@ -123,28 +182,88 @@ class ModelRunner:
         if not reserved:
             for rid, n in zip(rids, counts):
                 self.cache.reserve(rid, n)      # OutOfPages leaves every request's length as it was
-        arrays = self.cache.build_batch(rids, counts)
-        ctx = self._context(arrays)
-        ids = torch.from_numpy(ids_host.astype(np.int32)).to(self.device)
-        want_rows = torch.tensor(rows, dtype=torch.int32, device=self.device)
-        logits = self.model.forward(ids, ctx, self.layer_caches, want_rows)
+        decode = self.use_graphs and max(counts) == 1 and len(rids) <= self.graph_max_batch
+        arrays = self.cache.build_batch(rids, counts, max_pages=self._max_table if decode else None)
+        ids32 = ids_host.astype(np.int32)
+        rows32 = np.asarray(rows, dtype=np.int32)
+        if decode:
+            logits = self._replay_decode(arrays, ids32, rows32)
+        else:
+            ctx, ids, want_rows, _, _ = self._context(arrays, ids32, rows32)
+            logits = self.model.forward(ids, ctx, self.layer_caches, want_rows)
         if not reserved:
             for rid, n in zip(rids, counts):
                 self.cache.commit(rid, n)
         return logits
 
-    def _context(self, a: BatchArrays) -> StepContext:
+    # ---- index arrays on the device -------------------------------------------------
+    def _context(self, a: BatchArrays, ids32: np.ndarray, rows32: np.ndarray, dst32=None, dst64=None,
+                 max_ctx_len: Optional[int] = None, host_lengths: bool = True):
+        """Uploads the step's arrays (two copies) and returns (StepContext, ids, wanted rows,
+        32-bit buffer, 64-bit buffer); the first three are views of the two buffers."""
         dev = self.device
-        to = lambda x: torch.from_numpy(np.ascontiguousarray(x)).to(dev)
         G = len(self.cache.groups)
+        T, B = a.num_tokens, a.num_seqs
+        no_slots = np.full(T, -1, dtype=np.int64)
+        parts32 = [ids32, a.positions, a.tok_seq, a.cu_q, a.ctx_lens, rows32, a.block_tables]
+        parts64 = [a.state_slots.astype(np.int64), a.slots, no_slots]
+        d32, o32 = self._staging.upload(parts32, torch.int32, dst32)
+        d64, o64 = self._staging.upload(parts64, torch.int64, dst64)
+        self._staging.mark()
+        v32 = lambda i, n: d32[o32[i]:o32[i] + n]
+        P = a.max_pages
+        tables = v32(6, G * B * P).view(G, B, P)
+        slots = d64[o64[1]:o64[1] + G * T].view(G, T)
         q_lens = np.diff(a.cu_q)
-        return StepContext(
-            num_tokens=a.num_tokens, num_seqs=a.num_seqs, dtype=self.model.dtype, device=dev,
-            positions=to(a.positions), tok_seq=to(a.tok_seq), cu_q=to(a.cu_q),
-            ctx_lens=to(a.ctx_lens), state_slots=to(a.state_slots.astype(np.int64)),
-            slots=[to(a.slots[g]) for g in range(G)],
-            block_tables=[to(a.block_tables[g]) for g in range(G)],
-            cu_q_host=a.cu_q.tolist(), ctx_lens_host=a.ctx_lens.tolist(),
-            max_q_len=int(q_lens.max()), max_ctx_len=int(a.ctx_lens.max()),
-            no_slots=torch.full((a.num_tokens,), -1, dtype=torch.int64, device=dev),
-            empty_f32=self._empty_f32)
+        ctx = StepContext(
+            num_tokens=T, num_seqs=B, dtype=self.model.dtype, device=dev,
+            positions=v32(1, T), tok_seq=v32(2, T), cu_q=v32(3, B + 1), ctx_lens=v32(4, B),
+            state_slots=d64[o64[0]:o64[0] + B],
+            slots=[slots[g] for g in range(G)], block_tables=[tables[g] for g in range(G)],
+            cu_q_host=a.cu_q.tolist() if host_lengths else (),
+            ctx_lens_host=a.ctx_lens.tolist() if host_lengths else (),
+            max_q_len=int(q_lens.max()),
+            max_ctx_len=int(a.ctx_lens.max()) if max_ctx_len is None else int(max_ctx_len),
+            no_slots=d64[o64[2]:o64[2] + T], empty_f32=self._empty_f32)
+        return ctx, v32(0, T), v32(5, rows32.size), d32, d64
+
+    # ---- decode steps as HIP graphs ---------------------------------------------------
+    def _replay_decode(self, a: BatchArrays, ids32: np.ndarray, rows32: np.ndarray) -> torch.Tensor:
+        """A step of single tokens.  The graph of (batch size, context bucket) computes the
+        logits of every row; the wanted rows are gathered afterwards.  Kernels whose grid
+        depends on the longest context are recorded for the bucket's upper bound (work
+        beyond a request's own length ends at once)."""
+        B = a.num_seqs
+        longest = int(a.ctx_lens.max())
+        bucket = 1024
+        while bucket < longest:
+            bucket *= 4
+        key = (B, bucket)
+        all_rows = np.zeros(B, dtype=np.int32)
+        all_rows[:rows32.size] = rows32
+        g = self._graphs.get(key)
+        if g is None:
+            ctx, ids, want, d32, d64 = self._context(a, ids32, all_rows, max_ctx_len=bucket, host_lengths=False)
+            every_row = torch.arange(B, dtype=torch.int32, device=self.device)
+            cur = torch.cuda.current_stream(self.device)
+            side = torch.cuda.Stream(self.device)
+            side.wait_stream(cur)
+            with torch.cuda.stream(side):       # a first run outside the graph warms every kernel up
+                self.model.forward(ids, ctx, self.layer_caches, every_row)
+            cur.wait_stream(side)
+            torch.cuda.synchronize(self.device)
+            if self._graph_pool is None:
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                logits = self.model.forward(ids, ctx, self.layer_caches, every_row)
+            g = _DecodeGraph(graph, d32, d64, logits, want, keep=(every_row, ctx, ids))
+            self._graphs[key] = g
+        else:
+            self._context(a, ids32, all_rows, dst32=g.dev32, dst64=g.dev64, max_ctx_len=bucket,
+                          host_lengths=False)
+        g.graph.replay()
+        self.graph_replays += 1
+        if rows32.size == B and np.array_equal(rows32, np.arange(B)):
+            return g.logits.clone()
+        return g.logits.index_select(0, g.want[:rows32.size])

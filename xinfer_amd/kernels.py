@@ -354,15 +354,18 @@ def linear_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dt
     return out
 
 
-def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """bfloat16 x @ w.T with float32 accumulation.  Few rows (decode): the hand-written
-    streaming kernel.  Many rows: the vendor library (hipBLASLt through torch), which the
-    reference's engine also uses for its matrix products."""
+def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+                skinny_rows: int = SKINNY_ROWS) -> torch.Tensor:
+    """bfloat16 x @ w.T with float32 accumulation, rounded once to `out_dtype` (bfloat16 or
+    float32).  Up to `skinny_rows` rows (decode): the hand-written streaming kernel.  More
+    rows: the vendor library (hipBLASLt through torch), which the reference's engine also
+    uses for its matrix products."""
     _dev(x, w)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError("linear_bf16: operands must be bfloat16")
     out_dtype = out_dtype or torch.bfloat16
-    if 0 < x.shape[0] <= SKINNY_ROWS and x.shape[1] % 8 == 0:
+    if 0 < x.shape[0] <= min(skinny_rows, SKINNY_MAX_ROWS) and x.shape[1] % 8 == 0:
         return linear_skinny(x, w, out_dtype)
-    y = torch.nn.functional.linear(x, w)
-    return y if y.dtype == out_dtype else y.to(out_dtype)
+    if out_dtype == torch.float32:
+        return torch.mm(x, w.t(), out_dtype=torch.float32)
+    return torch.nn.functional.linear(x, w)

@@ -23,6 +23,8 @@ from .linear import Linear
 
 @register_mixer("attention")
 class PagedAttention(Mixer):
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, dtype: torch.dtype):
         super().__init__(spec, dtype)
         self.hidden = int(spec["hidden_size"])

@@ -94,6 +94,12 @@ class Stream:
 
 
 class Part:
+    # True if `forward` reads nothing of the step on the host (no lengths, no device-to-host
+    # copies) and launches the same kernels for every step of the same batch size, so that a
+    # decode step can be recorded once as a HIP graph and replayed.  Parts that do not say so
+    # keep the whole model on the launch-by-launch path.
+    graph_safe = False
+
     def __init__(self, spec: PartSpec, dtype: torch.dtype):
         self.spec = spec
         self.dtype = dtype
@@ -134,6 +140,8 @@ class PositionEncoding(Part):
 
 class Block:
     """Arrangement of a layer's parts around the residual stream."""
+
+    graph_safe = False
 
     def __init__(self, layer: LayerSpec, dtype: torch.dtype):
         self.layer = layer

@@ -51,6 +51,10 @@ class PreNormBlock(Block):
         self.norm1.load(store, f"{p}.{self.NORM_BEFORE_MIXER}", device)
         self.norm2.load(store, f"{p}.{self.NORM_BEFORE_FFN}", device)
 
+    @property
+    def graph_safe(self) -> bool:
+        return all(p.graph_safe for p in (self.mixer, self.ffn, self.norm1, self.norm2))
+
     def cache_need(self) -> Optional[KVNeed]:
         return self.mixer.cache_need()
 

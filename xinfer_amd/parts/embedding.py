@@ -18,6 +18,8 @@ from .linear import Linear
 
 
 class Embedding(Part):
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, dtype: torch.dtype):
         super().__init__(spec, dtype)
         self.vocab = int(spec["vocab_size"])
@@ -39,6 +41,8 @@ class Embedding(Part):
 
 
 class LMHead(Part):
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, dtype: torch.dtype):
         super().__init__(spec, dtype)
         self.tied = bool(spec.get("tied", False))
@@ -58,4 +62,7 @@ class LMHead(Part):
         self.proj = Linear(t)
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
-        return self.proj(h, out_dtype=torch.float32)
+        # float32 logits straight from the float32 sums for any number of rows; the streaming
+        # kernel serves every decode batch here, so a row's logits do not depend on how many
+        # rows were asked for
+        return self.proj(h, out_dtype=torch.float32, skinny_rows=kernels.SKINNY_MAX_ROWS)

@@ -25,7 +25,8 @@ class Linear:
         self.weight = weight.contiguous()
         self.out_features, self.in_features = weight.shape
 
-    def __call__(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    def __call__(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+                 skinny_rows: int = kernels.SKINNY_ROWS) -> torch.Tensor:
         w = self.weight
         out_dtype = out_dtype or x.dtype
         if w.dtype == torch.float32:
@@ -34,4 +35,4 @@ class Linear:
             return y if out_dtype == torch.float32 else y.to(out_dtype)
         if x.dtype != w.dtype:
             raise kernels.KernelError(f"linear: activations are {x.dtype} but the weight is {w.dtype}")
-        return kernels.linear_bf16(x, w, out_dtype)
+        return kernels.linear_bf16(x, w, out_dtype, skinny_rows)

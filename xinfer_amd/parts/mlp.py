@@ -19,6 +19,8 @@ from .linear import Linear
 
 @register_feed_forward("gated_mlp")
 class GatedMLP(FeedForward):
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, dtype: torch.dtype):
         super().__init__(spec, dtype)
         self.hidden = int(spec["hidden_size"])

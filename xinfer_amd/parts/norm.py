@@ -19,6 +19,8 @@ from .base import Norm, register_norm
 
 @register_norm("rmsnorm")
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, dtype: torch.dtype):
         super().__init__(spec, dtype)
         self.dim = int(spec["dim"])

@@ -17,6 +17,8 @@ from .base import PositionEncoding, register_position_encoding
 
 @register_position_encoding("rope")
 class RotaryEmbedding(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, dtype: torch.dtype):
         super().__init__(spec, dtype)
         self.head_dim = int(spec["head_dim"])
