@@ -361,7 +361,7 @@ def test_attention_prefill_mfma(nq, nkv, d, page, window, seqs):
     ref = _attention_ref(case, seqs, window, scale)
     q, kc, vt, bt = _mfma_inputs(case)
     cu, ctx = _cu_ctx(seqs)
-    qb = kernels.prefill_block(d)
+    qb = kernels.prefill_block(d, nq // nkv)
     tiles = torch.tensor([(b, q0) for b, (_, n) in enumerate(seqs) for q0 in range(0, n, qb)], dtype=torch.int32)
     out = kernels.attention_prefill_bf16(q, kc, vt, bt, tiles.to(DEV), cu.to(DEV), ctx.to(DEV), scale, window)
     err = (out.cpu().double() - ref).abs().max() / ref.abs().max()

@@ -1,6 +1,8 @@
-// bfloat16 paged causal GQA attention on the gfx950 matrix cores, for prefill and decode.
+// bfloat16 paged causal GQA attention on the gfx950 matrix cores: the wave-level step and
+// the split-K decode kernels (the prefill kernel, attention_prefill.hip, stages the same
+// operands through LDS).
 //
-// Both kernels are built on one wave-level step: 32 keys against NQT tiles of 16 query
+// The wave-level step: 32 keys against NQT tiles of 16 query
 // columns, with v_mfma_f32_16x16x32_bf16 and no transposes through LDS:
 //
 //   S^T[key, q] = K[key, :] . Q[q, :]          A = K rows      B = Q^T
@@ -173,72 +175,6 @@ struct WaveAttn {
 };
 
 // =====================================================================================
-// Prefill (and mixed batches): one workgroup of 4 waves per (query block, query head);
-// each wave owns NQT*16 consecutive query tokens and walks the keys they can see.
-//   tiles[i] = {sequence, first query token of the block within the sequence's portion}
-// =====================================================================================
-template <int KC, int DT, int NQT>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(
-    const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ vt_cache,
-    const int* __restrict__ block_tables, int max_pages, const int* __restrict__ tiles,
-    const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, bf16* __restrict__ out,
-    float scale_log2, int window, int page, int nq, int nkv, int d) {
-  constexpr int QW = 16 * NQT;  // queries per wave
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int r = lane & 15, j = lane >> 4;
-  const int seq = tiles[2 * blockIdx.x], q0_blk = tiles[2 * blockIdx.x + 1];
-  const int head = blockIdx.y;
-  const int q_begin = cu_q[seq], q_len = cu_q[seq + 1] - q_begin;
-  const int ctx = ctx_lens[seq];
-  const int q0 = q0_blk + wave * QW;  // first query of this wave within the portion
-  if (q0 >= q_len) return;
-  const int pos0 = ctx - q_len;  // position of the portion's first token
-
-  PagedKV kv{k_cache, vt_cache, block_tables + (size_t)seq * max_pages, page, nkv, d, head / (nq / nkv)};
-  WaveAttn<KC, DT, NQT> w;
-  w.init();
-  const bf16* q_rows[NQT];
-#pragma unroll
-  for (int ct = 0; ct < NQT; ++ct) {
-    const int qi = q0 + 16 * ct + r;
-    const bool ok = qi < q_len;
-    w.qpos[ct] = ok ? pos0 + qi : -1;
-    w.qlo[ct] = (ok && window > 0 && w.qpos[ct] - window + 1 > 0) ? w.qpos[ct] - window + 1 : 0;
-    q_rows[ct] = ok ? q + ((size_t)(q_begin + qi) * nq + head) * d : nullptr;
-  }
-  w.load_q(q_rows, d, j);
-  // range of keys this wave's queries see (wave-uniform)
-  const int n_q = min(QW, q_len - q0);
-  const int first_pos = pos0 + q0, last_pos = pos0 + q0 + n_q - 1;
-  const int lo_first = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
-  const int k_begin = lo_first & ~31;
-  for (int kb = k_begin; kb <= last_pos; kb += 32) {
-    // a step needs the mask unless every key is at or before every query and inside every window
-    const int lo_last = (window > 0 && last_pos - window + 1 > 0) ? last_pos - window + 1 : 0;
-    const bool masked = (kb + 31 > first_pos) || (kb < lo_last);
-    w.step(kv, kb, ctx - 1, scale_log2, masked, r, j);
-  }
-#pragma unroll
-  for (int ct = 0; ct < NQT; ++ct) {
-    const float lt = w.total_l(ct);
-    const int qi = q0 + 16 * ct + r;
-    if (qi >= q_len) continue;
-    const float inv = 1.f / lt;
-    bf16* o = out + ((size_t)(q_begin + qi) * nq + head) * d;
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      if (16 * dt >= d) break;
-      bf16* op = o + 16 * dt + 4 * j;
-      const f32x4 a = w.acc[dt][ct];
-      op[0] = __float2bfloat16(a[0] * inv);
-      op[1] = __float2bfloat16(a[1] * inv);
-      op[2] = __float2bfloat16(a[2] * inv);
-      op[3] = __float2bfloat16(a[3] * inv);
-    }
-  }
-}
-
-// =====================================================================================
 // Decode: every sequence has one query token.  Workgroup (split, kv head, sequence): the
 // query heads of the kv group are the columns of one tile; the workgroup's four waves
 // take alternate 32-key steps of its chunk of `keys_per_wg` keys and merge through LDS.
@@ -369,31 +305,6 @@ extern "C" {
 int xi_attention_mfma_supported(int nq, int nkv, int d, int page) {
   return (d % 16 == 0 && d >= 16 && d <= 256 && page % 8 == 0 && nq % nkv == 0) ? 1 : 0;
 }
-
-int xi_attention_prefill_bf16(const void* q, const void* k_cache, const void* vt_cache, const int* block_tables,
-                              int max_pages, const int* tiles, int n_tiles, const int* cu_q,
-                              const int* ctx_lens, void* out, float scale, int window, int page, int nq,
-                              int nkv, int d, hipStream_t stream) {
-  XI_CHECK(xi_attention_mfma_supported(nq, nkv, d, page), "attention_prefill: unsupported sizes nq=%d nkv=%d d=%d page=%d",
-           nq, nkv, d, page);
-  XI_CHECK(nq <= 65535, "attention_prefill: too many heads");
-  if (n_tiles == 0) return 0;
-  dim3 grid(n_tiles, nq);
-  const float sl = scale * kLog2e;
-#define XI_PF(KC, DT, NQT)                                                                           \
-  attn_prefill_kernel<KC, DT, NQT><<<grid, 256, 0, stream>>>(                                        \
-      (const bf16*)q, (const bf16*)k_cache, (const bf16*)vt_cache, block_tables, max_pages, tiles, cu_q, \
-      ctx_lens, (bf16*)out, sl, window, page, nq, nkv, d)
-  if (d <= 64) XI_PF(2, 4, 2);
-  else if (d <= 128) XI_PF(4, 8, 2);
-  else XI_PF(8, 16, 1);
-#undef XI_PF
-  XI_LAUNCH_CHECK("attention_prefill");
-  return 0;
-}
-
-// Queries per block of the prefill kernel for a head size (the host builds `tiles` with it).
-int xi_attention_prefill_block(int d) { return d <= 128 ? 128 : 64; }
 
 int xi_attention_decode_bf16(const void* q, const void* k_cache, const void* vt_cache, const int* block_tables,
                              int max_pages, const int* ctx_lens, void* out, float* part_o, float* part_ml,

@@ -1,0 +1,327 @@
+// bfloat16 paged causal GQA attention for prompt portions (and any mixed batch) on the
+// gfx950 matrix cores, with K and V^T tiles staged through LDS.
+//
+// A workgroup of four waves owns a block of consecutive query positions of one sequence
+// and GH query heads that share one kv head.  It walks the keys those queries can see in
+// tiles of 32: all 256 threads copy the K tile [32 keys, d] and the V^T tile [d, 32 keys]
+// from the paged cache into LDS (double buffered; the next tile's global loads are in
+// flight while the current one is multiplied), and every wave multiplies the same tile with
+// its own NQT column tiles of 16 queries.  A column tile is (position block, head): with
+// four heads per kv head a wave holds the same 16 positions of the four heads, so a K/V
+// tile is fetched from memory once per kv head, not once per query head, and every 16-byte
+// LDS read feeds NQT matrix instructions.
+//
+// The arithmetic is that of the decode kernel (attention_mfma.hip): S^T = K . Q^T with
+// v_mfma_f32_16x16x32_bf16 so that a query's scores lie in the lanes of its column, softmax
+// in float32 (exp2, log2(e) folded into the scale), P^T rounded to bfloat16 feeds
+// O^T += V^T . P^T straight from registers.  Row m of the two K tiles of a step is key
+// 8*(m/4) + m%4 (+4 for the second), which makes lane group j hold keys 8j..8j+7 of both
+// products.  The accumulators are rescaled only when some running maximum moved.
+//
+// LDS rows are padded by 16 bytes: the 16 lanes that read one matrix operand together
+// then fall into 16 different 16-byte bank groups.
+//
+// Reference: PagedAttention::forward prefill branch,
+// /root/reference/src/models/layers/attention.rs:947-958 (varlen over cu_seqlens with a
+// cached prefix); golden formula /root/reference/tests/probes/compare_flashinfer_probe.py:51-73.
+#include "common.h"
+
+namespace xi {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr float kLog2eP = 1.4426950408889634f;
+constexpr int kKeys = 32;    // keys per tile
+constexpr int kVPad = 8;     // bf16 elements of padding per LDS row
+
+__device__ __forceinline__ bf16x8 ld8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
+__device__ __forceinline__ void st8(bf16* p, bf16x8 v) { *reinterpret_cast<bf16x8*>(p) = v; }
+__device__ __forceinline__ bf16x8 zero8p() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.f;
+  return z;
+}
+
+template <int KC, int DT, int NQT, int GH>
+__global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ vt_cache,
+    const int* __restrict__ block_tables, int max_pages, const int* __restrict__ tiles,
+    const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, bf16* __restrict__ out, float scale_log2,
+    int window, int page, int nq, int nkv, int d) {
+  constexpr int PB = NQT / GH;   // blocks of 16 positions per wave
+  constexpr int QW = 16 * PB;    // query positions per wave
+  constexpr int LI = (KC + 1) / 2;  // 16-byte chunks per thread and tile, for K and for V^T
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int krow = d + kVPad;           // elements per K row in LDS
+  const int vrow = kKeys + kVPad;       // elements per V^T row in LDS
+  const int stage = kKeys * krow + d * vrow;
+  bf16* lds = reinterpret_cast<bf16*>(smem);
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, j = lane >> 4;
+  const int g = nq / nkv, groups = g / GH;
+  const int kvh = blockIdx.x / groups;
+  const int h0 = kvh * g + (blockIdx.x - kvh * groups) * GH;
+  const int seq = tiles[2 * blockIdx.y], q0_blk = tiles[2 * blockIdx.y + 1];
+  const int q_begin = cu_q[seq], q_len = cu_q[seq + 1] - q_begin;
+  const int ctx = ctx_lens[seq];
+  const int pos0 = ctx - q_len;         // position of the portion's first token
+  const int k_last = ctx - 1;
+  const int* bt = block_tables + (size_t)seq * max_pages;
+
+  // keys the workgroup walks
+  const int wg_nq = min(4 * QW, q_len - q0_blk);
+  const int wg_first = pos0 + q0_blk, wg_last = wg_first + wg_nq - 1;
+  const int wg_lo = (window > 0 && wg_first - window + 1 > 0) ? wg_first - window + 1 : 0;
+  const int k_begin = wg_lo & ~(kKeys - 1);
+
+  // this wave's queries
+  const int q0 = q0_blk + wave * QW;
+  const bool active = q0 < q_len;
+  const int n_q = active ? min(QW, q_len - q0) : 0;
+  const int first_pos = pos0 + q0, last_pos = first_pos + n_q - 1;
+  const int lo_first = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
+  const int lo_last = (window > 0 && last_pos - window + 1 > 0) ? last_pos - window + 1 : 0;
+  const int wave_k_begin = lo_first & ~(kKeys - 1);
+
+  bf16x8 qb[NQT][KC];
+  f32x4 acc[DT][NQT];
+  float m_run[NQT], l_run[NQT];
+  int qpos[NQT], qlo[NQT];
+#pragma unroll
+  for (int ct = 0; ct < NQT; ++ct) {
+    const int pb = ct / GH, hh = ct - pb * GH;
+    const int qi = q0 + 16 * pb + r;
+    const bool ok = active && qi < q_len;
+    qpos[ct] = ok ? pos0 + qi : -1;
+    qlo[ct] = (ok && window > 0 && qpos[ct] - window + 1 > 0) ? qpos[ct] - window + 1 : 0;
+    const bf16* qrow = q + ((size_t)(q_begin + (ok ? qi : 0)) * nq + h0 + hh) * d;
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+      const int off = 32 * c + 8 * j;
+      qb[ct][c] = (ok && off < d) ? ld8(qrow + off) : zero8p();
+    }
+    m_run[ct] = -INFINITY;
+    l_run[ct] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[dt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  // ---- cooperative tile copy: chunk idx = tid + 256*i of 4*d chunks, for K and for V^T
+  const int cpk = d >> 3;            // 16-byte chunks per key row
+  const int n_chunks = 4 * d;        // 32 keys * d/8 = d rows * 4 key groups
+  bf16x8 kreg[LI], vreg[LI];
+  auto fetch = [&](int kb) {
+#pragma unroll
+    for (int i = 0; i < LI; ++i) {
+      const int idx = tid + 256 * i;
+      if (idx < n_chunks) {
+        const int kl = idx / cpk, ch = idx - kl * cpk;
+        int key = kb + kl;
+        if (key > k_last) key = k_last;
+        const int kp = bt[key / page];
+        kreg[i] = ld8(k_cache + (((size_t)kp * nkv + kvh) * page + key % page) * d + 8 * ch);
+        const int row = idx >> 2, kg = idx & 3;
+        int key0 = kb + 8 * kg;
+        if (key0 > k_last) key0 = k_last & ~7;
+        const int vp = bt[key0 / page];
+        vreg[i] = ld8(vt_cache + (((size_t)vp * nkv + kvh) * d + row) * page + key0 % page);
+      }
+    }
+  };
+  auto stash = [&](int buf) {
+    bf16* Ks = lds + buf * stage;
+    bf16* Vs = Ks + kKeys * krow;
+#pragma unroll
+    for (int i = 0; i < LI; ++i) {
+      const int idx = tid + 256 * i;
+      if (idx < n_chunks) {
+        const int kl = idx / cpk, ch = idx - kl * cpk;
+        st8(Ks + kl * krow + 8 * ch, kreg[i]);
+        st8(Vs + (idx >> 2) * vrow + 8 * (idx & 3), vreg[i]);
+      }
+    }
+  };
+
+  fetch(k_begin);
+  stash(0);
+  __syncthreads();
+  int buf = 0;
+  for (int kb = k_begin; kb <= wg_last; kb += kKeys) {
+    const bool more = kb + kKeys <= wg_last;
+    if (more) fetch(kb + kKeys);
+    if (active && kb >= wave_k_begin && kb <= last_pos) {
+      const bf16* Ks = lds + buf * stage;
+      const bf16* Vs = Ks + kKeys * krow;
+      // a step needs the mask unless every key is at or before every query and inside every window
+      const bool masked = (kb + kKeys - 1 > first_pos) || (kb < lo_last);
+      const int kr0 = 8 * (r >> 2) + (r & 3);
+      bf16x8 ka[2][KC];
+#pragma unroll
+      for (int c = 0; c < KC; ++c) {
+        const int off = 32 * c + 8 * j;
+        if (off < d) {
+          ka[0][c] = ld8(Ks + kr0 * krow + off);
+          ka[1][c] = ld8(Ks + (kr0 + 4) * krow + off);
+        } else {
+          ka[0][c] = zero8p();
+          ka[1][c] = zero8p();
+        }
+      }
+      bf16x8 pb_[NQT];
+#pragma unroll
+      for (int ct = 0; ct < NQT; ++ct) {
+        f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+          s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[0][c], qb[ct][c], s0, 0, 0, 0);
+          s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[1][c], qb[ct][c], s1, 0, 0, 0);
+        }
+        float s[8];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          s[v] = s0[v] * scale_log2;
+          s[4 + v] = s1[v] * scale_log2;
+        }
+        if (masked) {
+          const int key0 = kb + 8 * j;
+#pragma unroll
+          for (int v = 0; v < 8; ++v) {
+            const int key = key0 + v;
+            if (key > qpos[ct] || key < qlo[ct]) s[v] = -INFINITY;
+          }
+        }
+        float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+        mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+        const float m_new = fmaxf(m_run[ct], mx);
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        float psum = 0.f;
+#pragma unroll
+        for (int v = 0; v < 8; ++v) {
+          const float p = __builtin_amdgcn_exp2f(s[v] - m_safe);
+          psum += p;
+          pb_[ct][v] = (__bf16)p;
+        }
+        if (__any(m_new != m_run[ct])) {   // some query's maximum moved: rescale this tile's sums
+          const float corr = __builtin_amdgcn_exp2f(m_run[ct] - m_safe);
+          l_run[ct] *= corr;
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) {
+            acc[dt][ct][0] *= corr;
+            acc[dt][ct][1] *= corr;
+            acc[dt][ct][2] *= corr;
+            acc[dt][ct][3] *= corr;
+          }
+          m_run[ct] = m_new;
+        }
+        l_run[ct] += psum;
+      }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        if (16 * dt < d) {
+          const bf16x8 va = ld8(Vs + (16 * dt + r) * vrow + 8 * j);
+#pragma unroll
+          for (int ct = 0; ct < NQT; ++ct)
+            acc[dt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb_[ct], acc[dt][ct], 0, 0, 0);
+        }
+      }
+    }
+    if (more) stash(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
+  }
+
+  if (!active) return;
+#pragma unroll
+  for (int ct = 0; ct < NQT; ++ct) {
+    float lt = l_run[ct] + __shfl_xor(l_run[ct], 16, kWave);
+    lt += __shfl_xor(lt, 32, kWave);
+    const int pb = ct / GH, hh = ct - pb * GH;
+    const int qi = q0 + 16 * pb + r;
+    if (qi >= q_len) continue;
+    const float inv = 1.f / lt;
+    bf16* o = out + ((size_t)(q_begin + qi) * nq + h0 + hh) * d;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      if (16 * dt >= d) break;
+      bf16* op = o + 16 * dt + 4 * j;
+      const f32x4 a = acc[dt][ct];
+      op[0] = __float2bfloat16(a[0] * inv);
+      op[1] = __float2bfloat16(a[1] * inv);
+      op[2] = __float2bfloat16(a[2] * inv);
+      op[3] = __float2bfloat16(a[3] * inv);
+    }
+  }
+}
+
+static inline int heads_per_wave(int g, int nqt) {
+  if (nqt >= 4 && g % 4 == 0) return 4;
+  if (g % 2 == 0) return 2;
+  return 1;
+}
+static inline int column_tiles(int d) { return d <= 128 ? 4 : 2; }
+
+}  // namespace xi
+
+using namespace xi;
+
+extern "C" {
+
+int xi_attention_mfma_supported(int nq, int nkv, int d, int page);
+
+// Query positions per workgroup for a head size and a number of query heads per kv head
+// (the host builds `tiles` in steps of it).
+int xi_attention_prefill_block(int d, int g) {
+  const int nqt = column_tiles(d);
+  return 64 * (nqt / heads_per_wave(g, nqt));
+}
+
+// tiles int32 [n_tiles, 2] = (sequence, first query position of the block within the
+// sequence's portion), first positions being multiples of xi_attention_prefill_block.
+int xi_attention_prefill_bf16(const void* q, const void* k_cache, const void* vt_cache, const int* block_tables,
+                              int max_pages, const int* tiles, int n_tiles, const int* cu_q,
+                              const int* ctx_lens, void* out, float scale, int window, int page, int nq,
+                              int nkv, int d, hipStream_t stream) {
+  XI_CHECK(xi_attention_mfma_supported(nq, nkv, d, page), "attention_prefill: unsupported sizes nq=%d nkv=%d d=%d page=%d",
+           nq, nkv, d, page);
+  XI_CHECK(n_tiles >= 0 && n_tiles <= 65535, "attention_prefill: %d query blocks are too many for one launch", n_tiles);
+  if (n_tiles == 0) return 0;
+  const int g = nq / nkv;
+  const int nqt = column_tiles(d);
+  const int gh = heads_per_wave(g, nqt);
+  dim3 grid(nkv * (g / gh), n_tiles);
+  const size_t lds = 2 * (size_t)(kKeys * (d + kVPad) + d * (kKeys + kVPad)) * sizeof(bf16);
+  const float sl = scale * kLog2eP;
+#define XI_PF(KC, DT, NQT, GH)                                                                          \
+  do {                                                                                                  \
+    auto kern = attn_prefill_lds_kernel<KC, DT, NQT, GH>;                                               \
+    if (lds > 48 * 1024) {                                                                              \
+      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                         (int)lds);                                                     \
+      XI_CHECK(e == hipSuccess, "attention_prefill: cannot get %zu bytes of LDS: %s", lds,              \
+               hipGetErrorString(e));                                                                   \
+    }                                                                                                   \
+    kern<<<grid, 256, lds, stream>>>((const bf16*)q, (const bf16*)k_cache, (const bf16*)vt_cache,       \
+                                     block_tables, max_pages, tiles, cu_q, ctx_lens, (bf16*)out, sl,    \
+                                     window, page, nq, nkv, d);                                         \
+  } while (0)
+#define XI_PF_GH(KC, DT, NQT)            \
+  do {                                   \
+    if (gh == 4) XI_PF(KC, DT, NQT, 4);  \
+    else if (gh == 2) XI_PF(KC, DT, NQT, 2); \
+    else XI_PF(KC, DT, NQT, 1);          \
+  } while (0)
+  if (d <= 64) XI_PF_GH(2, 4, 4);
+  else if (d <= 128) XI_PF_GH(4, 8, 4);
+  else if (gh == 2) XI_PF(8, 16, 2, 2);
+  else XI_PF(8, 16, 2, 1);
+#undef XI_PF_GH
+#undef XI_PF
+  XI_LAUNCH_CHECK("attention_prefill");
+  return 0;
+}
+
+}  // extern "C"

@@ -247,7 +247,7 @@ def mfma_attention_supported(nq: int, nkv: int, d: int, page: int) -> bool:
 
 def attention_prefill_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, scale, window=0, out=None):
     """MFMA attention for any mix of portions.  tiles int32 [n, 2] = (sequence, first query
-    token of a block of `prefill_block(d)` tokens within the sequence's portion)."""
+    token of a block of `prefill_block(d, nq // nkv)` tokens within the sequence's portion)."""
     _dev(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, out)
     T, nq, d = q.shape
     nkv, page = k_cache.shape[1], k_cache.shape[2]
@@ -267,8 +267,10 @@ def attention_prefill_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_
     return out
 
 
-def prefill_block(d: int) -> int:
-    return int(lib().xi_attention_prefill_block(int(d)))
+def prefill_block(d: int, group: int = 1) -> int:
+    """Query positions per workgroup of the prefill kernel for a head size and a number of
+    query heads per kv head."""
+    return int(lib().xi_attention_prefill_block(int(d), int(group)))
 
 
 def attention_decode_bf16(q, k_cache, vt_cache, block_tables, ctx_lens, max_ctx_len, scale, window=0, out=None):
@@ -309,12 +311,14 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx
         g = nq // nkv
         if ctx.max_q_len == 1 and g <= 16 and (4 * g * d + 8 * g) * 4 <= 64 * 1024:
             return attention_decode_bf16(q, k_cache, v_cache, bt, ctx.ctx_lens, ctx.max_ctx_len, scale, window)
-        qb = prefill_block(d)
+        qb = prefill_block(d, g)
         key = ("attention_tiles", qb)
         tiles = ctx.scratch.get(key)
         if tiles is None:
             rows = [(b, q0) for b in range(ctx.num_seqs)
                     for q0 in range(0, ctx.cu_q_host[b + 1] - ctx.cu_q_host[b], qb)]
+            # blocks that see the most keys start first: the short ones fill the gaps they leave
+            rows.sort(key=lambda t: -(ctx.ctx_lens_host[t[0]] - (ctx.cu_q_host[t[0] + 1] - ctx.cu_q_host[t[0]]) + t[1]))
             tiles = torch.tensor(rows, dtype=torch.int32, device=q.device).reshape(-1, 2)
             ctx.scratch[key] = tiles
         return attention_prefill_bf16(q, k_cache, v_cache, bt, tiles, ctx.cu_q, ctx.ctx_lens, scale, window)
