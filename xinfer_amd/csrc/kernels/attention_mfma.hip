@@ -300,10 +300,10 @@ using namespace xi;
 
 extern "C" {
 
-// Sizes the MFMA kernels take: head_dim a multiple of 16 up to 256, page size a multiple of 8,
-// at most 16 query heads per kv head (decode).  Returns 1 if supported.
+// Sizes the MFMA kernels take: head_dim a multiple of 16 up to 256, page size a power of two
+// of at least 8, at most 16 query heads per kv head (decode).  Returns 1 if supported.
 int xi_attention_mfma_supported(int nq, int nkv, int d, int page) {
-  return (d % 16 == 0 && d >= 16 && d <= 256 && page % 8 == 0 && nq % nkv == 0) ? 1 : 0;
+  return (d % 16 == 0 && d >= 16 && d <= 256 && page >= 8 && (page & (page - 1)) == 0 && nq % nkv == 0) ? 1 : 0;
 }
 
 int xi_attention_decode_bf16(const void* q, const void* k_cache, const void* vt_cache, const int* block_tables,

@@ -3,10 +3,11 @@
 //
 // A workgroup of four waves owns a block of consecutive query positions of one sequence
 // and GH query heads that share one kv head.  It walks the keys those queries can see in
-// tiles of 32: all 256 threads copy the K tile [32 keys, d] and the V^T tile [d, 32 keys]
+// tiles of 64: all 256 threads copy the K tile [64 keys, d] and the V^T tile [d, 64 keys]
 // from the paged cache into LDS (double buffered; the next tile's global loads are in
-// flight while the current one is multiplied), and every wave multiplies the same tile with
-// its own NQT column tiles of 16 queries.  A column tile is (position block, head): with
+// flight while the current one is multiplied, and the sequence's block table sits in LDS so
+// that a tile costs one memory round trip, not two), and every wave multiplies the same
+// tile, in two steps of 32 keys, with its own NQT column tiles of 16 queries.  A column tile is (position block, head): with
 // four heads per kv head a wave holds the same 16 positions of the four heads, so a K/V
 // tile is fetched from memory once per kv head, not once per query head, and every 16-byte
 // LDS read feeds NQT matrix instructions.
@@ -32,8 +33,9 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr float kLog2eP = 1.4426950408889634f;
-constexpr int kKeys = 32;    // keys per tile
+constexpr int kKeys = 64;    // keys per tile (two steps of 32)
 constexpr int kVPad = 8;     // bf16 elements of padding per LDS row
+constexpr float kSlack = 8.f;  // how far (log2) a score may exceed the softmax reference point
 
 __device__ __forceinline__ bf16x8 ld8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 __device__ __forceinline__ void st8(bf16* p, bf16x8 v) { *reinterpret_cast<bf16x8*>(p) = v; }
@@ -49,15 +51,18 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ vt_cache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ tiles,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, bf16* __restrict__ out, float scale_log2,
-    int window, int page, int nq, int nkv, int d) {
+    int window, int page_shift, int nq, int nkv, int d) {
+  const int page = 1 << page_shift;
   constexpr int PB = NQT / GH;   // blocks of 16 positions per wave
   constexpr int QW = 16 * PB;    // query positions per wave
-  constexpr int LI = (KC + 1) / 2;  // 16-byte chunks per thread and tile, for K and for V^T
+  constexpr int LI = KC;         // 16-byte chunks per thread and tile, for K and for V^T
   extern __shared__ __align__(16) unsigned char smem[];
-  const int krow = d + kVPad;           // elements per K row in LDS
+  constexpr int krow = 32 * KC + kVPad;  // elements per K row in LDS: head_dim rounded up to the
+                                         // 32-wide steps of the matrix product (the rest is zero)
   const int vrow = kKeys + kVPad;       // elements per V^T row in LDS
   const int stage = kKeys * krow + d * vrow;
   bf16* lds = reinterpret_cast<bf16*>(smem);
+  int* bt_s = reinterpret_cast<int*>(smem + 2 * (size_t)stage * sizeof(bf16));  // [max_pages]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, j = lane >> 4;
@@ -69,7 +74,11 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
   const int ctx = ctx_lens[seq];
   const int pos0 = ctx - q_len;         // position of the portion's first token
   const int k_last = ctx - 1;
-  const int* bt = block_tables + (size_t)seq * max_pages;
+  {
+    const int* bt = block_tables + (size_t)seq * max_pages;
+    const int n_pages = (k_last + page) / page;    // pages that hold keys 0..k_last
+    for (int i = threadIdx.x; i < n_pages; i += 256) bt_s[i] = bt[i];
+  }
 
   // keys the workgroup walks
   const int wg_nq = min(4 * QW, q_len - q0_blk);
@@ -84,7 +93,7 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
   const int first_pos = pos0 + q0, last_pos = first_pos + n_q - 1;
   const int lo_first = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
   const int lo_last = (window > 0 && last_pos - window + 1 > 0) ? last_pos - window + 1 : 0;
-  const int wave_k_begin = lo_first & ~(kKeys - 1);
+  const int wave_k_begin = lo_first & ~31;
 
   bf16x8 qb[NQT][KC];
   f32x4 acc[DT][NQT];
@@ -109,26 +118,42 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
     for (int dt = 0; dt < DT; ++dt) acc[dt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  // ---- cooperative tile copy: chunk idx = tid + 256*i of 4*d chunks, for K and for V^T
-  const int cpk = d >> 3;            // 16-byte chunks per key row
-  const int n_chunks = 4 * d;        // 32 keys * d/8 = d rows * 4 key groups
+  // ---- cooperative tile copy.  K tile: 64 keys of 4*KC 16-byte chunks (chunks past
+  // head_dim are zero), thread t moves chunks t, t + 256, ...; in LDS the keys of each
+  // 32-key step are permuted so that the 16 rows one matrix operand reads are consecutive:
+  // key k sits at row 16*((k>>2)&1) + 4*(k>>3) + (k&3) of its step.  V^T tile: d rows of 8
+  // key groups, same distribution.
+  constexpr int CPK = 4 * KC;        // chunks per K row in LDS
+  const int n_vchunks = 8 * d;
+  int c_kl[LI], c_koff[LI], c_kdst[LI], c_vdst[LI];
+#pragma unroll
+  for (int i = 0; i < LI; ++i) {
+    const int idx = tid + 256 * i;
+    const int kl = idx / CPK, ch = idx % CPK;
+    const int k32 = kl & 31;
+    c_kl[i] = kl;
+    c_koff[i] = 8 * ch < d ? 8 * ch : -1;       // -1: a chunk of zeros
+    c_kdst[i] = ((kl & 32) + 16 * ((k32 >> 2) & 1) + 4 * (k32 >> 3) + (k32 & 3)) * krow + 8 * ch;
+    c_vdst[i] = (idx >> 3) * vrow + 8 * (idx & 7);
+  }
+  const size_t kv_head_stride = (size_t)d << page_shift;     // elements of one (page, kv head) block
   bf16x8 kreg[LI], vreg[LI];
   auto fetch = [&](int kb) {
 #pragma unroll
     for (int i = 0; i < LI; ++i) {
       const int idx = tid + 256 * i;
-      if (idx < n_chunks) {
-        const int kl = idx / cpk, ch = idx - kl * cpk;
-        int key = kb + kl;
-        if (key > k_last) key = k_last;
-        const int kp = bt[key / page];
-        kreg[i] = ld8(k_cache + (((size_t)kp * nkv + kvh) * page + key % page) * d + 8 * ch);
-        const int row = idx >> 2, kg = idx & 3;
-        int key0 = kb + 8 * kg;
-        if (key0 > k_last) key0 = k_last & ~7;
-        const int vp = bt[key0 / page];
-        vreg[i] = ld8(vt_cache + (((size_t)vp * nkv + kvh) * d + row) * page + key0 % page);
-      }
+      int key = kb + c_kl[i];
+      key = key > k_last ? k_last : key;
+      const int kp = bt_s[key >> page_shift];
+      const bf16* ksrc = k_cache + ((size_t)kp * nkv + kvh) * kv_head_stride +
+                         (size_t)(key & (page - 1)) * d + (c_koff[i] < 0 ? 0 : c_koff[i]);
+      kreg[i] = ld8(ksrc);
+      int key0 = kb + 8 * (idx & 7);
+      key0 = key0 > k_last ? (k_last & ~7) : key0;
+      const int vp = bt_s[key0 >> page_shift];
+      const int vr = (idx >> 3) < d ? (idx >> 3) : d - 1;     // rows past head_dim are not stored
+      vreg[i] = ld8(vt_cache + ((size_t)vp * nkv + kvh) * kv_head_stride + ((size_t)vr << page_shift) +
+                    (key0 & (page - 1)));
     }
   };
   auto stash = [&](int buf) {
@@ -136,39 +161,37 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
     bf16* Vs = Ks + kKeys * krow;
 #pragma unroll
     for (int i = 0; i < LI; ++i) {
-      const int idx = tid + 256 * i;
-      if (idx < n_chunks) {
-        const int kl = idx / cpk, ch = idx - kl * cpk;
-        st8(Ks + kl * krow + 8 * ch, kreg[i]);
-        st8(Vs + (idx >> 2) * vrow + 8 * (idx & 3), vreg[i]);
-      }
+      st8(Ks + c_kdst[i], c_koff[i] < 0 ? zero8p() : kreg[i]);   // zeroed here, not at the load: the
+                                                                  // load stays in flight meanwhile
+      if (tid + 256 * i < n_vchunks) st8(Vs + c_vdst[i], vreg[i]);
     }
   };
 
+  __syncthreads();   // the block table is in LDS
   fetch(k_begin);
   stash(0);
+  // every load so far (the queries among them) has landed before the loop starts, so that
+  // inside it only the tile in flight is ever waited for: vmcnt(0), other counters untouched
+  __builtin_amdgcn_s_waitcnt(0x0F70);
   __syncthreads();
   int buf = 0;
-  for (int kb = k_begin; kb <= wg_last; kb += kKeys) {
-    const bool more = kb + kKeys <= wg_last;
-    if (more) fetch(kb + kKeys);
+  for (int kt = k_begin; kt <= wg_last; kt += kKeys) {
+    const bool more = kt + kKeys <= wg_last;
+    if (more) fetch(kt + kKeys);
+#pragma unroll
+    for (int sub = 0; sub < kKeys / 32; ++sub) {
+    const int kb = kt + 32 * sub;
     if (active && kb >= wave_k_begin && kb <= last_pos) {
-      const bf16* Ks = lds + buf * stage;
-      const bf16* Vs = Ks + kKeys * krow;
+      const bf16* Ks = lds + buf * stage + 32 * sub * krow;
+      const bf16* Vs = lds + buf * stage + kKeys * krow + 32 * sub;
       // a step needs the mask unless every key is at or before every query and inside every window
-      const bool masked = (kb + kKeys - 1 > first_pos) || (kb < lo_last);
-      const int kr0 = 8 * (r >> 2) + (r & 3);
+      const bool masked = (kb + 31 > first_pos) || (kb < lo_last);
       bf16x8 ka[2][KC];
 #pragma unroll
       for (int c = 0; c < KC; ++c) {
         const int off = 32 * c + 8 * j;
-        if (off < d) {
-          ka[0][c] = ld8(Ks + kr0 * krow + off);
-          ka[1][c] = ld8(Ks + (kr0 + 4) * krow + off);
-        } else {
-          ka[0][c] = zero8p();
-          ka[1][c] = zero8p();
-        }
+        ka[0][c] = ld8(Ks + r * krow + off);
+        ka[1][c] = ld8(Ks + (16 + r) * krow + off);
       }
       bf16x8 pb_[NQT];
 #pragma unroll
@@ -182,8 +205,8 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
         float s[8];
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-          s[v] = s0[v] * scale_log2;
-          s[4 + v] = s1[v] * scale_log2;
+          s[v] = s0[v];
+          s[4 + v] = s1[v];
         }
         if (masked) {
           const int key0 = kb + 8 * j;
@@ -193,20 +216,17 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
             if (key > qpos[ct] || key < qlo[ct]) s[v] = -INFINITY;
           }
         }
-        float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
-        mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-        const float m_new = fmaxf(m_run[ct], mx);
-        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        float psum = 0.f;
-#pragma unroll
-        for (int v = 0; v < 8; ++v) {
-          const float p = __builtin_amdgcn_exp2f(s[v] - m_safe);
-          psum += p;
-          pb_[ct][v] = (__bf16)p;
-        }
-        if (__any(m_new != m_run[ct])) {   // some query's maximum moved: rescale this tile's sums
-          const float corr = __builtin_amdgcn_exp2f(m_run[ct] - m_safe);
+        // this lane's largest score (raw: the scale is positive and is applied with the shift)
+        const float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+        // The reference point m_run of the exponentials only has to be near the maximum: it
+        // moves when some score exceeds it by more than 2^kSlack, which is rare after the
+        // first keys, and then the sums so far are rescaled.  P stays below 2^kSlack.
+        if (__any(mx * scale_log2 > m_run[ct] + kSlack)) {
+          float mc = mx * scale_log2;
+          mc = fmaxf(mc, __shfl_xor(mc, 16, kWave));
+          mc = fmaxf(mc, __shfl_xor(mc, 32, kWave));
+          const float m_new = fmaxf(m_run[ct], mc);
+          const float corr = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_run[ct] - m_new);
           l_run[ct] *= corr;
 #pragma unroll
           for (int dt = 0; dt < DT; ++dt) {
@@ -216,6 +236,14 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
             acc[dt][ct][3] *= corr;
           }
           m_run[ct] = m_new;
+        }
+        const float m_safe = (m_run[ct] == -INFINITY) ? 0.f : m_run[ct];
+        float psum = 0.f;
+#pragma unroll
+        for (int v = 0; v < 8; ++v) {
+          const float p = __builtin_amdgcn_exp2f(fmaf(s[v], scale_log2, -m_safe));
+          psum += p;
+          pb_[ct][v] = (__bf16)p;
         }
         l_run[ct] += psum;
       }
@@ -228,6 +256,7 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
             acc[dt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb_[ct], acc[dt][ct], 0, 0, 0);
         }
       }
+    }
     }
     if (more) stash(buf ^ 1);
     __syncthreads();
@@ -293,11 +322,18 @@ int xi_attention_prefill_bf16(const void* q, const void* k_cache, const void* vt
   const int nqt = column_tiles(d);
   const int gh = heads_per_wave(g, nqt);
   dim3 grid(nkv * (g / gh), n_tiles);
-  const size_t lds = 2 * (size_t)(kKeys * (d + kVPad) + d * (kKeys + kVPad)) * sizeof(bf16);
   const float sl = scale * kLog2eP;
+  XI_CHECK(sl > 0.f, "attention_prefill: the scale must be positive");
+  int page_shift = -1;
+  for (int b = 0; b < 31; ++b)
+    if ((1 << b) == page) page_shift = b;
+  XI_CHECK(page_shift >= 3, "attention_prefill: the page size %d must be a power of two of at least 8", page);
 #define XI_PF(KC, DT, NQT, GH)                                                                          \
   do {                                                                                                  \
     auto kern = attn_prefill_lds_kernel<KC, DT, NQT, GH>;                                               \
+    const size_t lds = 2 * (size_t)(kKeys * (32 * KC + kVPad) + d * (kKeys + kVPad)) * sizeof(bf16) +   \
+                       (size_t)max_pages * sizeof(int);                                                 \
+    XI_CHECK(lds <= 160 * 1024, "attention_prefill: block tables of %d pages do not fit in LDS", max_pages); \
     if (lds > 48 * 1024) {                                                                              \
       hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, \
                                          (int)lds);                                                     \
@@ -306,7 +342,7 @@ int xi_attention_prefill_bf16(const void* q, const void* k_cache, const void* vt
     }                                                                                                   \
     kern<<<grid, 256, lds, stream>>>((const bf16*)q, (const bf16*)k_cache, (const bf16*)vt_cache,       \
                                      block_tables, max_pages, tiles, cu_q, ctx_lens, (bf16*)out, sl,    \
-                                     window, page, nq, nkv, d);                                         \
+                                     window, page_shift, nq, nkv, d);                                   \
   } while (0)
 #define XI_PF_GH(KC, DT, NQT)            \
   do {                                   \
