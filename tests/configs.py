@@ -27,3 +27,19 @@ TINY = {
                     layer_types=["sliding_attention", "full_attention", "sliding_attention"]),
         seed=2, linear_std=0.05, norm_std=0.2, page_size=16),
 }
+
+
+# Real layer sizes (Qwen3-8B and Qwen3-32B) with few layers and a small vocabulary: the
+# kernels run at the head size, group, widths and K lengths they serve in production.
+REAL = {
+    "8B": dict(
+        config=_cfg(num_hidden_layers=2, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
+                    head_dim=128, intermediate_size=12288, vocab_size=2003, rope_theta=1e6,
+                    rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=1024),
+        seed=3, linear_std=0.02, norm_std=0.1, page_size=64),
+    "32B": dict(
+        config=_cfg(num_hidden_layers=1, hidden_size=5120, num_attention_heads=64, num_key_value_heads=8,
+                    head_dim=128, intermediate_size=25600, vocab_size=1501, rope_theta=1e6,
+                    rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=1024),
+        seed=4, linear_std=0.02, norm_std=0.1, page_size=64),
+}

@@ -24,3 +24,20 @@ def model_dirs(tmp_path_factory):
         write_random_model(d, t["config"], t["seed"], t["linear_std"], t["norm_std"])
         out[name] = d
     return out
+
+
+@pytest.fixture(scope="session")
+def real_model_dirs(tmp_path_factory):
+    """Model folders with real layer sizes and few layers (see configs.REAL), written on demand."""
+    from configs import REAL
+    from xinfer_amd.weights import write_random_model
+    root = tmp_path_factory.mktemp("real_models")
+    made = {}
+
+    def get(name):
+        if name not in made:
+            t = REAL[name]
+            made[name] = write_random_model(str(root / name), t["config"], t["seed"], t["linear_std"],
+                                            t["norm_std"])
+        return made[name]
+    return get

@@ -9,7 +9,7 @@ import torch
 
 import harness
 import plain_qwen3 as plain
-from configs import TINY
+from configs import REAL, TINY
 
 pytestmark = pytest.mark.gpu
 
@@ -101,3 +101,32 @@ def test_float32_does_not_depend_on_cutting(name, model_dirs):
     for key in a:
         assert torch.equal(a[key], b[key]), key
         assert torch.equal(a[key], c[key]), key
+
+
+# ---- real layer sizes ---------------------------------------------------------------------------
+@pytest.mark.parametrize("name", list(REAL))
+def test_real_layer_sizes(name, real_model_dirs):
+    """Qwen3-8B and Qwen3-32B layer sizes (few layers, small vocabulary): whole requests, a
+    mixed trace with pages used again and a tail decoded one by one, in float32 and in
+    bfloat16, against the plain implementation."""
+    from xinfer_amd.engine import ModelRunner, load_model
+    t = REAL[name]
+    d = real_model_dirs(name)
+    vocab, page = t["config"]["vocab_size"], t["page_size"]
+    rng = random.Random(5)
+    reqs = {f"r{i}": harness.random_prompt(rng, n, vocab) for i, n in enumerate([70, 200, 129, 33])}
+    pm = plain.PlainModel(d)
+    ref = {rid: pm.logits(toks) for rid, toks in reqs.items()}
+    del pm
+    for dtype in DTYPES:
+        model = load_model(d, dtype, "cuda:0")
+        for what, steps in (("whole", harness.trace_whole(reqs)), ("mixed", harness.trace_mixed(reqs, 3, max_live=3)),
+                            ("tail", harness.trace_tail_one_by_one(reqs, tail=8))):
+            need = harness.tokens_needed(steps, page)
+            runner = ModelRunner(model, page_size=page, num_pages=need // page, max_requests=4)
+            got = harness.replay(runner, steps)
+            rel = harness.compare(got, ref, harness.TOL[dtype], f"{name}/{dtype}/{what}")
+            print(f"{name}/{dtype}/{what}: worst error {rel:.2e} of the largest logit")
+            del runner
+        del model
+        torch.cuda.empty_cache()
