@@ -241,6 +241,15 @@ def gemm_tn(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] =
 DECODE_KEYS_PER_WORKGROUP = 256
 
 
+def decode_keys_per_workgroup(pairs: int, span: int) -> int:
+    """Keys per workgroup of the split-K decode kernel for `pairs` (sequence, kv head) pairs of
+    up to `span` keys: 256 (each of the four waves takes two steps, both in flight at once)
+    unless that makes thousands of workgroups, where 512 halves the partial results to write
+    and combine (measured on an MI355X at contexts of 512 to 16384)."""
+    kpw = DECODE_KEYS_PER_WORKGROUP
+    return kpw if pairs * (span // kpw + 1) <= 3000 else 2 * kpw
+
+
 def mfma_attention_supported(nq: int, nkv: int, d: int, page: int) -> bool:
     return bool(lib().xi_attention_mfma_supported(nq, nkv, d, page))
 
@@ -273,8 +282,10 @@ def prefill_block(d: int, group: int = 1) -> int:
     return int(lib().xi_attention_prefill_block(int(d), int(group)))
 
 
-def attention_decode_bf16(q, k_cache, vt_cache, block_tables, ctx_lens, max_ctx_len, scale, window=0, out=None):
-    """Split-K MFMA attention for a batch in which every sequence has one token (q [B, nq, d])."""
+def attention_decode_bf16(q, k_cache, vt_cache, block_tables, ctx_lens, max_ctx_len, scale, window=0, out=None,
+                          keys_per_workgroup=None):
+    """Split-K MFMA attention for a batch in which every sequence has one token (q [B, nq, d]).
+    `keys_per_workgroup` (a multiple of 128) is chosen from the batch if not given."""
     _dev(q, k_cache, vt_cache, block_tables, ctx_lens, out)
     B, nq, d = q.shape
     nkv, page = k_cache.shape[1], k_cache.shape[2]
@@ -285,7 +296,7 @@ def attention_decode_bf16(q, k_cache, vt_cache, block_tables, ctx_lens, max_ctx_
     if block_tables.shape[0] != B or ctx_lens.shape != (B,):
         raise KernelError("attention_decode: one block table row and one context length per sequence")
     span = min(int(max_ctx_len), int(window) + 31) if window > 0 else int(max_ctx_len)
-    kpw = DECODE_KEYS_PER_WORKGROUP
+    kpw = int(keys_per_workgroup or decode_keys_per_workgroup(B * nkv, span))
     max_splits = span // kpw + 1
     part_o = torch.empty((B, nq, max_splits, d), dtype=torch.float32, device=q.device)
     part_ml = torch.empty((B, nq, max_splits, 2), dtype=torch.float32, device=q.device)
