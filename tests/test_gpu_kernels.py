@@ -225,16 +225,62 @@ def test_qk_norm_rope_kv(dtype, nq, nkv, d, rot, interleaved, norm):
         assert torch.equal(vcd[p, :, o].double(), v[t]), t
     # the transposed V pool [pages, nkv, d, page] holds the same values
     vt = torch.zeros((pages, nkv, d, page), dtype=dtype, device=DEV)
-    kernels.qk_norm_rope_kv(
+    q_out_t = kernels.qk_norm_rope_kv(
         qkv.to(DEV), qw.to(DEV) if norm else None, kw.to(DEV) if norm else None, eps, cos.to(DEV),
-        sin.to(DEV), rot, interleaved, positions.to(DEV), slots.to(DEV), kc.to(DEV), vt, nq, nkv, d,
-        v_transposed=True)
+        sin.to(DEV), rot, interleaved, positions.to(DEV), slots.to(DEV), (kct := kc.to(DEV)), vt, nq, nkv, d,
+        v_transposed=True, vector_min_tokens=1)
     assert torch.equal(vt.cpu().transpose(2, 3), vcd)
+    # q and K of the transposed form (another kernel for bfloat16) against the same reference
+    assert (q_out_t.cpu().double() - q).abs().max() / q.abs().max() < tol
+    kct = kct.cpu().double()
+    for t in range(T):
+        p, o = int(slots[t]) // page, int(slots[t]) % page
+        assert (kct[p, :, o] - k[t]).abs().max() / k.abs().max() < tol, t
+    assert float(kct.permute(0, 2, 1, 3).reshape(pages * page, -1)[~torch.isin(torch.arange(pages * page), slots)].abs().max()) == 0.0
     # nothing but the named slots was written
     touched = torch.zeros(pages * page, dtype=torch.bool)
     touched[slots] = True
     flat = kcd.permute(0, 2, 1, 3).reshape(pages * page, -1)
     assert float(flat[~touched].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("nq,nkv,d,rot,interleaved", [(32, 8, 128, 128, False), (6, 3, 48, 32, False), (4, 4, 64, 64, True),
+                                                    (10, 2, 80, 80, False)])
+def test_qk_norm_rope_kv_many_tokens(nq, nkv, d, rot, interleaved):
+    """The bfloat16 form with the transposed V pool over several blocks of 64 tokens: runs of
+    tokens that follow each other in a page, a block that is not full, and tokens whose slot is
+    negative (nothing of theirs may be stored)."""
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(17)
+    T, page, pages, eps = 150, 16, 12, 1e-6
+    positions = torch.cat([torch.arange(40, 40 + 100), torch.arange(0, 50)]).to(torch.int32)
+    cos, sin = plain.rope_tables(1e6, rot, 256)
+    qkv = _rand((T, (nq + 2 * nkv) * d), torch.bfloat16, g)
+    qw, kw = 1 + 0.2 * torch.randn(d, generator=g), 1 + 0.2 * torch.randn(d, generator=g)
+    page_of = torch.randperm(pages, generator=g)
+    slots = torch.cat([page_of[(torch.arange(100) + 8) // page] * page + (torch.arange(100) + 8) % page,
+                       page_of[7 + torch.arange(50) // page] * page + torch.arange(50) % page]).to(torch.int64)
+    slots[torch.tensor([3, 64, 149])] = -1
+    kc = torch.zeros((pages, nkv, page, d), dtype=torch.bfloat16, device=DEV)
+    vt = torch.zeros((pages, nkv, d, page), dtype=torch.bfloat16, device=DEV)
+    q_out = kernels.qk_norm_rope_kv(qkv.to(DEV), qw.to(DEV), kw.to(DEV), eps, cos.to(DEV), sin.to(DEV), rot,
+                                    interleaved, positions.to(DEV), slots.to(DEV), kc, vt, nq, nkv, d,
+                                    v_transposed=True)
+    x = qkv.double().reshape(T, nq + 2 * nkv, d)
+    q = _rope_ref(plain.rms_norm(x[:, :nq], qw.double(), eps), positions.long(), cos, sin, rot, interleaved)
+    k = _rope_ref(plain.rms_norm(x[:, nq:nq + nkv], kw.double(), eps), positions.long(), cos, sin, rot, interleaved)
+    v = x[:, nq + nkv:]
+    tol = _tol(torch.bfloat16)
+    assert (q_out.cpu().double() - q).abs().max() / q.abs().max() < tol
+    want_k = torch.zeros((pages * page, nkv, d), dtype=torch.float64)
+    want_v = torch.zeros((pages * page, nkv, d), dtype=torch.float64)
+    keep = slots >= 0
+    want_k[slots[keep]] = k[keep]
+    want_v[slots[keep]] = v[keep]
+    got_k = kc.cpu().double().permute(0, 2, 1, 3).reshape(pages * page, nkv, d)
+    got_v = vt.cpu().double().permute(0, 3, 1, 2).reshape(pages * page, nkv, d)
+    assert (got_k - want_k).abs().max() / k.abs().max() < tol
+    assert torch.equal(got_v, want_v)
 
 
 def _paged_case(g, dtype, nq, nkv, d, page, seqs, extra_pages=3):

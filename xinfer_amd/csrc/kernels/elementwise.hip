@@ -279,6 +279,144 @@ __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, const float* _
   }
 }
 
+// The same for bfloat16 with the transposed V pool, 16 bytes per lane and one pass: a
+// workgroup owns one head of the packed row for a block of consecutive tokens.  A head of a
+// token is d/8 lanes of 8 elements (sums and the rotary partner are exchanged inside that
+// group of lanes), a wave holds 64/(d/8) tokens, the workgroup's waves hold the block.  The
+// workgroup of a V head turns its [tokens, d] tile through LDS so that the transposed pool
+// is written with lanes along the token axis: tokens that follow each other in a page
+// become one contiguous store.
+// Needs d % 8 == 0 and, for the half layout, rotary_dim % 16 == 0 (the partner of a lane's
+// 8 elements is then another lane's 8 elements).
+struct alignas(16) bf16x8v { bf16 v[8]; };
+
+__global__ __launch_bounds__(1024) void qk_norm_rope_kvt_bf16_kernel(
+    const bf16* __restrict__ qkv, const float* __restrict__ qw, const float* __restrict__ kw, float eps,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot, int interleaved,
+    const int* __restrict__ positions, const long long* __restrict__ slots, bf16* __restrict__ q_out,
+    bf16* __restrict__ k_cache, bf16* __restrict__ vt_cache, int page_size, int n_tok, int nq, int nkv, int d) {
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int heads = nq + 2 * nkv;
+  const int lph = d >> 3;          // lanes per head
+  const int hpw = 64 / lph;        // tokens a wave holds
+  const int tpw = (blockDim.x >> 6) * hpw;   // tokens of the workgroup (at most 64)
+  const int sub = lane / lph, c = lane - sub * lph;
+  const int h = blockIdx.y;
+  const int t0 = blockIdx.x * tpw;
+  const int tl = wave * hpw + sub;  // this lane's token within the block
+  const int t = t0 + tl;
+  const bool on = sub < hpw && t < n_tok;
+
+  if (h >= nq + nkv) {
+    // ---- a V head: tile into LDS, then lanes along the token axis
+    const int kvh = h - nq - nkv;
+    bf16* vs = reinterpret_cast<bf16*>(smem_raw);  // [tpw][d + 2]
+    const int vstride = d + 2;                      // an odd number of 32-bit words per row
+    if (on) {
+      const uint4 raw = *reinterpret_cast<const uint4*>(qkv + ((size_t)t * heads + h) * d + 8 * c);
+      unsigned* dst = reinterpret_cast<unsigned*>(vs + tl * vstride + 8 * c);
+      dst[0] = raw.x;
+      dst[1] = raw.y;
+      dst[2] = raw.z;
+      dst[3] = raw.w;
+    }
+    __syncthreads();
+    const int tok = lane;   // token of the block this lane writes
+    const long long slot = (tok < tpw && t0 + tok < n_tok) ? slots[t0 + tok] : -1;
+    if (slot >= 0) {
+      const long long page = slot / page_size;
+      const int off = (int)(slot - page * page_size);
+      bf16* dst = vt_cache + ((size_t)page * nkv + kvh) * d * page_size + off;
+      const bf16* src = vs + tok * vstride;
+      for (int i = wave; i < d; i += (int)(blockDim.x >> 6)) dst[(size_t)i * page_size] = src[i];
+    }
+    return;
+  }
+
+  // ---- a query head or a k head
+  const bool is_k = h >= nq;
+  float v[8];
+  {
+    bf16x8v x;
+    if (on) x = *reinterpret_cast<const bf16x8v*>(qkv + ((size_t)t * heads + h) * d + 8 * c);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = on ? to_float(x.v[e]) : 0.f;
+  }
+  const float* w = is_k ? kw : qw;
+  if (w) {
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += v[e] * v[e];
+    float total;
+    if ((lph & (lph - 1)) == 0) {
+      total = ss;
+      for (int off = 1; off < lph; off <<= 1) total += __shfl_xor(total, off, kWave);
+    } else {
+      total = 0.f;
+      const int first = lane - c;
+      for (int o = 0; o < lph; ++o) total += __shfl(ss, first + o, kWave);
+    }
+    const float inv = rsqrtf(total / (float)d + eps);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      v[e] *= inv;
+      v[e] *= w[8 * c + e];
+    }
+  }
+  const int half = rot >> 1;
+  const int pos = positions[t < n_tok ? t : n_tok - 1];
+  float o[8];
+  if (interleaved) {
+#pragma unroll
+    for (int e = 0; e < 8; e += 2) {
+      const int i = 8 * c + e;
+      if (i < rot) {
+        const float cs = cos_t[(size_t)pos * half + (i >> 1)], sn = sin_t[(size_t)pos * half + (i >> 1)];
+        o[e] = v[e] * cs - v[e + 1] * sn;
+        o[e + 1] = v[e] * sn + v[e + 1] * cs;
+      } else {
+        o[e] = v[e];
+        o[e + 1] = v[e + 1];
+      }
+    }
+  } else {
+    const int hop = rot >> 4;        // lanes between rotary partners
+    const bool in_rot = 8 * c < rot;
+    const bool first = 8 * c < half;
+    int partner = first ? lane + hop : lane - hop;
+    if (!in_rot) partner = lane;
+    const int p0 = first ? 8 * c : 8 * c - half;   // pair index of this lane's first element
+    float cs[8], sn[8];
+    if (in_rot) {
+      const float4* cp = reinterpret_cast<const float4*>(cos_t + (size_t)pos * half + p0);
+      const float4* sp = reinterpret_cast<const float4*>(sin_t + (size_t)pos * half + p0);
+      const float4 c0 = cp[0], c1 = cp[1], s0 = sp[0], s1 = sp[1];
+      cs[0] = c0.x; cs[1] = c0.y; cs[2] = c0.z; cs[3] = c0.w; cs[4] = c1.x; cs[5] = c1.y; cs[6] = c1.z; cs[7] = c1.w;
+      sn[0] = s0.x; sn[1] = s0.y; sn[2] = s0.z; sn[3] = s0.w; sn[4] = s1.x; sn[5] = s1.y; sn[6] = s1.z; sn[7] = s1.w;
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float pv = __shfl(v[e], partner, kWave);
+      o[e] = !in_rot ? v[e] : (first ? v[e] * cs[e] - pv * sn[e] : pv * sn[e] + v[e] * cs[e]);
+    }
+  }
+  if (!on) return;
+  bf16x8v y;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) y.v[e] = from_float<bf16>(o[e]);
+  if (!is_k) {
+    *reinterpret_cast<bf16x8v*>(q_out + ((size_t)t * nq + h) * d + 8 * c) = y;
+  } else {
+    const long long slot = slots[t];
+    if (slot >= 0) {
+      const long long page = slot / page_size;
+      const int off = (int)(slot - page * page_size);
+      *reinterpret_cast<bf16x8v*>(k_cache + (((size_t)page * nkv + (h - nq)) * page_size + off) * d + 8 * c) = y;
+    }
+  }
+}
+
 }  // namespace xi
 
 using namespace xi;
@@ -353,12 +491,30 @@ int xi_qk_norm_rope_kv(const void* qkv, int dtype, const float* qw, const float*
                        const float* cos_t, const float* sin_t, int rot, int interleaved,
                        const int* positions, const long long* slots, void* q_out, void* k_cache,
                        void* v_cache, int page_size, int n_tok, int nq, int nkv, int d, int v_transposed,
-                       hipStream_t stream) {
+                       int vector_min_tokens, hipStream_t stream) {
   XI_CHECK(n_tok >= 0 && nq > 0 && nkv > 0 && d > 0 && page_size > 0,
            "qk_norm_rope_kv: bad sizes T=%d nq=%d nkv=%d d=%d page=%d", n_tok, nq, nkv, d, page_size);
   XI_CHECK(rot >= 0 && rot <= d && rot % 2 == 0, "qk_norm_rope_kv: rotary_dim %d must be even and <= head_dim %d", rot, d);
   XI_CHECK((qw == nullptr) == (kw == nullptr), "qk_norm_rope_kv: q and k norm weights must both be given or both absent");
   if (n_tok == 0) return 0;
+  // Many tokens (prompt portions): the vectorized form.  Few (decode steps): one wave per
+  // (token, head) below, whose shorter chain of dependent loads finishes sooner.
+  if (n_tok >= vector_min_tokens && dtype == kBF16 && v_transposed && d % 8 == 0 && d <= 256 &&
+      (interleaved || rot % 16 == 0) &&
+      ((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)cos_t | (uintptr_t)sin_t) % 16 == 0) {
+    const int lph = d / 8, hpw = 64 / lph;
+    int n_waves = 64 / hpw;                       // waves of a workgroup: at most 64 tokens, at most 16 waves
+    if (n_waves > 16) n_waves = 16;
+    const int tpw = n_waves * hpw;
+    const unsigned blocks_x = (unsigned)((n_tok + tpw - 1) / tpw);
+    XI_CHECK(nq + 2 * nkv <= 65535, "qk_norm_rope_kv: too many heads");
+    const size_t lds = (size_t)tpw * (d + 2) * sizeof(bf16);
+    qk_norm_rope_kvt_bf16_kernel<<<dim3(blocks_x, nq + 2 * nkv), n_waves * 64, lds, stream>>>(
+        (const bf16*)qkv, qw, kw, eps, cos_t, sin_t, rot, interleaved, positions, slots, (bf16*)q_out,
+        (bf16*)k_cache, (bf16*)v_cache, page_size, n_tok, nq, nkv, d);
+    XI_LAUNCH_CHECK("qk_norm_rope_kv");
+    return 0;
+  }
   const long long waves = (long long)n_tok * (nq + 2 * nkv);
   const int wpb = 4;
   const long long blocks = (waves + wpb - 1) / wpb;

@@ -139,10 +139,12 @@ def qk_norm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor],
                     sin: torch.Tensor, rotary_dim: int, interleaved: bool,
                     positions: torch.Tensor, slots: torch.Tensor, k_cache: torch.Tensor,
                     v_cache: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
-                    q_out: Optional[torch.Tensor] = None, v_transposed: bool = False) -> torch.Tensor:
+                    q_out: Optional[torch.Tensor] = None, v_transposed: bool = False,
+                    vector_min_tokens: int = 128) -> torch.Tensor:
     """Per-head RMSNorm of q and k (if weights are given), rotation by position, q to q_out
     [T, nq, d], k and v into the paged cache [pages, nkv, page_size, d] at `slots`; with
-    `v_transposed` the V pool is [pages, nkv, d, page_size]."""
+    `v_transposed` the V pool is [pages, nkv, d, page_size].  From `vector_min_tokens` tokens
+    on, bfloat16 with the transposed pool runs the vectorized kernel."""
     _dev(qkv, q_weight, k_weight, cos, sin, positions, slots, k_cache, v_cache, q_out)
     nq, nkv, d = num_heads, num_kv_heads, head_dim
     T = qkv.shape[0]
@@ -170,7 +172,7 @@ def qk_norm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor],
         _p(qkv), _code(qkv, "qk_norm_rope_kv"), _p(q_weight), _p(k_weight), ctypes.c_float(eps),
         _p(cos), _p(sin), int(rotary_dim), int(bool(interleaved)), _p(positions), _p(slots),
         _p(q_out), _p(k_cache), _p(v_cache), int(k_cache.shape[2]), T, nq, nkv, d,
-        int(bool(v_transposed)), _stream()))
+        int(bool(v_transposed)), int(vector_min_tokens), _stream()))
     return q_out
 
 
