@@ -69,7 +69,16 @@ def _lib_dir() -> str:
         os.remove(probe)
         return d
     except OSError:
-        d = os.path.join(tempfile.gettempdir(), f"xinfer_amd-{os.getuid()}", "_lib")
+        # a folder of this user alone: nobody else may plant a library there
+        base = os.path.join(tempfile.gettempdir(), f"xinfer_amd-{os.getuid()}")
+        try:
+            os.makedirs(base, mode=0o700, exist_ok=True)
+            st = os.stat(base)
+            if st.st_uid != os.getuid() or (st.st_mode & 0o022):
+                raise OSError("not ours")
+        except OSError:
+            base = tempfile.mkdtemp(prefix="xinfer_amd-")
+        d = os.path.join(base, "_lib")
         os.makedirs(d, exist_ok=True)
         return d
 
@@ -86,7 +95,9 @@ def _find(tool: str, extra: List[str]) -> Optional[str]:
 
 def _run(cmd: List[str], what: str) -> None:
     env = dict(os.environ)
-    env.setdefault("HOME", tempfile.gettempdir())      # hipcc wants a HOME for its caches
+    home = env.get("HOME")
+    if not home or not os.path.isdir(home) or not os.access(home, os.W_OK):
+        env["HOME"] = tempfile.gettempdir()            # hipcc wants a HOME it can write its caches to
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env)
     if r.returncode != 0:
         raise BuildError(f"{what} failed (exit {r.returncode}):\n{' '.join(cmd)}\n{r.stdout}")

@@ -77,6 +77,58 @@ __global__ __launch_bounds__(kSampleThreads) void argmax_kernel(const float* __r
   if (threadIdx.x == 0) out[blockIdx.x] = r;
 }
 
+// argmax in two stages, so that a few rows still use many compute units: stage one takes
+// the row in `n_chunks` slices (lowest index wins ties within a slice), stage two merges the
+// slices' winners in slice order (lowest index wins again).
+__global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __restrict__ logits, int V, int n_chunks,
+                                                             float* __restrict__ pval, int* __restrict__ pidx) {
+  __shared__ float sf[4];
+  __shared__ int si[4];
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  const int per = (V + n_chunks - 1) / n_chunks;
+  const int lo = chunk * per, hi = min(V, lo + per);
+  const float* r = logits + (size_t)row * V;
+  float best = -INFINITY;
+  int idx = 0x7fffffff;
+  for (int i = lo + threadIdx.x; i < hi; i += 256) {
+    const float v = r[i];
+    if (v > best || (v == best && i < idx)) { best = v; idx = i; }
+  }
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    const float ob = __shfl_xor(best, off, kWave);
+    const int oi = __shfl_xor(idx, off, kWave);
+    if (ob > best || (ob == best && oi < idx)) { best = ob; idx = oi; }
+  }
+  if ((threadIdx.x & (kWave - 1)) == 0) { sf[threadIdx.x / kWave] = best; si[threadIdx.x / kWave] = idx; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int i = 1; i < 4; ++i)
+      if (sf[i] > best || (sf[i] == best && si[i] < idx)) { best = sf[i]; idx = si[i]; }
+    pval[(size_t)row * n_chunks + chunk] = best;
+    pidx[(size_t)row * n_chunks + chunk] = idx;
+  }
+}
+
+__global__ __launch_bounds__(64) void argmax_merge_kernel(const float* __restrict__ pval, const int* __restrict__ pidx,
+                                                          int n_chunks, int* __restrict__ out) {
+  const int row = blockIdx.x;
+  float best = -INFINITY;
+  int idx = 0x7fffffff;
+  for (int c = threadIdx.x; c < n_chunks; c += kWave) {
+    const float v = pval[(size_t)row * n_chunks + c];
+    const int i = pidx[(size_t)row * n_chunks + c];
+    if (v > best || (v == best && i < idx)) { best = v; idx = i; }
+  }
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    const float ob = __shfl_xor(best, off, kWave);
+    const int oi = __shfl_xor(idx, off, kWave);
+    if (ob > best || (ob == best && oi < idx)) { best = ob; idx = oi; }
+  }
+  if (threadIdx.x == 0) out[row] = idx;
+}
+
 // logits[row, t] -= count(t) * freq + presence for each token t among `recent[row, :]`
 // (entries < 0 are padding).
 __global__ void penalty_kernel(float* __restrict__ logits, int V, const int* __restrict__ recent, int n_recent,
@@ -100,12 +152,102 @@ __global__ void penalty_kernel(float* __restrict__ logits, int V, const int* __r
   }
 }
 
-// count of p >= x and sum of p > x over the row
-__device__ __forceinline__ int count_ge(const float* p, int V, float x, int* si) {
-  int c = 0;
-  for (int i = threadIdx.x; i < V; i += kSampleThreads) c += p[i] >= x;
-  return block_sum_i(c, si);
+// ---- selection without sorting -------------------------------------------------------------
+// Both cut-offs are "walk the values in descending order until a running total reaches a
+// target": for top-k the total counts tokens, for top-p it adds probabilities.  Probabilities
+// are non-negative floats, so their bit patterns order like the values, and the walk is done
+// on a histogram of bit fields: 11 bits, then 11, then 9, each level one pass over the row
+// that looks only at values inside the bin the level above chose.  Totals are integers
+// (probabilities in units of 2^-40), so they do not depend on the order of the atomic adds.
+typedef unsigned long long u64;
+constexpr int kBins = 2048;
+constexpr float kFix = 1099511627776.f;  // 2^40
+
+__device__ __forceinline__ u64 shfl_up_u64(u64 v, int delta) {
+  const unsigned lo = __shfl_up((unsigned)v, delta, kWave), hi = __shfl_up((unsigned)(v >> 32), delta, kWave);
+  return ((u64)hi << 32) | lo;
 }
+
+// Bins hold weights w[0..n_bins).  Walking bins from the highest down, finds the bin b with
+// (total of bins above b) < target <= (total of bins above b) + w[b]; returns it in *bin and
+// the total above it in *above.  *bin = -1 if the target exceeds the total of all bins.
+// scan: kSampleWaves + 2 u64 of LDS.
+__device__ void find_crossing(const u64* w, int n_bins, u64 target, u64* scan, int* bin, u64* above) {
+  const int per = (n_bins + kSampleThreads - 1) / kSampleThreads;
+  const int top = n_bins - 1 - (int)threadIdx.x * per;      // this thread's highest bin
+  u64 local = 0;
+  for (int i = 0; i < per; ++i)
+    if (top - i >= 0) local += w[top - i];
+  // exclusive prefix over threads, thread 0 first
+  u64 incl = local;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const u64 o = shfl_up_u64(incl, d);
+    if (lane >= d) incl += o;
+  }
+  __syncthreads();
+  if (lane == kWave - 1) scan[wave] = incl;
+  if (threadIdx.x == 0) {
+    *bin = -1;
+    *above = 0;
+  }
+  __syncthreads();
+  u64 before = incl - local;
+  for (int i = 0; i < wave; ++i) before += scan[i];
+  u64 run = before;
+  for (int i = 0; i < per; ++i) {
+    const int b = top - i;
+    if (b < 0) break;
+    const u64 wb = w[b];
+    if (run < target && target <= run + wb) {
+      *bin = b;
+      *above = run;
+    }
+    run += wb;
+  }
+  __syncthreads();
+}
+
+// Descends the three levels.  weighted: totals add probabilities (top-p), else count tokens
+// (top-k).  Returns the bit pattern of the value at which the walk reaches `target` and, in
+// *above, the total of everything strictly greater than that value; *at = number of tokens
+// equal to it.  Returns 0xffffffff if the target exceeds the total over positive values.
+__device__ unsigned select_value(const float* p, int V, bool weighted, u64 target, u64* hist, int* cnt_hist,
+                                 u64* scan, int* s_bin, u64* s_above, u64* above, int* at) {
+  unsigned prefix = 0;    // bits chosen so far (the high ones)
+  u64 total_above = 0;
+  const int shifts[3] = {20, 9, 0};
+  const int widths[3] = {11, 11, 9};
+  for (int level = 0; level < 3; ++level) {
+    const int shift = shifts[level], n_bins = 1 << widths[level];
+    for (int i = threadIdx.x; i < n_bins; i += kSampleThreads) {
+      hist[i] = 0;
+      cnt_hist[i] = 0;
+    }
+    __syncthreads();
+    const unsigned hi_mask = level == 0 ? 0u : (0xffffffffu << (shift + widths[level]));
+    for (int i = threadIdx.x; i < V; i += kSampleThreads) {
+      const float pi = p[i];
+      const unsigned bits = __float_as_uint(pi);
+      if (bits == 0 || (bits & hi_mask) != (prefix & hi_mask)) continue;   // zero, or outside the chosen bin
+      const int b = (bits >> shift) & (n_bins - 1);
+      atomicAdd(&hist[b], weighted ? (u64)(pi * kFix) : (u64)1);
+      if (level == 2) atomicAdd(&cnt_hist[b], 1);
+    }
+    __syncthreads();
+    find_crossing(hist, n_bins, target - total_above, scan, s_bin, s_above);
+    const int b = *s_bin;
+    if (b < 0) return 0xffffffffu;
+    prefix |= (unsigned)b << shift;
+    total_above += *s_above;
+    if (level == 2) *at = cnt_hist[b];
+    __syncthreads();
+  }
+  *above = total_above;
+  return prefix;
+}
+
 __device__ __forceinline__ float sum_gt(const float* p, int V, float x, float* sf) {
   float s = 0.f;
   for (int i = threadIdx.x; i < V; i += kSampleThreads) s += p[i] > x ? p[i] : 0.f;
@@ -120,6 +262,11 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   __shared__ int si[kSampleWaves];
   __shared__ float scan_f[kSampleThreads];
   __shared__ int scan_i[kSampleThreads];
+  __shared__ u64 hist[kBins];
+  __shared__ int cnt_hist[kBins];
+  __shared__ u64 scan64[kSampleWaves];
+  __shared__ int s_bin;
+  __shared__ u64 s_above;
   __shared__ int result;
   const int row = blockIdx.x;
   const float* lg = logits + (size_t)row * V;
@@ -148,43 +295,39 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   int ties = 0;
   const int k = top_k[row];
   if (k > 0 && k < V) {
-    // largest x with count(p >= x) >= k, i.e. the k-th largest value
-    unsigned bits = 0;
-    for (int b = 30; b >= 0; --b) {
-      const unsigned cand = bits | (1u << b);
-      if (count_ge(p, V, __uint_as_float(cand), si) >= k) bits = cand;
+    // the k-th largest value, the number of tokens above it, and how many of its ties fit
+    u64 above;
+    int at;
+    const unsigned bits = select_value(p, V, false, (u64)k, hist, cnt_hist, scan64, &s_bin, &s_above, &above, &at);
+    if (bits != 0xffffffffu) {   // else fewer than k tokens have a positive probability: keep them all
+      v = __uint_as_float(bits);
+      ties = k - (int)above;
+      mass = sum_gt(p, V, v, sf) + (float)ties * v;
     }
-    v = __uint_as_float(bits);
-    const int n_gt = count_ge(p, V, __uint_as_float(bits + 1), si);
-    ties = k - n_gt;
-    mass = sum_gt(p, V, v, sf) + (float)ties * v;
   }
   const float tp = top_p[row];
   if (tp > 0.f && tp < 1.f) {
     const float target = tp * mass;
-    // largest x with sum(p > x) >= target; the kept values are those above it
-    unsigned bits = 0;
-    if (sum_gt(p, V, 0.f, sf) >= target) {
-      for (int b = 30; b >= 0; --b) {
-        const unsigned cand = bits | (1u << b);
-        if (sum_gt(p, V, __uint_as_float(cand), sf) >= target) bits = cand;
+    // the smallest value whose strictly greater mass is still below the target: the last
+    // token kept in descending order has it (logits_processor.rs:82-111)
+    u64 above;
+    int at = 0;
+    const unsigned bits = select_value(p, V, true, (u64)(target * kFix), hist, cnt_hist, scan64, &s_bin, &s_above,
+                                       &above, &at);
+    if (bits != 0xffffffffu) {
+      float vm = __uint_as_float(bits);
+      int cnt = at;
+      if (vm <= v) {   // top-k already cut higher (or here): its bound and its ties stand
+        vm = v;
+        cnt = ties;
       }
-      bits += 1;  // smallest x whose strictly-greater mass is below the target
+      const float s_above_f = sum_gt(p, V, vm, sf);
+      int keep = (int)ceilf((target - s_above_f) / vm);
+      keep = max(1, min(keep, cnt));
+      v = vm;
+      ties = keep;
+      mass = s_above_f + (float)ties * v;
     }
-    const float x = fmaxf(__uint_as_float(bits), v);
-    // the smallest kept value is the smallest actual value >= x
-    float vm = INFINITY;
-    for (int i = threadIdx.x; i < V; i += kSampleThreads)
-      if (p[i] >= x && p[i] > 0.f) vm = fminf(vm, p[i]);
-    vm = block_min_f(vm, sf);
-    const float s_above = sum_gt(p, V, vm, sf);
-    int cnt = count_ge(p, V, vm, si) - count_ge(p, V, __uint_as_float(__float_as_uint(vm) + 1), si);
-    if (vm == v) cnt = ties;  // top-k already limited the ties at this value
-    int keep = (int)ceilf((target - s_above) / vm);
-    keep = max(1, min(keep, cnt));
-    v = vm;
-    ties = keep;
-    mass = s_above + (float)ties * v;
   }
 
   // draw: walk the kept tokens in index order until the cumulative mass passes u * mass
@@ -262,11 +405,24 @@ using namespace xi;
 
 extern "C" {
 
-int xi_argmax(const float* logits, int rows, int V, int* out, hipStream_t stream) {
+// Chunks stage one of the argmax cuts a row of V logits into.
+int xi_argmax_chunks(int V) { return V >= 16384 ? 32 : 1; }
+
+// pval / pidx: scratch [rows, xi_argmax_chunks(V)] (unused when that is 1).
+int xi_argmax(const float* logits, int rows, int V, int* out, float* pval, int* pidx, hipStream_t stream) {
   XI_CHECK(rows >= 0 && V > 0, "argmax: bad sizes rows=%d V=%d", rows, V);
   if (rows == 0) return 0;
-  argmax_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, V, out);
-  XI_LAUNCH_CHECK("argmax");
+  const int n_chunks = xi_argmax_chunks(V);
+  if (n_chunks == 1) {
+    argmax_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, V, out);
+    XI_LAUNCH_CHECK("argmax");
+    return 0;
+  }
+  XI_CHECK(pval != nullptr && pidx != nullptr && rows <= 65535, "argmax: scratch for %d chunks is missing", n_chunks);
+  argmax_partial_kernel<<<dim3(n_chunks, rows), 256, 0, stream>>>(logits, V, n_chunks, pval, pidx);
+  XI_LAUNCH_CHECK("argmax_partial");
+  argmax_merge_kernel<<<rows, 64, 0, stream>>>(pval, pidx, n_chunks, out);
+  XI_LAUNCH_CHECK("argmax_merge");
   return 0;
 }
 

@@ -91,9 +91,17 @@ class Sampler:
     def argmax(self, logits: torch.Tensor) -> torch.Tensor:
         kernels._dev(logits)
         kernels._want(logits, torch.float32, "argmax: logits")
-        out = torch.empty((logits.shape[0],), dtype=torch.int32, device=logits.device)
-        kernels._ok(self._lib.xi_argmax(kernels._p(logits), logits.shape[0], logits.shape[1],
-                                        kernels._p(out), kernels._stream()))
+        if logits.dim() != 2:
+            raise kernels.KernelError("argmax: logits must be [rows, vocab]")
+        rows, V = logits.shape
+        out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+        chunks = int(self._lib.xi_argmax_chunks(V))
+        pval = pidx = None
+        if chunks > 1:
+            pval = torch.empty((rows, chunks), dtype=torch.float32, device=logits.device)
+            pidx = torch.empty((rows, chunks), dtype=torch.int32, device=logits.device)
+        kernels._ok(self._lib.xi_argmax(kernels._p(logits), rows, V, kernels._p(out), kernels._p(pval),
+                                        kernels._p(pidx), kernels._stream()))
         return out
 
     def sample(self, logits: torch.Tensor, strategies: Sequence[Strategy], uniforms: Sequence[float],
