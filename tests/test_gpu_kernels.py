@@ -117,29 +117,59 @@ def test_linear_bf16(M, N, K):
 @pytest.mark.parametrize("N,K", [(509, 96), (77, 136), (1536, 4096), (4096, 1408), (16, 8)])
 def test_linear_skinny(M, N, K, out_dtype):
     """The streaming matrix-core product for few rows: widths that are no multiple of the 16-row
-    tile or the 32-wide k step, every tile shape it can choose, and a row alone bit-equal to the
-    same row inside a batch."""
+    tile or the 32-wide k step, and every tile shape.  The order of the float32 sums is fixed by
+    the number of waves alone: with the same waves, any number of row tiles and a row alone
+    give bit-equal results."""
     from xinfer_amd import kernels
     g = torch.Generator().manual_seed(7)
     x = _rand((M, K), torch.bfloat16, g)
     w = _rand((N, K), torch.bfloat16, g, 0.05)
     ref = x.double() @ w.double().T
     tol = 2.0 ** -8 if out_dtype == torch.bfloat16 else 1e-5
-    outs = []
-    for variant in (0, 1, 2, 3, 4):
-        y = kernels.linear_skinny(x.to(DEV), w.to(DEV), out_dtype, variant=variant)
+    xd, wd = x.to(DEV), w.to(DEV)
+    outs = {}
+    for rt, nw in [(0, 0), (1, 8), (2, 8), (4, 8), (1, 16), (2, 16)]:
+        y = kernels.linear_skinny(xd, wd, out_dtype, row_tiles=rt, waves=nw)
         assert y.dtype == out_dtype and y.shape == (M, N)
         err = (y.cpu().double() - ref).abs().max() / ref.abs().max()
-        assert err < tol, (variant, err)
-        outs.append(y.cpu())
-    # with the same split of K over waves (variant 4: eight waves) a row alone is bit-equal to
-    # the same row inside the batch; the default choice may split K differently for few rows,
-    # which changes the order of the float32 sums and nothing else
+        assert err < tol, (rt, nw, err)
+        outs[(rt, nw)] = y.cpu()
+    assert torch.equal(outs[(1, 8)], outs[(2, 8)]) and torch.equal(outs[(1, 8)], outs[(4, 8)])
+    assert torch.equal(outs[(1, 16)], outs[(2, 16)])
     r = M // 2
-    y1 = kernels.linear_skinny(x[r:r + 1].contiguous().to(DEV), w.to(DEV), out_dtype, variant=4)
-    assert torch.equal(y1.cpu()[0], outs[4][r])
-    y0 = kernels.linear_skinny(x[r:r + 1].contiguous().to(DEV), w.to(DEV), out_dtype)
-    assert float((y0.cpu()[0].double() - ref[r]).abs().max() / ref.abs().max()) < tol
+    for nw in (8, 16):
+        y1 = kernels.linear_skinny(x[r:r + 1].contiguous().to(DEV), wd, out_dtype, waves=nw)
+        assert torch.equal(y1.cpu()[0], outs[(1, nw)][r])
+    # the default choice of waves comes from (N, K) alone: a row alone equals the row in the batch
+    y0 = kernels.linear_skinny(x[r:r + 1].contiguous().to(DEV), wd, out_dtype)
+    assert torch.equal(y0.cpu()[0], outs[(0, 0)][r])
+
+
+@pytest.mark.parametrize("M", [1, 8, 40])
+@pytest.mark.parametrize("N,K", [(4096, 4096), (320, 2048), (1000, 1544), (4096, 12288)])
+def test_linear_skinny_partial_sums(M, N, K):
+    """Narrow outputs may come back as float32 partial sums over slices of K; their sum is the
+    product, the fused add + RMSNorm adds them in order, and a row's parts do not depend on the
+    rows beside it."""
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(9)
+    x = _rand((M, K), torch.bfloat16, g)
+    w = _rand((N, K), torch.bfloat16, g, 0.05)
+    ref = x.double() @ w.double().T
+    parts = kernels.linear_skinny(x.to(DEV), w.to(DEV), allow_split=True)
+    assert parts.dtype == torch.float32 and parts.dim() == 3 and parts.shape[1:] == (M, N) and parts.shape[0] > 1
+    err = (parts.cpu().double().sum(0) - ref).abs().max() / ref.abs().max()
+    assert err < 1e-5, err
+    one = kernels.linear_skinny(x[M // 2:M // 2 + 1].contiguous().to(DEV), w.to(DEV), allow_split=True)
+    assert torch.equal(one.cpu()[:, 0], parts.cpu()[:, M // 2])
+    resid = _rand((M, N), torch.float32, g, 2.0)
+    wn = 1 + 0.1 * torch.randn(N, generator=g)
+    r_dev = resid.to(DEV)
+    out = kernels.add_rmsnorm(r_dev, parts, wn.to(DEV), 1e-6, torch.bfloat16)
+    s = resid.double() + ref
+    want = plain.rms_norm(s, wn.double(), 1e-6)
+    assert (out.cpu().double() - want).abs().max() / want.abs().max() < 2.0 ** -8
+    assert (r_dev.cpu().double() - s).abs().max() / s.abs().max() < 1e-5
 
 
 @pytest.mark.parametrize("M", [1, 8, 20, 64])
@@ -167,6 +197,8 @@ def test_linear_skinny_refuses():
         kernels.linear_skinny(x[:4, :60].contiguous(), w[:, :60].contiguous())
     with pytest.raises(kernels.KernelError, match="bfloat16"):
         kernels.linear_skinny(x[:4].float(), w.float())
+    with pytest.raises(kernels.KernelError, match="LDS"):
+        kernels.linear_skinny(x[:4].contiguous(), w, row_tiles=4, waves=16)
 
 
 def _rope_ref(x, pos, cos, sin, rot, interleaved):

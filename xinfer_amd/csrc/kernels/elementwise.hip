@@ -36,8 +36,9 @@ __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict_
 //   out[r] = s * rsqrt(mean(s^2) + eps) * w, rounded once to the output type.
 // The residual stream is float32 in both precisions.
 // ---------------------------------------------------------------------------------
+// y may hold `parts` partial sums [parts, T, H] (part stride T*H elements), added in order.
 template <typename TY, typename TO, int NT>
-__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TY* __restrict__ y,
+__global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TY* __restrict__ y, int parts, size_t part_stride,
                                    const float* __restrict__ w, float eps, TO* __restrict__ out,
                                    const int* __restrict__ rows, int H) {
   __shared__ float scratch[NT / kWave];
@@ -51,7 +52,8 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TY* __restri
   // a narrower TO, so the sum is recomputed in the second pass from the same operands).
   for (int i = threadIdx.x; i < H; i += NT) {
     float s = x[i];
-    if (yr) s += to_float(yr[i]);
+    if (yr)
+      for (int p = 0; p < parts; ++p) s += to_float(yr[p * part_stride + i]);
     ss += s * s;
   }
   const float total = block_sum<NT / kWave>(ss, scratch);
@@ -59,7 +61,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ resid, const TY* __restri
   for (int i = threadIdx.x; i < H; i += NT) {
     float s = x[i];
     if (yr) {
-      s += to_float(yr[i]);
+      for (int p = 0; p < parts; ++p) s += to_float(yr[p * part_stride + i]);
       if (!rows) x[i] = s;
     }
     o[i] = from_float<TO>(s * inv * w[i]);
@@ -87,6 +89,7 @@ __device__ __forceinline__ void store4(bf16* p, float4 v) {
 
 template <typename TY, typename TO, int NT, int MAXV>
 __global__ __launch_bounds__(NT) void add_rmsnorm_vec_kernel(float* __restrict__ resid, const TY* __restrict__ y,
+                                                             int parts, size_t part_stride,
                                                              const float* __restrict__ w, float eps,
                                                              TO* __restrict__ out, const int* __restrict__ rows,
                                                              int H) {
@@ -105,11 +108,13 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_vec_kernel(float* __restrict__
       s[v] = load4(x + 4 * i);
       wv[v] = load4(w + 4 * i);
       if (yr) {
-        const float4 yy = load4(yr + 4 * i);
-        s[v].x += yy.x;
-        s[v].y += yy.y;
-        s[v].z += yy.z;
-        s[v].w += yy.w;
+        for (int p = 0; p < parts; ++p) {
+          const float4 yy = load4(yr + p * part_stride + 4 * i);
+          s[v].x += yy.x;
+          s[v].y += yy.y;
+          s[v].z += yy.z;
+          s[v].w += yy.w;
+        }
       }
     } else {
       s[v] = float4{0.f, 0.f, 0.f, 0.f};
@@ -440,20 +445,24 @@ int xi_embed(const void* table, int dtype, const int* ids, float* out, int n_tok
 }
 
 // y may be null (no add).  rows may be null (all n_rows rows in place).
-int xi_add_rmsnorm(float* resid, const void* y, int y_dtype, const float* w, float eps, void* out,
-                   int out_dtype, const int* rows, int n_rows, int H, hipStream_t stream) {
+// y: null, [T, H], or `parts` partial sums [parts, T, H] (T = resid_rows), added in order.
+int xi_add_rmsnorm(float* resid, const void* y, int y_dtype, int parts, int resid_rows, const float* w, float eps,
+                   void* out, int out_dtype, const int* rows, int n_rows, int H, hipStream_t stream) {
   XI_CHECK(n_rows >= 0 && H > 0, "add_rmsnorm: bad sizes rows=%d H=%d", n_rows, H);
+  XI_CHECK(parts >= 1 && resid_rows >= 0, "add_rmsnorm: bad partial sums (%d parts of %d rows)", parts, resid_rows);
+  const size_t part_stride = (size_t)resid_rows * H;
   if (n_rows == 0) return 0;
   constexpr int NT = 256, MAXV = 8;
   const bool vec = H % 4 == 0 && H <= 4 * NT * MAXV && ((uintptr_t)resid | (uintptr_t)y | (uintptr_t)w | (uintptr_t)out) % 16 == 0;
 #define XI_NORM(TY, TO)                                                                            \
   do {                                                                                             \
     if (vec)                                                                                       \
-      add_rmsnorm_vec_kernel<TY, TO, NT, MAXV><<<n_rows, NT, 0, stream>>>(resid, (const TY*)y, w, eps, \
-                                                                          (TO*)out, rows, H);      \
+      add_rmsnorm_vec_kernel<TY, TO, NT, MAXV><<<n_rows, NT, 0, stream>>>(                         \
+          resid, (const TY*)y, parts, part_stride, w, eps, (TO*)out, rows, H);                     \
     else                                                                                           \
-      add_rmsnorm_kernel<TY, TO, NT><<<n_rows, NT, 0, stream>>>(resid, (const TY*)y, w, eps,       \
-                                                                (TO*)out, rows, H);                \
+      add_rmsnorm_kernel<TY, TO, NT><<<n_rows, NT, 0, stream>>>(resid, (const TY*)y, parts,        \
+                                                                part_stride, w, eps, (TO*)out,     \
+                                                                rows, H);                          \
   } while (0)
   if (y_dtype == kF32 && out_dtype == kF32) XI_NORM(float, float);
   else if (y_dtype == kBF16 && out_dtype == kBF16) XI_NORM(bf16, bf16);

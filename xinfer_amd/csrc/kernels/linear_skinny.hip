@@ -1,12 +1,18 @@
-// y[M,N] = x[M,K] @ w[N,K]^T in bfloat16 for few rows (decode batches): bound by the one
-// pass over w, so the kernel is a streaming read of w through the matrix cores.
+// y[M,N] = x[M,K] @ w[N,K]^T in bfloat16 for few rows (decode batches, M <= 64): bound by
+// the one pass over w, so the kernel is a streaming read of w through the matrix cores.
 //
-// One workgroup owns 16*RT rows of w (output features) over all of K; its NW waves take
-// consecutive K ranges and merge through LDS in wave order, so an output element's value
-// depends on (K, NW) alone, never on M or on what else is in the batch.  Per 32-wide k
-// step a wave issues v_mfma_f32_16x16x32_bf16 with A = 16 rows of w (lane l: row l%16,
-// k group l/16, one 16-byte load) and B = x^T (lane l: token l%16, same k group), for
-// MT tiles of 16 tokens.  x is small (M <= 64 rows) and is read from L2 by every wave.
+// A workgroup owns 16*RT rows of w (output features) and one of KS slices of K.  Its NW
+// waves take consecutive parts of the slice and merge through LDS in a fixed order, so an
+// output element's value depends on (K, KS, NW) alone, never on M, on RT or on what else is
+// in the batch.  Per 32-wide k step a wave issues v_mfma_f32_16x16x32_bf16 with A = 16 rows
+// of w (lane l: row l%16, k group l/16, one 16-byte load) and B = x^T (lane l: token l%16,
+// same k group), for RT row tiles and MT tiles of 16 tokens: every x operand is used RT
+// times and every w operand MT times.  x is small and is read from L2.
+//
+// With KS > 1 the workgroups of different slices write float32 partial sums [KS, M, N]; the
+// consumer (the fused add + RMSNorm) adds them in slice order.  That gives narrow outputs
+// (N = hidden size) enough workgroups for every compute unit and still lets a workgroup
+// keep several row tiles per x operand.
 //
 // GATED: w is [2N, K] = [gate; up]; the workgroup computes rows n (gate) and N + n (up)
 // and stores silu(gate) * up, float32 math and one rounding, so the packed [M, 2N]
@@ -15,6 +21,7 @@
 // Reference call sites: candle matmul in /root/reference/src/models/layers/linear.rs:76-124
 // (vendor BLAS); fused gate/up + silu_and_mul in /root/reference/src/models/layers/mlp.rs:613-633.
 #include "common.h"
+#include <type_traits>
 
 namespace xi {
 
@@ -29,23 +36,36 @@ __device__ __forceinline__ bf16x8 zeros8() {
   return z;
 }
 
+// Row of w that tile t of the workgroup at n0 reads.  Plain: tiles are consecutive blocks of
+// 16 rows.  Gated: tiles 0..RT/2-1 are gate rows, tiles RT/2..RT-1 the matching up rows.
+template <int RT, bool GATED>
+__device__ __forceinline__ int tile_row0(int t, int n0, int N) {
+  if (!GATED) return n0 + 16 * t;
+  return t < RT / 2 ? n0 + 16 * t : N + n0 + 16 * (t - RT / 2);
+}
+
 template <int MT, int RT, int NW, int U, bool GATED, typename TO>
 __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16* __restrict__ x,
                                                                 const bf16* __restrict__ w,
-                                                                TO* __restrict__ y, int M, int N, int K) {
-  static_assert(!GATED || RT == 2, "the gated form pairs one gate tile with one up tile");
-  __shared__ float red[NW * RT * MT * 256];
+                                                                TO* __restrict__ y, int M, int N, int K,
+                                                                int steps_per_slice) {
+  static_assert(!GATED || RT % 2 == 0, "the gated form pairs gate tiles with up tiles");
+  static_assert((NW / 2) * RT * MT <= 64, "the merge buffer must fit in 64 KB of LDS");
+  __shared__ float red[(NW / 2) * RT * MT * 256];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, j = lane >> 4;
-  const int n0 = blockIdx.x * (GATED ? 16 : 16 * RT);
+  const int n0 = blockIdx.x * (GATED ? 16 * (RT / 2) : 16 * RT);
+  const int ks = blockIdx.y;
+  const int w_rows = GATED ? 2 * N : N;
 
   // rows of w and x this lane loads; rows past the end are clamped (their results are dropped)
   const bf16* wp[RT];
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
-    int row = GATED ? (t == 0 ? n0 + r : N + n0 + r) : n0 + 16 * t + r;
-    const int last = GATED ? (t == 0 ? N - 1 : 2 * N - 1) : N - 1;
+    int row = tile_row0<RT, GATED>(t, n0, N) + r;
+    const int last = GATED ? (t < RT / 2 ? N - 1 : 2 * N - 1) : N - 1;
     if (row > last) row = last;
+    if (row > w_rows - 1) row = w_rows - 1;
     wp[t] = w + (size_t)row * K + 8 * j;
   }
   const bf16* xp[MT];
@@ -64,27 +84,39 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16* __re
 
   const int steps = (K + 31) / 32;      // k steps of 32
   const int steps_full = K / 32;        // steps in which every lane's 8 elements exist
-  const int per = (steps + NW - 1) / NW;
-  const int s0 = wave * per;
-  const int s1 = min(steps, s0 + per);
+  const int slice0 = ks * steps_per_slice;
+  const int slice1 = min(steps, slice0 + steps_per_slice);
+  const int per = (steps_per_slice + NW - 1) / NW;
+  const int s0 = slice0 + wave * per;
+  const int s1 = min(slice1, s0 + per);
   const int s_fast = min(s1, steps_full);
   int s = s0;
-  for (; s + U <= s_fast; s += U) {
-    bf16x8 a[RT][U], b[MT][U];
+  // UU steps at once: all their loads are issued before the first product
+  auto block = [&](auto uu_tag) {
+    constexpr int UU = decltype(uu_tag)::value;
+    bf16x8 a[RT][UU], b[MT][UU];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
+    for (int u = 0; u < UU; ++u) {
 #pragma unroll
       for (int t = 0; t < RT; ++t) a[t][u] = ldg8(wp[t] + 32 * (s + u));
 #pragma unroll
       for (int m = 0; m < MT; ++m) b[m][u] = ldg8(xp[m] + 32 * (s + u));
     }
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+    for (int u = 0; u < UU; ++u)
 #pragma unroll
       for (int t = 0; t < RT; ++t)
 #pragma unroll
         for (int m = 0; m < MT; ++m)
           acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], b[m][u], acc[t][m], 0, 0, 0);
+    s += UU;
+  };
+  while (s + U <= s_fast) block(std::integral_constant<int, U>{});
+  if constexpr (U >= 8) {
+    if (s + 4 <= s_fast) block(std::integral_constant<int, 4>{});
+  }
+  if constexpr (U >= 4) {
+    if (s + 2 <= s_fast) block(std::integral_constant<int, 2>{});
   }
   for (; s < s1; ++s) {  // the rest, one step at a time; K % 8 == 0 so a lane's chunk exists or not
     const bool ok = 32 * s + 8 * j < K;
@@ -99,45 +131,106 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16* __re
     }
   }
 
-  // lane holds token r, features 4j..4j+3 of each tile
+  // merge the waves in a fixed order: wave w + NW/2 hands its sums to wave w, then all threads
+  // add the NW/2 sums that are left, in wave order, and store.  A lane's 4 values of a tile:
+  // token r, features 4j..4j+3.
+  constexpr int H = NW / 2;
+  if (wave >= H) {
 #pragma unroll
-  for (int t = 0; t < RT; ++t)
+    for (int t = 0; t < RT; ++t)
 #pragma unroll
-    for (int m = 0; m < MT; ++m)
-      *reinterpret_cast<f32x4*>(&red[((wave * RT + t) * MT + m) * 256 + r * 16 + 4 * j]) = acc[t][m];
+      for (int m = 0; m < MT; ++m)
+        *reinterpret_cast<f32x4*>(&red[(((wave - H) * RT + t) * MT + m) * 256 + lane * 4]) = acc[t][m];
+  }
+  __syncthreads();
+  if (wave < H) {
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        f32x4* slot = reinterpret_cast<f32x4*>(&red[((wave * RT + t) * MT + m) * 256 + lane * 4]);
+        const f32x4 o = *slot;
+        f32x4 sum = acc[t][m];
+        sum[0] += o[0];
+        sum[1] += o[1];
+        sum[2] += o[2];
+        sum[3] += o[3];
+        *slot = sum;      // the same lane wrote and reads this slot: no barrier in between
+      }
+  }
   __syncthreads();
 
-  if (GATED) {
-    for (int idx = threadIdx.x; idx < MT * 256; idx += NW * 64) {
-      const int m = idx >> 8, tok = (idx >> 4) & 15, f = idx & 15;
-      float g = 0.f, u = 0.f;
+  TO* yk = y + (size_t)ks * M * N;   // this slice's partial sums (ks is 0 without slices)
+  constexpr int PAIRS = GATED ? RT / 2 : RT;
+  for (int idx = threadIdx.x; idx < PAIRS * MT * 256; idx += NW * 64) {
+    const int tile = idx >> 8, e = idx & 255;
+    const int p = tile / MT, m = tile - p * MT;
+    const int ln = e >> 2, v = e & 3;
+    const int token = 16 * m + (ln & 15), n = n0 + 16 * p + 4 * (ln >> 4) + v;
+    float a0 = 0.f, a1 = 0.f;
 #pragma unroll
-      for (int wv = 0; wv < NW; ++wv) {
-        g += red[((wv * RT + 0) * MT + m) * 256 + tok * 16 + f];
-        u += red[((wv * RT + 1) * MT + m) * 256 + tok * 16 + f];
-      }
-      const int token = 16 * m + tok, n = n0 + f;
-      if (token < M && n < N) y[(size_t)token * N + n] = from_float<TO>(g / (1.f + __expf(-g)) * u);
+    for (int wv = 0; wv < H; ++wv) {
+      a0 += red[((wv * RT + p) * MT + m) * 256 + e];
+      if (GATED) a1 += red[((wv * RT + RT / 2 + p) * MT + m) * 256 + e];
     }
-  } else {
-    for (int idx = threadIdx.x; idx < RT * MT * 256; idx += NW * 64) {
-      const int t = idx / (MT * 256), rem = idx - t * (MT * 256);
-      const int m = rem >> 8, tok = (rem >> 4) & 15, f = rem & 15;
-      float sum = 0.f;
-#pragma unroll
-      for (int wv = 0; wv < NW; ++wv) sum += red[((wv * RT + t) * MT + m) * 256 + tok * 16 + f];
-      const int token = 16 * m + tok, n = n0 + 16 * t + f;
-      if (token < M && n < N) y[(size_t)token * N + n] = from_float<TO>(sum);
-    }
+    if (token < M && n < N)
+      yk[(size_t)token * N + n] = from_float<TO>(GATED ? a0 / (1.f + __expf(-a0)) * a1 : a0);
   }
 }
 
-template <int MT, int RT, int NW, int U, bool GATED, typename TO>
-static void launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, hipStream_t stream) {
-  const int rows_per_wg = GATED ? 16 : 16 * RT;
-  const unsigned grid = (unsigned)((N + rows_per_wg - 1) / rows_per_wg);
+struct SkinnyPlan {
+  int ks;    // slices of K across workgroups
+  int nw;    // waves per workgroup
+  int rt;    // row tiles per workgroup
+};
+
+// ks and nw fix the order of the sums: they come from (N, K) and the caller's wish alone.
+// rt only says which workgroup computes what; it grows with M (reuse of the x operands) as
+// long as enough workgroups remain.
+static SkinnyPlan plan_skinny(int M, int N, int K, bool gated, bool allow_split) {
+  SkinnyPlan p;
+  const int tiles = (N + 15) / 16;
+  p.ks = 1;
+  if (allow_split && !gated) {
+    p.ks = (1024 + tiles - 1) / tiles;
+    if (p.ks > 4) p.ks = 4;
+    while (p.ks > 1 && K / p.ks < 512) --p.ks;
+  }
+  p.nw = (gated || tiles * p.ks >= 1024) ? 8 : 16;
+  const int mt = (M + 15) / 16;
+  if (gated) {
+    p.rt = (mt >= 2 && tiles / 2 >= 256) ? 4 : 2;
+  } else {
+    int rt_max = M <= 4 ? 1 : (mt == 1 ? 2 : 4);
+    if (p.nw == 16 && rt_max > 2) rt_max = 2;
+    const int enough = mt >= 3 ? 256 : 512;      // workgroups that still fill the chip
+    p.rt = 1;
+    for (int rt = rt_max; rt > 1; rt >>= 1)
+      if ((tiles + rt - 1) / rt * p.ks >= enough) {
+        p.rt = rt;
+        break;
+      }
+  }
+  return p;
+}
+
+template <int MT, int RT, int NW, bool GATED, typename TO>
+static void launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, int ks, hipStream_t stream) {
+  constexpr int U = (RT + MT <= 2) ? 8 : (RT + MT <= 4 ? 4 : 2);
+  const int rows_per_wg = GATED ? 16 * (RT / 2) : 16 * RT;
+  const int steps = (K + 31) / 32;
+  const int sps = (steps + ks - 1) / ks;
+  dim3 grid((unsigned)((N + rows_per_wg - 1) / rows_per_wg), (unsigned)ks);
   linear_skinny_kernel<MT, RT, NW, U, GATED, TO><<<grid, NW * 64, 0, stream>>>(
-      (const bf16*)x, (const bf16*)w, (TO*)y, M, N, K);
+      (const bf16*)x, (const bf16*)w, (TO*)y, M, N, K, sps);
+}
+
+template <int RT, int NW, bool GATED, typename TO>
+static void launch_skinny_mt(int mt, const void* x, const void* w, void* y, int M, int N, int K, int ks,
+                             hipStream_t stream) {
+  if (mt == 1) launch_skinny<1, RT, NW, GATED, TO>(x, w, y, M, N, K, ks, stream);
+  else if (mt == 2) launch_skinny<2, RT, NW, GATED, TO>(x, w, y, M, N, K, ks, stream);
+  else launch_skinny<4, RT, NW, GATED, TO>(x, w, y, M, N, K, ks, stream);   // 33..64 rows
 }
 
 }  // namespace xi
@@ -149,64 +242,55 @@ extern "C" {
 // Most rows of x the skinny kernels take.
 int xi_linear_skinny_max_rows() { return 64; }
 
-// x [M, K] bf16, w [N, K] bf16 -> y [M, N] in out_dtype (bf16 or float32).
-// gated != 0: w is [2N, K] and y [M, N] = silu(x @ w[:N]^T) * (x @ w[N:]^T).
-// variant: 0 = chosen from the sizes; other values select a tile shape (for measurements).
+// The number of K slices xi_linear_skinny will use for these sizes (the leading dimension of
+// its output when greater than 1).
+int xi_linear_skinny_slices(int N, int K, int gated, int allow_split) {
+  return plan_skinny(1, N, K, gated != 0, allow_split != 0).ks;
+}
+
+// x [M, K] bf16, w [N, K] bf16 -> y [M, N] in out_dtype (bf16 or float32); with
+// allow_split and xi_linear_skinny_slices(...) = KS > 1, y is float32 [KS, M, N] partial sums.
+// gated != 0: w is [2N, K] and y [M, N] = silu(x @ w[:N]^T) * (x @ w[N:]^T), bfloat16.
+// force_rt / force_nw: 0 = chosen from the sizes; other values select a shape (for measurements
+// and tests; nw * rt must not exceed 32).
 int xi_linear_skinny(const void* x, const void* w, void* y, int M, int N, int K, int out_dtype, int gated,
-                     int variant, hipStream_t stream) {
+                     int allow_split, int force_rt, int force_nw, hipStream_t stream) {
   XI_CHECK(M >= 0 && N > 0 && K > 0, "linear_skinny: bad sizes M=%d N=%d K=%d", M, N, K);
   XI_CHECK(M <= 64, "linear_skinny: %d rows exceed 64 (use the library product)", M);
   XI_CHECK(K % 8 == 0, "linear_skinny: K=%d must be a multiple of 8", K);
   XI_CHECK(out_dtype == kBF16 || out_dtype == kF32, "linear_skinny: unknown output dtype %d", out_dtype);
   if (M == 0) return 0;
+  SkinnyPlan p = plan_skinny(M, N, K, gated != 0, allow_split != 0);
+  XI_CHECK(p.ks == 1 || out_dtype == kF32, "linear_skinny: partial sums of %d slices must be float32", p.ks);
+  XI_CHECK(!gated || out_dtype == kBF16, "linear_skinny: the gated form writes bfloat16");
+  if (force_nw) p.nw = force_nw;
+  if (force_rt) p.rt = force_rt;
+  XI_CHECK(p.nw == 8 || p.nw == 16, "linear_skinny: %d waves (8 or 16)", p.nw);
+  XI_CHECK(gated ? (p.rt == 2 || p.rt == 4) : (p.rt == 1 || p.rt == 2 || p.rt == 4), "linear_skinny: %d row tiles", p.rt);
+  XI_CHECK(p.nw * p.rt <= 32, "linear_skinny: %d waves of %d row tiles do not fit in LDS", p.nw, p.rt);
   const int mt = (M + 15) / 16;
-  const int tiles = (N + 15) / 16;  // 16-row tiles of the output
-  // Wide outputs keep two row tiles per workgroup (x operands are reused); narrow ones one
-  // tile and sixteen waves so that every compute unit still has work.  The number of waves
-  // fixes the order of the float32 sums, so it is chosen from N alone and a row's result
-  // does not depend on how many rows came with it (the gated form with more than 32 rows
-  // is the exception: sixteen waves of two tiles do not fit in LDS there).
-  int rt = (variant == 1) ? 1 : (variant == 2) ? 2 : (tiles >= 2048 ? 2 : 1);
-  if (gated) rt = 2;
-  int nw = (variant == 3) ? 16 : (variant == 4) ? 8 : ((gated ? tiles : tiles / rt) < 512 ? 16 : 8);
-  if (nw == 16 && rt * mt > 4) {
-    if (rt == 2 && !gated && variant != 2) rt = 1;
-    else nw = 8;
-  }
-#define XI_SK(MT, RT, NW, U, G, TO) launch_skinny<MT, RT, NW, U, G, TO>(x, w, y, M, N, K, stream)
-#define XI_SK_TO(MT, RT, NW, U, G)                         \
-  do {                                                     \
-    if (out_dtype == kBF16) XI_SK(MT, RT, NW, U, G, bf16); \
-    else XI_SK(MT, RT, NW, U, G, float);                   \
+#define XI_SK_PLAIN(RT, NW)                                                       \
+  do {                                                                            \
+    if (out_dtype == kBF16)                                                       \
+      launch_skinny_mt<RT, NW, false, bf16>(mt, x, w, y, M, N, K, p.ks, stream);  \
+    else                                                                          \
+      launch_skinny_mt<RT, NW, false, float>(mt, x, w, y, M, N, K, p.ks, stream); \
   } while (0)
-#define XI_SK_MT(RT, NW, G)                                   \
-  do {                                                        \
-    if (mt == 1) XI_SK_TO(1, RT, NW, (RT == 1 ? 8 : 4), G);   \
-    else if (mt == 2) XI_SK_TO(2, RT, NW, 4, G);              \
-    else if (mt == 3) XI_SK_TO(3, RT, NW, (RT == 1 ? 4 : 2), G); \
-    else XI_SK_TO(4, RT, NW, (RT == 1 ? 4 : 2), G);           \
-  } while (0)
+#define XI_SK_GATED(RT, NW) launch_skinny_mt<RT, NW, true, bf16>(mt, x, w, y, M, N, K, p.ks, stream)
   if (gated) {
-    if (nw == 16) {
-      if (mt == 1) XI_SK_TO(1, 2, 16, 4, true);
-      else XI_SK_TO(2, 2, 16, 4, true);
-    } else {
-      XI_SK_MT(2, 8, true);
-    }
-  } else if (rt == 2) {
-    if (nw == 16) {
-      if (mt == 1) XI_SK_TO(1, 2, 16, 4, false);
-      else XI_SK_TO(2, 2, 16, 4, false);
-    } else {
-      XI_SK_MT(2, 8, false);
-    }
+    if (p.nw == 16) XI_SK_GATED(2, 16);
+    else if (p.rt == 2) XI_SK_GATED(2, 8);
+    else XI_SK_GATED(4, 8);
+  } else if (p.nw == 16) {
+    if (p.rt == 1) XI_SK_PLAIN(1, 16);
+    else XI_SK_PLAIN(2, 16);
   } else {
-    if (nw == 16) XI_SK_MT(1, 16, false);
-    else XI_SK_MT(1, 8, false);
+    if (p.rt == 1) XI_SK_PLAIN(1, 8);
+    else if (p.rt == 2) XI_SK_PLAIN(2, 8);
+    else XI_SK_PLAIN(4, 8);
   }
-#undef XI_SK_MT
-#undef XI_SK_TO
-#undef XI_SK
+#undef XI_SK_PLAIN
+#undef XI_SK_GATED
   XI_LAUNCH_CHECK("linear_skinny");
   return 0;
 }

@@ -96,13 +96,19 @@ def add_rmsnorm(resid: torch.Tensor, y: Optional[torch.Tensor], weight: torch.Te
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """s = resid (+ y); out = rms(s) * weight in `out_dtype`.  Without `rows` every row is
     normed and the sum is written back into resid; with `rows` (int32 indices) only those
-    rows are produced and resid is left alone."""
+    rows are produced and resid is left alone.  y may be a stack [P, T, H] of float32 partial
+    sums, which are added in order."""
     _dev(resid, y, weight, rows, out)
     _want(resid, torch.float32, "add_rmsnorm: residual stream")
     _want(weight, torch.float32, "add_rmsnorm: weight")
     if resid.dim() != 2 or weight.shape != (resid.shape[1],):
         raise KernelError(f"add_rmsnorm: resid {tuple(resid.shape)} and weight {tuple(weight.shape)} do not match")
-    if y is not None and y.shape != resid.shape:
+    parts = 1
+    if y is not None and y.dim() == 3:
+        if y.dtype != torch.float32 or tuple(y.shape[1:]) != tuple(resid.shape):
+            raise KernelError(f"add_rmsnorm: partial sums {tuple(y.shape)} {y.dtype} must be float32 [P, T, H]")
+        parts = int(y.shape[0])
+    elif y is not None and y.shape != resid.shape:
         raise KernelError(f"add_rmsnorm: y {tuple(y.shape)} differs from resid {tuple(resid.shape)}")
     H = resid.shape[1]
     if rows is not None:
@@ -114,9 +120,9 @@ def add_rmsnorm(resid: torch.Tensor, y: Optional[torch.Tensor], weight: torch.Te
         out = torch.empty((n, H), dtype=out_dtype, device=resid.device)
     elif out.shape != (n, H) or out.dtype != out_dtype:
         raise KernelError("add_rmsnorm: out has the wrong shape or dtype")
-    _ok(lib().xi_add_rmsnorm(_p(resid), _p(y), _code(y, "add_rmsnorm") if y is not None else F32,
-                             _p(weight), ctypes.c_float(eps), _p(out), _code(out, "add_rmsnorm"),
-                             _p(rows), n, H, _stream()))
+    _ok(lib().xi_add_rmsnorm(_p(resid), _p(y), _code(y, "add_rmsnorm") if y is not None else F32, parts,
+                             int(resid.shape[0]), _p(weight), ctypes.c_float(eps), _p(out),
+                             _code(out, "add_rmsnorm"), _p(rows), n, H, _stream()))
     return out
 
 
@@ -345,9 +351,13 @@ SKINNY_GATED_ROWS = 16    # the same for the fused gate/up/silu form, which also
 
 
 def linear_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
-                  gated: bool = False, out: Optional[torch.Tensor] = None, variant: int = 0) -> torch.Tensor:
+                  gated: bool = False, out: Optional[torch.Tensor] = None, allow_split: bool = False,
+                  row_tiles: int = 0, waves: int = 0) -> torch.Tensor:
     """bfloat16 x [M, K] @ w [N, K]^T for M <= 64 rows with the streaming matrix-core kernel.
-    `gated`: w is [2N, K] = [gate; up] and the result is silu(x @ gate^T) * (x @ up^T), [M, N]."""
+    `gated`: w is [2N, K] = [gate; up] and the result is silu(x @ gate^T) * (x @ up^T), [M, N].
+    `allow_split`: for narrow outputs the kernel may cut K into slices across workgroups and
+    return float32 partial sums [slices, M, N] for the consumer to add in order (the fused
+    add + RMSNorm does).  `row_tiles`, `waves`: 0 = chosen from the sizes."""
     _dev(x, w, out)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError("linear_skinny: operands must be bfloat16")
@@ -361,18 +371,22 @@ def linear_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dt
         N //= 2
     if M > SKINNY_MAX_ROWS or K % 8:
         raise KernelError(f"linear_skinny: M={M} must be <= {SKINNY_MAX_ROWS} and K={K} a multiple of 8")
-    out_dtype = out_dtype or torch.bfloat16
+    slices = int(lib().xi_linear_skinny_slices(N, K, int(bool(gated)), int(bool(allow_split))))
+    if slices > 1:
+        out_dtype, shape = torch.float32, (slices, M, N)
+    else:
+        out_dtype, shape = out_dtype or torch.bfloat16, (M, N)
     if out is None:
-        out = torch.empty((M, N), dtype=out_dtype, device=x.device)
-    elif out.shape != (M, N) or out.dtype != out_dtype:
+        out = torch.empty(shape, dtype=out_dtype, device=x.device)
+    elif tuple(out.shape) != shape or out.dtype != out_dtype:
         raise KernelError("linear_skinny: out has the wrong shape or dtype")
     _ok(lib().xi_linear_skinny(_p(x), _p(w), _p(out), M, N, K, _code(out, "linear_skinny"), int(bool(gated)),
-                               int(variant), _stream()))
+                               int(bool(allow_split)), int(row_tiles), int(waves), _stream()))
     return out
 
 
 def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
-                skinny_rows: int = SKINNY_ROWS) -> torch.Tensor:
+                skinny_rows: int = SKINNY_ROWS, allow_split: bool = False) -> torch.Tensor:
     """bfloat16 x @ w.T with float32 accumulation, rounded once to `out_dtype` (bfloat16 or
     float32).  Up to `skinny_rows` rows (decode): the hand-written streaming kernel.  More
     rows: the vendor library (hipBLASLt through torch), which the reference's engine also
@@ -382,7 +396,7 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtyp
         raise KernelError("linear_bf16: operands must be bfloat16")
     out_dtype = out_dtype or torch.bfloat16
     if 0 < x.shape[0] <= min(skinny_rows, SKINNY_MAX_ROWS) and x.shape[1] % 8 == 0:
-        return linear_skinny(x, w, out_dtype)
+        return linear_skinny(x, w, out_dtype, allow_split=allow_split)
     if out_dtype == torch.float32:
         return torch.mm(x, w.t(), out_dtype=torch.float32)
     return torch.nn.functional.linear(x, w)

@@ -4,10 +4,12 @@ A part is built from a `PartSpec` (its sizes and constants) and the activation d
 declares the tensors it needs under a name prefix, loads them from a weight store, and
 runs on the tokens of one step.  A part never learns which model it is in.
 
-  Mixer            forward(x, ctx, cache) -> y        x, y: [T, hidden]
+  Mixer            forward(x, ctx, cache) -> y        x, y: [T, hidden]; y may also be a stack
+                                                      [P, T, hidden] of float32 partial sums,
+                                                      which the next norm adds in order
                    cache_need() -> KVNeed | None      paged keys/values it wants
                    state_need() -> StateNeed | None   fixed-size per-request state it wants
-  FeedForward      forward(x, ctx) -> y
+  FeedForward      forward(x, ctx) -> y               (y as for the mixer)
   Norm             forward(resid, add, out_dtype, rows=None, out=None) -> normed
                    resid is the float32 residual stream; `add` (if given) is summed into
                    it first; with `rows` only those rows are produced and resid is not
