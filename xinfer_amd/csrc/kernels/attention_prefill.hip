@@ -46,16 +46,21 @@ __device__ __forceinline__ bf16x8 zero8p() {
   return z;
 }
 
-template <int KC, int DT, int NQT, int GH>
-__global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
+// NWV waves of NQT column tiles each: the workgroup's NWV * NQT tiles are (position block,
+// head) pairs, GH heads per position block.  Eight waves of two tiles keep a wave within
+// half of a SIMD's registers, so two waves share a SIMD and one's exponentials overlap the
+// other's matrix instructions.
+template <int KC, int DT, int NQT, int GH, int NWV>
+__global__ __launch_bounds__(64 * NWV) void attn_prefill_lds_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ vt_cache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ tiles,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, bf16* __restrict__ out, float scale_log2,
     int window, int page_shift, int nq, int nkv, int d) {
   const int page = 1 << page_shift;
-  constexpr int PB = NQT / GH;   // blocks of 16 positions per wave
-  constexpr int QW = 16 * PB;    // query positions per wave
-  constexpr int LI = KC;         // 16-byte chunks per thread and tile, for K and for V^T
+  constexpr int NT = 64 * NWV;                    // threads
+  constexpr int QB = 16 * (NWV * NQT / GH);       // query positions per workgroup
+  constexpr int LI = (256 * KC + NT - 1) / NT;    // 16-byte chunks per thread and tile, for K and for V^T
+  static_assert((NWV * NQT) % GH == 0, "tiles must divide into whole position blocks");
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr int krow = 32 * KC + kVPad;  // elements per K row in LDS: head_dim rounded up to the
                                          // 32-wide steps of the matrix product (the rest is zero)
@@ -77,19 +82,20 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
   {
     const int* bt = block_tables + (size_t)seq * max_pages;
     const int n_pages = (k_last + page) / page;    // pages that hold keys 0..k_last
-    for (int i = threadIdx.x; i < n_pages; i += 256) bt_s[i] = bt[i];
+    for (int i = threadIdx.x; i < n_pages; i += NT) bt_s[i] = bt[i];
   }
 
   // keys the workgroup walks
-  const int wg_nq = min(4 * QW, q_len - q0_blk);
+  const int wg_nq = min(QB, q_len - q0_blk);
   const int wg_first = pos0 + q0_blk, wg_last = wg_first + wg_nq - 1;
   const int wg_lo = (window > 0 && wg_first - window + 1 > 0) ? wg_first - window + 1 : 0;
   const int k_begin = wg_lo & ~(kKeys - 1);
 
-  // this wave's queries
-  const int q0 = q0_blk + wave * QW;
+  // this wave's queries: the position blocks its tiles lie in
+  const int pb_lo = (wave * NQT) / GH, pb_hi = (wave * NQT + NQT - 1) / GH;
+  const int q0 = q0_blk + 16 * pb_lo;
   const bool active = q0 < q_len;
-  const int n_q = active ? min(QW, q_len - q0) : 0;
+  const int n_q = active ? min(16 * (pb_hi - pb_lo + 1), q_len - q0) : 0;
   const int first_pos = pos0 + q0, last_pos = first_pos + n_q - 1;
   const int lo_first = (window > 0 && first_pos - window + 1 > 0) ? first_pos - window + 1 : 0;
   const int lo_last = (window > 0 && last_pos - window + 1 > 0) ? last_pos - window + 1 : 0;
@@ -101,8 +107,9 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
   int qpos[NQT], qlo[NQT];
 #pragma unroll
   for (int ct = 0; ct < NQT; ++ct) {
-    const int pb = ct / GH, hh = ct - pb * GH;
-    const int qi = q0 + 16 * pb + r;
+    const int tile = wave * NQT + ct;
+    const int pb = tile / GH, hh = tile - pb * GH;
+    const int qi = q0_blk + 16 * pb + r;
     const bool ok = active && qi < q_len;
     qpos[ct] = ok ? pos0 + qi : -1;
     qlo[ct] = (ok && window > 0 && qpos[ct] - window + 1 > 0) ? qpos[ct] - window + 1 : 0;
@@ -128,7 +135,7 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
   int c_kl[LI], c_koff[LI], c_kdst[LI], c_vdst[LI];
 #pragma unroll
   for (int i = 0; i < LI; ++i) {
-    const int idx = tid + 256 * i;
+    const int idx = tid + NT * i;
     const int kl = idx / CPK, ch = idx % CPK;
     const int k32 = kl & 31;
     c_kl[i] = kl;
@@ -141,7 +148,7 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
   auto fetch = [&](int kb) {
 #pragma unroll
     for (int i = 0; i < LI; ++i) {
-      const int idx = tid + 256 * i;
+      const int idx = tid + NT * i;
       int key = kb + c_kl[i];
       key = key > k_last ? k_last : key;
       const int kp = bt_s[key >> page_shift];
@@ -163,7 +170,7 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
     for (int i = 0; i < LI; ++i) {
       st8(Ks + c_kdst[i], c_koff[i] < 0 ? zero8p() : kreg[i]);   // zeroed here, not at the load: the
                                                                   // load stays in flight meanwhile
-      if (tid + 256 * i < n_vchunks) st8(Vs + c_vdst[i], vreg[i]);
+      if (tid + NT * i < n_vchunks) st8(Vs + c_vdst[i], vreg[i]);
     }
   };
 
@@ -268,8 +275,9 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
   for (int ct = 0; ct < NQT; ++ct) {
     float lt = l_run[ct] + __shfl_xor(l_run[ct], 16, kWave);
     lt += __shfl_xor(lt, 32, kWave);
-    const int pb = ct / GH, hh = ct - pb * GH;
-    const int qi = q0 + 16 * pb + r;
+    const int tile = wave * NQT + ct;
+    const int pb = tile / GH, hh = tile - pb * GH;
+    const int qi = q0_blk + 16 * pb + r;
     if (qi >= q_len) continue;
     const float inv = 1.f / lt;
     bf16* o = out + ((size_t)(q_begin + qi) * nq + h0 + hh) * d;
@@ -286,12 +294,11 @@ __global__ __launch_bounds__(256) void attn_prefill_lds_kernel(
   }
 }
 
-static inline int heads_per_wave(int g, int nqt) {
-  if (nqt >= 4 && g % 4 == 0) return 4;
-  if (g % 2 == 0) return 2;
-  return 1;
-}
-static inline int column_tiles(int d) { return d <= 128 ? 4 : 2; }
+// Column tiles of a workgroup by head size: eight waves of two tiles up to 128, of one tile
+// above (the accumulators of a tile take twice the registers there).
+static inline int tiles_of(int d) { return d <= 128 ? 16 : 8; }
+// Query heads of a kv head that one workgroup takes together.
+static inline int heads_together(int g) { return g % 4 == 0 ? 4 : (g % 2 == 0 ? 2 : 1); }
 
 }  // namespace xi
 
@@ -303,10 +310,7 @@ int xi_attention_mfma_supported(int nq, int nkv, int d, int page);
 
 // Query positions per workgroup for a head size and a number of query heads per kv head
 // (the host builds `tiles` in steps of it).
-int xi_attention_prefill_block(int d, int g) {
-  const int nqt = column_tiles(d);
-  return 64 * (nqt / heads_per_wave(g, nqt));
-}
+int xi_attention_prefill_block(int d, int g) { return 16 * (tiles_of(d) / heads_together(g)); }
 
 // tiles int32 [n_tiles, 2] = (sequence, first query position of the block within the
 // sequence's portion), first positions being multiples of xi_attention_prefill_block.
@@ -319,8 +323,7 @@ int xi_attention_prefill_bf16(const void* q, const void* k_cache, const void* vt
   XI_CHECK(n_tiles >= 0 && n_tiles <= 65535, "attention_prefill: %d query blocks are too many for one launch", n_tiles);
   if (n_tiles == 0) return 0;
   const int g = nq / nkv;
-  const int nqt = column_tiles(d);
-  const int gh = heads_per_wave(g, nqt);
+  const int gh = heads_together(g);
   dim3 grid(nkv * (g / gh), n_tiles);
   const float sl = scale * kLog2eP;
   XI_CHECK(sl > 0.f, "attention_prefill: the scale must be positive");
@@ -328,9 +331,9 @@ int xi_attention_prefill_bf16(const void* q, const void* k_cache, const void* vt
   for (int b = 0; b < 31; ++b)
     if ((1 << b) == page) page_shift = b;
   XI_CHECK(page_shift >= 3, "attention_prefill: the page size %d must be a power of two of at least 8", page);
-#define XI_PF(KC, DT, NQT, GH)                                                                          \
+#define XI_PF(KC, DT, NQT, GH, NWV)                                                                     \
   do {                                                                                                  \
-    auto kern = attn_prefill_lds_kernel<KC, DT, NQT, GH>;                                               \
+    auto kern = attn_prefill_lds_kernel<KC, DT, NQT, GH, NWV>;                                          \
     const size_t lds = 2 * (size_t)(kKeys * (32 * KC + kVPad) + d * (kKeys + kVPad)) * sizeof(bf16) +   \
                        (size_t)max_pages * sizeof(int);                                                 \
     XI_CHECK(lds <= 160 * 1024, "attention_prefill: block tables of %d pages do not fit in LDS", max_pages); \
@@ -340,20 +343,19 @@ int xi_attention_prefill_bf16(const void* q, const void* k_cache, const void* vt
       XI_CHECK(e == hipSuccess, "attention_prefill: cannot get %zu bytes of LDS: %s", lds,              \
                hipGetErrorString(e));                                                                   \
     }                                                                                                   \
-    kern<<<grid, 256, lds, stream>>>((const bf16*)q, (const bf16*)k_cache, (const bf16*)vt_cache,       \
-                                     block_tables, max_pages, tiles, cu_q, ctx_lens, (bf16*)out, sl,    \
-                                     window, page_shift, nq, nkv, d);                                   \
+    kern<<<grid, 64 * NWV, lds, stream>>>((const bf16*)q, (const bf16*)k_cache, (const bf16*)vt_cache,  \
+                                          block_tables, max_pages, tiles, cu_q, ctx_lens, (bf16*)out,   \
+                                          sl, window, page_shift, nq, nkv, d);                          \
   } while (0)
-#define XI_PF_GH(KC, DT, NQT)            \
-  do {                                   \
-    if (gh == 4) XI_PF(KC, DT, NQT, 4);  \
-    else if (gh == 2) XI_PF(KC, DT, NQT, 2); \
-    else XI_PF(KC, DT, NQT, 1);          \
+#define XI_PF_GH(KC, DT, NQT, NWV)             \
+  do {                                         \
+    if (gh == 4) XI_PF(KC, DT, NQT, 4, NWV);   \
+    else if (gh == 2) XI_PF(KC, DT, NQT, 2, NWV); \
+    else XI_PF(KC, DT, NQT, 1, NWV);           \
   } while (0)
-  if (d <= 64) XI_PF_GH(2, 4, 4);
-  else if (d <= 128) XI_PF_GH(4, 8, 4);
-  else if (gh == 2) XI_PF(8, 16, 2, 2);
-  else XI_PF(8, 16, 2, 1);
+  if (d <= 64) XI_PF_GH(2, 4, 2, 8);
+  else if (d <= 128) XI_PF_GH(4, 8, 2, 8);
+  else XI_PF_GH(8, 16, 1, 8);
 #undef XI_PF_GH
 #undef XI_PF
   XI_LAUNCH_CHECK("attention_prefill");
