@@ -439,9 +439,19 @@ def test_attention_prefill_mfma(nq, nkv, d, page, window, seqs):
     ref = _attention_ref(case, seqs, window, scale)
     q, kc, vt, bt = _mfma_inputs(case)
     cu, ctx = _cu_ctx(seqs)
-    qb = kernels.prefill_block(d, nq // nkv)
-    tiles = torch.tensor([(b, q0) for b, (_, n) in enumerate(seqs) for q0 in range(0, n, qb)], dtype=torch.int32)
-    out = kernels.attention_prefill_bf16(q, kc, vt, bt, tiles.to(DEV), cu.to(DEV), ctx.to(DEV), scale, window)
+    for small in (False, True):          # both workgroup shapes
+        qb = kernels.prefill_block(d, nq // nkv, small)
+        tiles = torch.tensor([(b, q0) for b, (_, n) in enumerate(seqs) for q0 in range(0, n, qb)], dtype=torch.int32)
+        out = kernels.attention_prefill_bf16(q, kc, vt, bt, tiles.to(DEV), cu.to(DEV), ctx.to(DEV), scale, window,
+                                             small=small)
+        err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
+        assert err < _tol(torch.bfloat16, 2), (small, err)
+    # the launch order the engine uses: every block once
+    rows, small = kernels.prefill_tiles([n for _, n in seqs], [c for c, _ in seqs], d, nq, nkv)
+    qb = kernels.prefill_block(d, nq // nkv, small)
+    assert sorted(rows) == sorted((b, q0) for b, (_, n) in enumerate(seqs) for q0 in range(0, n, qb))
+    out = kernels.attention_prefill_bf16(q, kc, vt, bt, torch.tensor(rows, dtype=torch.int32).to(DEV), cu.to(DEV),
+                                         ctx.to(DEV), scale, window, small=small)
     err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
     assert err < _tol(torch.bfloat16, 2), err
     # the generic kernel reads the transposed pool too

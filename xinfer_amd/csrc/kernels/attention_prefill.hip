@@ -50,8 +50,10 @@ __device__ __forceinline__ bf16x8 zero8p() {
 // head) pairs, GH heads per position block.  Eight waves of two tiles keep a wave within
 // half of a SIMD's registers, so two waves share a SIMD and one's exponentials overlap the
 // other's matrix instructions.
-template <int KC, int DT, int NQT, int GH, int NWV>
-__global__ __launch_bounds__(64 * NWV) void attn_prefill_lds_kernel(
+// FULLD: head_dim is exactly 16 * DT, so no row tile of V^T lies past the end and the
+// products with V^T are straight-line code.
+template <int KC, int DT, int NQT, int GH, int NWV, bool FULLD>
+__global__ __launch_bounds__(64 * NWV, 2) void attn_prefill_lds_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ vt_cache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ tiles,
     const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, bf16* __restrict__ out, float scale_log2,
@@ -200,36 +202,48 @@ __global__ __launch_bounds__(64 * NWV) void attn_prefill_lds_kernel(
         ka[0][c] = ld8(Ks + r * krow + off);
         ka[1][c] = ld8(Ks + (16 + r) * krow + off);
       }
-      bf16x8 pb_[NQT];
+      // ---- all scores of the step first: 2 * KC * NQT matrix instructions with nothing
+      // between them that waits for their results
+      f32x4 s0[NQT], s1[NQT];
 #pragma unroll
       for (int ct = 0; ct < NQT; ++ct) {
-        f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+        s0[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+        s1[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
 #pragma unroll
-        for (int c = 0; c < KC; ++c) {
-          s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[0][c], qb[ct][c], s0, 0, 0, 0);
-          s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[1][c], qb[ct][c], s1, 0, 0, 0);
+      for (int c = 0; c < KC; ++c)
+#pragma unroll
+        for (int ct = 0; ct < NQT; ++ct) {
+          s0[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[0][c], qb[ct][c], s0[ct], 0, 0, 0);
+          s1[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[1][c], qb[ct][c], s1[ct], 0, 0, 0);
         }
-        float s[8];
+      if (masked) {
+        const int key0 = kb + 8 * j;
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          s[v] = s0[v];
-          s[4 + v] = s1[v];
-        }
-        if (masked) {
-          const int key0 = kb + 8 * j;
+        for (int ct = 0; ct < NQT; ++ct)
 #pragma unroll
-          for (int v = 0; v < 8; ++v) {
-            const int key = key0 + v;
-            if (key > qpos[ct] || key < qlo[ct]) s[v] = -INFINITY;
+          for (int v = 0; v < 4; ++v) {
+            if (key0 + v > qpos[ct] || key0 + v < qlo[ct]) s0[ct][v] = -INFINITY;
+            if (key0 + 4 + v > qpos[ct] || key0 + 4 + v < qlo[ct]) s1[ct][v] = -INFINITY;
           }
-        }
-        // this lane's largest score (raw: the scale is positive and is applied with the shift)
-        const float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
-        // The reference point m_run of the exponentials only has to be near the maximum: it
-        // moves when some score exceeds it by more than 2^kSlack, which is rare after the
-        // first keys, and then the sums so far are rescaled.  P stays below 2^kSlack.
-        if (__any(mx * scale_log2 > m_run[ct] + kSlack)) {
-          float mc = mx * scale_log2;
+      }
+      // ---- this lane's largest score per column tile (raw: the scale is positive and is
+      // applied with the shift).  The reference point m_run of the exponentials only has to
+      // be near the maximum: it moves when some score exceeds it by more than 2^kSlack, which
+      // is rare after the first keys; then the sums so far are rescaled.  P stays below
+      // 2^kSlack.  One test for all column tiles keeps the common path free of branches.
+      float mx[NQT];
+      bool moved = false;
+#pragma unroll
+      for (int ct = 0; ct < NQT; ++ct) {
+        mx[ct] = fmaxf(fmaxf(fmaxf(s0[ct][0], s0[ct][1]), fmaxf(s0[ct][2], s0[ct][3])),
+                       fmaxf(fmaxf(s1[ct][0], s1[ct][1]), fmaxf(s1[ct][2], s1[ct][3]))) * scale_log2;
+        moved = moved || (mx[ct] > m_run[ct] + kSlack);
+      }
+      if (__any(moved)) {
+#pragma unroll
+        for (int ct = 0; ct < NQT; ++ct) {
+          float mc = mx[ct];
           mc = fmaxf(mc, __shfl_xor(mc, 16, kWave));
           mc = fmaxf(mc, __shfl_xor(mc, 32, kWave));
           const float m_new = fmaxf(m_run[ct], mc);
@@ -244,19 +258,26 @@ __global__ __launch_bounds__(64 * NWV) void attn_prefill_lds_kernel(
           }
           m_run[ct] = m_new;
         }
+      }
+      // ---- exponentials, then the products with V^T: straight-line code
+      bf16x8 pb_[NQT];
+#pragma unroll
+      for (int ct = 0; ct < NQT; ++ct) {
         const float m_safe = (m_run[ct] == -INFINITY) ? 0.f : m_run[ct];
         float psum = 0.f;
 #pragma unroll
-        for (int v = 0; v < 8; ++v) {
-          const float p = __builtin_amdgcn_exp2f(fmaf(s[v], scale_log2, -m_safe));
-          psum += p;
-          pb_[ct][v] = (__bf16)p;
+        for (int v = 0; v < 4; ++v) {
+          const float p0 = __builtin_amdgcn_exp2f(fmaf(s0[ct][v], scale_log2, -m_safe));
+          const float p1 = __builtin_amdgcn_exp2f(fmaf(s1[ct][v], scale_log2, -m_safe));
+          psum += p0 + p1;
+          pb_[ct][v] = (__bf16)p0;
+          pb_[ct][4 + v] = (__bf16)p1;
         }
         l_run[ct] += psum;
       }
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
-        if (16 * dt < d) {
+        if (FULLD || 16 * dt < d) {
           const bf16x8 va = ld8(Vs + (16 * dt + r) * vrow + 8 * j);
 #pragma unroll
           for (int ct = 0; ct < NQT; ++ct)
@@ -294,9 +315,12 @@ __global__ __launch_bounds__(64 * NWV) void attn_prefill_lds_kernel(
   }
 }
 
-// Column tiles of a workgroup by head size: eight waves of two tiles up to 128, of one tile
-// above (the accumulators of a tile take twice the registers there).
-static inline int tiles_of(int d) { return d <= 128 ? 16 : 8; }
+// Column tiles of a workgroup by head size and shape: eight waves of two tiles up to 128, of
+// one tile above (the accumulators of a tile take twice the registers there).  The small
+// shape has four waves: half the query positions per workgroup, twice the workgroups, two
+// of them resident on a compute unit.  It serves batches with too few query blocks to give
+// every compute unit two workgroups of different length.
+static inline int tiles_of(int d, int small) { return (d <= 128 ? 16 : 8) / (small ? 2 : 1); }
 // Query heads of a kv head that one workgroup takes together.
 static inline int heads_together(int g) { return g % 4 == 0 ? 4 : (g % 2 == 0 ? 2 : 1); }
 
@@ -310,14 +334,14 @@ int xi_attention_mfma_supported(int nq, int nkv, int d, int page);
 
 // Query positions per workgroup for a head size and a number of query heads per kv head
 // (the host builds `tiles` in steps of it).
-int xi_attention_prefill_block(int d, int g) { return 16 * (tiles_of(d) / heads_together(g)); }
+int xi_attention_prefill_block(int d, int g, int small) { return 16 * (tiles_of(d, small) / heads_together(g)); }
 
 // tiles int32 [n_tiles, 2] = (sequence, first query position of the block within the
-// sequence's portion), first positions being multiples of xi_attention_prefill_block.
+// sequence's portion), first positions being multiples of xi_attention_prefill_block(d, g, small).
 int xi_attention_prefill_bf16(const void* q, const void* k_cache, const void* vt_cache, const int* block_tables,
                               int max_pages, const int* tiles, int n_tiles, const int* cu_q,
                               const int* ctx_lens, void* out, float scale, int window, int page, int nq,
-                              int nkv, int d, hipStream_t stream) {
+                              int nkv, int d, int small, hipStream_t stream) {
   XI_CHECK(xi_attention_mfma_supported(nq, nkv, d, page), "attention_prefill: unsupported sizes nq=%d nkv=%d d=%d page=%d",
            nq, nkv, d, page);
   XI_CHECK(n_tiles >= 0 && n_tiles <= 65535, "attention_prefill: %d query blocks are too many for one launch", n_tiles);
@@ -333,7 +357,8 @@ int xi_attention_prefill_bf16(const void* q, const void* k_cache, const void* vt
   XI_CHECK(page_shift >= 3, "attention_prefill: the page size %d must be a power of two of at least 8", page);
 #define XI_PF(KC, DT, NQT, GH, NWV)                                                                     \
   do {                                                                                                  \
-    auto kern = attn_prefill_lds_kernel<KC, DT, NQT, GH, NWV>;                                          \
+    auto kern = d == 16 * DT ? attn_prefill_lds_kernel<KC, DT, NQT, GH, NWV, true>                      \
+                             : attn_prefill_lds_kernel<KC, DT, NQT, GH, NWV, false>;                    \
     const size_t lds = 2 * (size_t)(kKeys * (32 * KC + kVPad) + d * (kKeys + kVPad)) * sizeof(bf16) +   \
                        (size_t)max_pages * sizeof(int);                                                 \
     XI_CHECK(lds <= 160 * 1024, "attention_prefill: block tables of %d pages do not fit in LDS", max_pages); \
@@ -353,9 +378,15 @@ int xi_attention_prefill_bf16(const void* q, const void* k_cache, const void* vt
     else if (gh == 2) XI_PF(KC, DT, NQT, 2, NWV); \
     else XI_PF(KC, DT, NQT, 1, NWV);           \
   } while (0)
-  if (d <= 64) XI_PF_GH(2, 4, 2, 8);
-  else if (d <= 128) XI_PF_GH(4, 8, 2, 8);
-  else XI_PF_GH(8, 16, 1, 8);
+  if (small) {
+    if (d <= 64) XI_PF_GH(2, 4, 2, 4);
+    else if (d <= 128) XI_PF_GH(4, 8, 2, 4);
+    else XI_PF_GH(8, 16, 1, 4);
+  } else {
+    if (d <= 64) XI_PF_GH(2, 4, 2, 8);
+    else if (d <= 128) XI_PF_GH(4, 8, 2, 8);
+    else XI_PF_GH(8, 16, 1, 8);
+  }
 #undef XI_PF_GH
 #undef XI_PF
   XI_LAUNCH_CHECK("attention_prefill");

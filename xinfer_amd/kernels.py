@@ -262,9 +262,11 @@ def mfma_attention_supported(nq: int, nkv: int, d: int, page: int) -> bool:
     return bool(lib().xi_attention_mfma_supported(nq, nkv, d, page))
 
 
-def attention_prefill_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, scale, window=0, out=None):
+def attention_prefill_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, scale, window=0, out=None,
+                           small=False):
     """MFMA attention for any mix of portions.  tiles int32 [n, 2] = (sequence, first query
-    token of a block of `prefill_block(d, nq // nkv)` tokens within the sequence's portion)."""
+    token of a block of `prefill_block(d, nq // nkv, small)` tokens within the sequence's
+    portion); `small` selects the four-wave workgroup shape (see `prefill_tiles`)."""
     _dev(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, out)
     T, nq, d = q.shape
     nkv, page = k_cache.shape[1], k_cache.shape[2]
@@ -280,14 +282,42 @@ def attention_prefill_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_
     _ok(lib().xi_attention_prefill_bf16(
         _p(q), _p(k_cache), _p(vt_cache), _p(block_tables), int(block_tables.shape[1]), _p(tiles),
         int(tiles.shape[0]), _p(cu_q), _p(ctx_lens), _p(out), ctypes.c_float(scale), int(window), int(page),
-        nq, nkv, d, _stream()))
+        nq, nkv, d, int(bool(small)), _stream()))
     return out
 
 
-def prefill_block(d: int, group: int = 1) -> int:
-    """Query positions per workgroup of the prefill kernel for a head size and a number of
-    query heads per kv head."""
-    return int(lib().xi_attention_prefill_block(int(d), int(group)))
+def prefill_block(d: int, group: int = 1, small: bool = False) -> int:
+    """Query positions per workgroup of the prefill kernel for a head size, a number of
+    query heads per kv head and a workgroup shape."""
+    return int(lib().xi_attention_prefill_block(int(d), int(group), int(bool(small))))
+
+
+COMPUTE_UNITS = 256
+
+
+def prefill_tiles(q_lens, ctx_lens, d: int, nq: int, nkv: int, small: Optional[bool] = None):
+    """The query blocks of a batch of portions for the prefill kernel: (rows, small).
+    rows = [(sequence, first query of the block)] in launch order.  A block's work grows
+    with the keys it sees, and the compute units take workgroups in launch order, so the
+    blocks are sorted by work and laid out in a zigzag over rounds of one workgroup per
+    compute unit.  With few blocks the four-wave shape is used (`small`; chosen here unless
+    given): it doubles the workgroups and lets two of them share a compute unit, and the
+    zigzag gives a unit that got a long block in the first round a short one in the second.
+    The eight-wave shape has one workgroup per unit at a time: longest first."""
+    g = nq // nkv
+    heads = nkv * (g // (4 if g % 4 == 0 else 2 if g % 2 == 0 else 1))     # workgroups per query block
+    big = prefill_block(d, g, False)
+    if small is None:
+        small = sum(-(-n // big) for n in q_lens) * heads < 2 * COMPUTE_UNITS
+    qb = prefill_block(d, g, small)
+    rows = [(b, q0) for b, n in enumerate(q_lens) for q0 in range(0, n, qb)]
+    rows.sort(key=lambda t: -(ctx_lens[t[0]] - q_lens[t[0]] + t[1]))
+    per_round = max(1, COMPUTE_UNITS // heads)
+    out = []
+    for i in range(0, len(rows), per_round):
+        chunk = rows[i:i + per_round]
+        out += chunk if (not small or (i // per_round) % 2 == 0) else chunk[::-1]
+    return out, small
 
 
 def attention_decode_bf16(q, k_cache, vt_cache, block_tables, ctx_lens, max_ctx_len, scale, window=0, out=None,
@@ -330,17 +360,16 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx
         g = nq // nkv
         if ctx.max_q_len == 1 and g <= 16 and (4 * g * d + 8 * g) * 4 <= 64 * 1024:
             return attention_decode_bf16(q, k_cache, v_cache, bt, ctx.ctx_lens, ctx.max_ctx_len, scale, window)
-        qb = prefill_block(d, g)
-        key = ("attention_tiles", qb)
-        tiles = ctx.scratch.get(key)
-        if tiles is None:
-            rows = [(b, q0) for b in range(ctx.num_seqs)
-                    for q0 in range(0, ctx.cu_q_host[b + 1] - ctx.cu_q_host[b], qb)]
-            # blocks that see the most keys start first: the short ones fill the gaps they leave
-            rows.sort(key=lambda t: -(ctx.ctx_lens_host[t[0]] - (ctx.cu_q_host[t[0] + 1] - ctx.cu_q_host[t[0]]) + t[1]))
-            tiles = torch.tensor(rows, dtype=torch.int32, device=q.device).reshape(-1, 2)
-            ctx.scratch[key] = tiles
-        return attention_prefill_bf16(q, k_cache, v_cache, bt, tiles, ctx.cu_q, ctx.ctx_lens, scale, window)
+        key = ("attention_tiles", d, nq, nkv)
+        cached = ctx.scratch.get(key)
+        if cached is None:
+            q_lens = [ctx.cu_q_host[b + 1] - ctx.cu_q_host[b] for b in range(ctx.num_seqs)]
+            rows, small = prefill_tiles(q_lens, ctx.ctx_lens_host, d, nq, nkv)
+            cached = (torch.tensor(rows, dtype=torch.int32, device=q.device).reshape(-1, 2), small)
+            ctx.scratch[key] = cached
+        tiles, small = cached
+        return attention_prefill_bf16(q, k_cache, v_cache, bt, tiles, ctx.cu_q, ctx.ctx_lens, scale, window,
+                                      small=small)
     return attention_generic(q, k_cache, v_cache, bt, ctx.tok_seq, ctx.positions, scale, window,
                              v_transposed=v_transposed)
 
