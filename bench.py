@@ -12,6 +12,10 @@ kernels) followed by greedy sampling on the GPU.  Beside it: the prefill of one
 Data is synthetic: weights are seeded random values of the architecture's shapes made
 on the GPU, token ids are seeded uniform, and the cache contents the decode steps read
 are random values (decode timing does not depend on what the cache holds).
+
+`--workload serve14b` and `--workload long32b` instead run the two serving workloads of the
+larger configurations through the whole engine (scheduler, chunked prefill, continuous
+batching, greedy sampling) and print their own JSON line: total generated tokens per second.
 """
 from __future__ import annotations
 
@@ -29,6 +33,17 @@ QWEN3_8B = dict(
     num_hidden_layers=36, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
     vocab_size=151936, rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False,
     max_position_embeddings=40960, hidden_act="silu")
+QWEN3_14B = dict(QWEN3_8B, hidden_size=5120, intermediate_size=17408, num_hidden_layers=40,
+                 num_attention_heads=40, num_key_value_heads=8)
+QWEN3_32B = dict(QWEN3_8B, hidden_size=5120, intermediate_size=25600, num_hidden_layers=64,
+                 num_attention_heads=64, num_key_value_heads=8)
+# the serving workloads of the two larger configurations
+WORKLOADS = {
+    "serve14b": dict(model=QWEN3_14B, name="Qwen3-14B layer sizes", requests=64, prompt=(128, 2048), new_tokens=256,
+                     chunk=2048, max_model_len=2304),
+    "long32b": dict(model=QWEN3_32B, name="Qwen3-32B layer sizes", requests=16, prompt=(8192, 8192), new_tokens=512,
+                    chunk=2048, max_model_len=8704),
+}
 FULL_LAYERS = QWEN3_8B["num_hidden_layers"]
 CONTEXT = 4096
 PREFILL_TOKENS = 2048
@@ -54,13 +69,61 @@ def prefill_flops(cfg, T):
     return linear + attn
 
 
+def serve(workload: str, layers) -> int:
+    """One of the serving workloads through the whole engine."""
+    import torch
+    from xinfer_amd import EngineConfig, SamplingParams
+    from xinfer_amd.engine import build_model
+    from xinfer_amd.engine.llm_engine import LLMEngine
+    from xinfer_amd.models import config_from_dict
+    from xinfer_amd.weights.random_init import random_store_for
+
+    w = WORKLOADS[workload]
+    full = w["model"]["num_hidden_layers"]
+    raw = dict(w["model"], num_hidden_layers=layers or full)
+    _, cfg = config_from_dict(raw)
+    t0 = time.time()
+    model = build_model(cfg, random_store_for(cfg, seed=0), "bf16", "cuda:0")
+    torch.cuda.synchronize()
+    print(f"[bench] {w['name']}, {cfg.num_hidden_layers} layers, built in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
+    page = 64
+    n = w["requests"]
+    pages = n * (-(-w["max_model_len"] // page)) + 8
+    eng = LLMEngine(EngineConfig(max_num_seqs=n, max_model_len=w["max_model_len"], num_pages=pages, page_size=page,
+                                 prefill_chunk_size=w["chunk"], max_num_batched_tokens=w["chunk"] + n, seed=1),
+                    model=model)
+    g = torch.Generator().manual_seed(4)
+    lo, hi = w["prompt"]
+    lens = [lo] * n if lo == hi else torch.randint(lo, hi + 1, (n,), generator=g).tolist()
+    prompts = [torch.randint(0, cfg.vocab_size, (m,), generator=g).tolist() for m in lens]
+    sp = SamplingParams(temperature=0.0, max_tokens=w["new_tokens"], ignore_eos=True)
+    eng.generate(prompts[:2], SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True))   # warm-up
+    steps0 = eng.steps
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    outs = eng.generate(prompts, sp)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t
+    new = sum(o.decoded_length for o in outs)
+    print(json.dumps({
+        "metric": f"generated tok/s, {workload} workload, bf16", "value": round(new / dt, 1), "unit": "tokens/s",
+        "n_gpus": 1, "seconds": round(dt, 3), "engine_steps": eng.steps - steps0, "higher_is_better": True,
+        "dtype": "bf16", "data": "synthetic: seeded random weights, uniform random token ids",
+        "config": {"model": w["name"], "layers": cfg.num_hidden_layers, "layers_of_model": full, "requests": n,
+                   "prompt_tokens": sum(lens), "new_tokens": new, "prefill_chunk": w["chunk"],
+                   "preemptions": eng.num_preemptions, "total_tok_per_s": round((sum(lens) + new) / dt, 1)}}), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS,
+    ap.add_argument("--layers", type=int, default=None,
                     help="fewer layers than the configuration has (reported in config)")
+    ap.add_argument("--workload", choices=["decode"] + sorted(WORKLOADS), default="decode",
+                    help="decode: the contract's run (default); the others: a serving workload end to end")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--skip-points", action="store_true", help="only the default decode run")
     ap.add_argument("--only", choices=["all", "decode", "prefill"], default="all",
@@ -69,6 +132,10 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.workload != "decode":
+        return serve(args.workload, args.layers)
+    if args.layers is None:
+        args.layers = FULL_LAYERS
 
     import torch
     from xinfer_amd.engine import ModelRunner, StepEntry, build_model

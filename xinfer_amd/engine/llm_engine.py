@@ -52,16 +52,23 @@ class _Request:
 
 
 class LLMEngine:
-    def __init__(self, econfig: EngineConfig, dtype="bf16"):
+    def __init__(self, econfig: EngineConfig, dtype="bf16", model=None):
+        """`model`: a loaded `CausalLM` to run instead of the folder `econfig` names (random
+        weights built in memory, for measurements); the tokenizer is then the byte tokenizer."""
         self.econfig = econfig
-        self.dtype = parse_dtype(dtype)
-        model_dir = econfig.model_dir()
-        self.model = load_model(model_dir, self.dtype, econfig.device)
+        if model is None:
+            self.dtype = parse_dtype(dtype)
+            model_dir = econfig.model_dir()
+            self.model = load_model(model_dir, self.dtype, econfig.device)
+        else:
+            model_dir = None
+            self.model = model
+            self.dtype = model.dtype
         spec = self.model.spec
         self.max_model_len = min(econfig.max_model_len or spec.max_positions, spec.max_positions)
         self.tokenizer = load_tokenizer(model_dir, spec.vocab_size)
         self.eos_token_ids = set(spec.eos_token_ids) | set(self.tokenizer.eos_token_ids())
-        self.generation_cfg = econfig.generation_cfg or _read_generation_config(model_dir)
+        self.generation_cfg = econfig.generation_cfg or (_read_generation_config(model_dir) if model_dir else None)
         self.seed = econfig.seed if econfig.seed is not None else int.from_bytes(os.urandom(4), "little")
         page = econfig.page_size
         num_pages = econfig.num_pages or self._plan_pages(page)

@@ -70,7 +70,8 @@ class FileTokenizer:
         return list(self._eos)
 
 
-def load_tokenizer(model_dir: str, vocab_size: int):
-    if os.path.isfile(os.path.join(model_dir, "tokenizer.json")):
+def load_tokenizer(model_dir, vocab_size: int):
+    """`model_dir` may be None (a model built in memory): the byte tokenizer."""
+    if model_dir and os.path.isfile(os.path.join(model_dir, "tokenizer.json")):
         return FileTokenizer(model_dir)
     return ByteTokenizer(vocab_size)
