@@ -28,6 +28,14 @@ TINY = {
         seed=2, linear_std=0.05, norm_std=0.2, page_size=16),
 }
 
+# O: widths that are multiples of neither 8 nor 4, a group of three heads and one layer: every
+# kernel's vectorized form has to step aside for its plain one.
+TINY["O"] = dict(
+    config=_cfg(num_hidden_layers=1, hidden_size=102, num_attention_heads=3, num_key_value_heads=1,
+                head_dim=16, intermediate_size=182, vocab_size=257, rope_theta=777.0,
+                rms_norm_eps=3e-6, tie_word_embeddings=True, max_position_embeddings=256),
+    seed=5, linear_std=0.04, norm_std=0.15, page_size=8)
+
 
 # Real layer sizes (Qwen3-8B and Qwen3-32B) with few layers and a small vocabulary: the
 # kernels run at the head size, group, widths and K lengths they serve in production.

@@ -431,8 +431,8 @@ PREFILL_CASES = ATTN_CASES + [
 @pytest.mark.parametrize("nq,nkv,d,page,window,seqs", PREFILL_CASES)
 def test_attention_prefill_mfma(nq, nkv, d, page, window, seqs):
     from xinfer_amd import kernels
-    if page % 8:
-        pytest.skip("the matrix-core kernels need pages of a multiple of 8 tokens")
+    if not kernels.mfma_attention_supported(nq, nkv, d, page):
+        pytest.skip("the matrix-core kernels need a page of a power of two of at least 8 tokens")
     g = torch.Generator().manual_seed(21)
     case = _paged_case(g, torch.bfloat16, nq, nkv, d, page, seqs)
     scale = 1.0 / math.sqrt(d)
