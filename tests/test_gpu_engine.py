@@ -188,6 +188,27 @@ def test_eos_and_limits(model_dirs):
         eng.generate([[1] * 40], SamplingParams(max_tokens=2))
 
 
+# ---- the command line ----------------------------------------------------------------------------
+def test_command_line(model_dirs, capsys):
+    """`python -m xinfer_amd` with the reference's option names: prompts as text (the folder has
+    no tokenizer.json, so bytes are the tokens) and as token ids, greedy, and the two
+    throughput lines of the reference's output."""
+    from xinfer_amd import cli
+    rc = cli.main(["--w", model_dirs["A"], "--prompts", "How are you?|Tell me", "--max-tokens", "6",
+                   "--max-model-len", "64", "--temperature", "0", "--ignore-eos", "--page-size", "16",
+                   "--num-pages", "8", "--dtype", "f32"])
+    out = capsys.readouterr().out
+    assert rc == 0
+    assert "[Prompt 1]" in out and "[Prompt 2]" in out and "Response:" in out
+    assert "Prompt tokens: 19 in" in out and "Decoded tokens: 12 in" in out
+    rc = cli.main(["--m", model_dirs["A"], "--prompt-ids", "1,2,3|4,5", "--max-tokens", "4", "--max-model-len", "32",
+                   "--seed", "3", "--page-size", "16", "--num-pages", "4", "--batch", "3", "--ignore-eos"])
+    out = capsys.readouterr().out
+    assert rc == 0 and "Decoded tokens: 12 in" in out and "[Prompt 1]" not in out     # --batch repeats the first prompt
+    assert cli.main(["--m", model_dirs["A"], "--w", model_dirs["A"]]) == 2
+    assert cli.main([]) == 2
+
+
 # ---- long decoding and first tokens ----------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_one_by_one(dtype, model_dirs):
