@@ -188,6 +188,39 @@ def test_eos_and_limits(model_dirs):
         eng.generate([[1] * 40], SamplingParams(max_tokens=2))
 
 
+# ---- streaming -----------------------------------------------------------------------------------
+def test_streams_interleave_and_cancel(model_dirs):
+    """Two streams read in turn give the tokens `generate` gives; a cancelled stream gives its
+    pages back at once."""
+    from xinfer_amd import Message, SamplingParams
+    rng = random.Random(6)
+    p1, p2 = harness.random_prompt(rng, 21, 256), harness.random_prompt(rng, 9, 256)
+    sp = SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True)
+    eng = _engine(model_dirs["A"], "A", "f32", max_num_seqs=3, num_pages=12, prefill_chunk_size=8)
+    want = [o.token_ids for o in eng.generate([p1, p2], sp)]
+    id1, n1, s1 = eng.generate_stream(sp, p1)
+    id2, n2, s2 = eng.generate_stream(sp, p2)
+    assert (n1, n2) == (21, 9) and id1 != id2 and s1.seq_id == id1
+    got1, got2, done = [], [], []
+    for a, b in zip(s1, s2):
+        for item, got in ((a, got1), (b, got2)):
+            if item.datatype == "TOKEN_ID":
+                got.append(item.data)
+            elif item.datatype == "DONE":
+                done.append(item.data)
+            else:
+                assert item.datatype == "TOKEN" and isinstance(item.data, str)
+    assert [got1, got2] == want and len(done) == 2 and done[0][3] == 10 and s1.finished and s2.finished
+    _, _, s3 = eng.generate_stream(SamplingParams(temperature=0.0, max_tokens=50, ignore_eos=True),
+                                   [Message("user", "hello there")])
+    first = [next(s3) for _ in range(4)]
+    assert [i.datatype for i in first] == ["TOKEN_ID", "TOKEN"] * 2
+    assert eng.get_available_kv_tokens() < 12 * 16
+    s3.cancel()
+    assert s3.cancelled and list(s3) == []
+    assert eng.get_available_kv_tokens() == 12 * 16 and eng.runner.cache.live_requests() == 0
+
+
 # ---- the command line ----------------------------------------------------------------------------
 def test_command_line(model_dirs, capsys):
     """`python -m xinfer_amd` with the reference's option names: prompts as text (the folder has

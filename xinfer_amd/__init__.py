@@ -7,7 +7,7 @@
 Names follow the reference's Python package (xinfer.pyi).
 """
 from .config.engine_config import (EngineConfig, GenerationConfig, GenerationOutput, Message,
-                                   SamplingParams)
+                                   SamplingParams, StreamItem)
 
 
 def __getattr__(name):
@@ -19,4 +19,4 @@ def __getattr__(name):
 
 
 __all__ = ["Engine", "EngineConfig", "GenerationConfig", "GenerationOutput", "LLMEngine", "Message",
-           "SamplingParams"]
+           "SamplingParams", "StreamItem"]

@@ -55,6 +55,15 @@ class GenerationOutput:
     finish_reason: str = ""                                 # "eos", "length", "max_model_len"
 
 
+@dataclass(frozen=True)
+class StreamItem:
+    """An item of an `EngineStream` (xinfer.pyi:160-180).  datatype / data:
+    "TOKEN" / the token's text; "TOKEN_ID" / its id; "DONE" / (prompt_start_time,
+    decode_start_time, decode_finish_time, decoded_length); "ERROR" / a message."""
+    datatype: str
+    data: object
+
+
 @dataclass
 class EngineConfig:
     model_id: Optional[str] = None          # a local model folder (there is no hub download here)

@@ -16,7 +16,8 @@ from typing import Dict, Iterable, List, Optional, Sequence, Union
 
 import torch
 
-from ..config.engine_config import EngineConfig, GenerationConfig, GenerationOutput, Message, SamplingParams
+from ..config.engine_config import (EngineConfig, GenerationConfig, GenerationOutput, Message, SamplingParams,
+                                    StreamItem)
 from ..sampling import Sampler, Strategy, resolve_strategy, uniform
 from .loading import load_model, parse_dtype
 from .runner import ModelRunner, StepEntry
@@ -207,12 +208,82 @@ class LLMEngine:
         self.run_until_done()
         return [self._output(self._finished.pop(rid)) for rid in rids]
 
+    def generate_stream(self, params: SamplingParams,
+                        messages: Union[Sequence[Message], str, Sequence[int]]):
+        """The reference's streaming entry point (xinfer.pyi:206-216): returns (seq_id,
+        prompt_length, stream).  `messages` is a chat (rendered with the chat template), or a
+        prompt as text or token ids."""
+        if isinstance(messages, str):
+            ids = self.tokenizer.encode(messages)
+        elif messages and isinstance(messages[0], Message):
+            ids = self.tokenizer.encode(self.tokenizer.apply_chat_template(list(messages)))
+        else:
+            ids = [int(t) for t in messages]
+        rid = self.add_request(ids, params)
+        return rid, len(ids), EngineStream(self, rid, len(ids))
+
+    def cancel(self, rid: int) -> None:
+        """Ends a request now and gives back what it holds (reference: Scheduler::cancel,
+        /root/reference/src/core/scheduler.rs:780-818)."""
+        r = self._requests.pop(rid, None)
+        if r is None:
+            return
+        self.scheduler.finish(rid)
+        r.finish_reason = "cancelled"
+        r.decode_finish = _now_ms()
+
     def generate_sync(self, params: Sequence[SamplingParams],
                       message_list: Sequence[Sequence[Message]]) -> List[GenerationOutput]:
         """The reference's blocking chat entry point (xinfer.pyi:199-205): every message list
         is rendered with the chat template and completed."""
         prompts = [self.tokenizer.apply_chat_template(list(m)) for m in message_list]
         return self.generate(prompts, list(params))
+
+
+class EngineStream:
+    """Tokens of one request as they are generated (the reference's EngineStream,
+    xinfer.pyi:182-189).  Iterating drives the engine: every step also advances whatever other
+    requests are live.  Each token comes as a TOKEN_ID item followed by a TOKEN item with its
+    text; the last item is DONE."""
+
+    def __init__(self, engine: "LLMEngine", rid: int, prompt_length: int):
+        self._engine = engine
+        self.seq_id = rid
+        self.prompt_length = prompt_length
+        self.finished = False
+        self.cancelled = False
+        self._sent = 0
+        self._pending: List[StreamItem] = []
+
+    def cancel(self) -> None:
+        if not self.finished and not self.cancelled:
+            self._engine.cancel(self.seq_id)
+            self.cancelled = True
+
+    def __iter__(self):
+        return self
+
+    def __next__(self) -> StreamItem:
+        eng = self._engine
+        while not self._pending:
+            if self.finished or self.cancelled:
+                raise StopIteration
+            r = eng._requests.get(self.seq_id) or eng._finished.get(self.seq_id)
+            if r is None:
+                self.finished = True
+                return StreamItem("ERROR", f"request {self.seq_id} is gone")
+            gen = r.generated
+            if self._sent < len(gen):
+                tok = gen[self._sent]
+                self._sent += 1
+                self._pending = [StreamItem("TOKEN", eng.tokenizer.decode([tok]))]
+                return StreamItem("TOKEN_ID", tok)
+            if self.seq_id in eng._finished:
+                eng._finished.pop(self.seq_id)
+                self.finished = True
+                return StreamItem("DONE", (r.prompt_start, r.decode_start, r.decode_finish, len(gen)))
+            eng.step()
+        return self._pending.pop(0)
 
 
 def _read_generation_config(model_dir: str) -> Optional[GenerationConfig]:
