@@ -171,7 +171,8 @@ def main() -> int:
     def decode_run(batch, steps, warmup):
         """`batch` requests whose caches already hold CONTEXT - steps - warmup tokens decode
         steps + warmup tokens, so that the last timed step ends at CONTEXT."""
-        start = CONTEXT - steps - warmup
+        prep = runner.graph_after          # steps before the warm-up in which the decode graph is recorded
+        start = CONTEXT - steps - warmup - prep
         rids = list(range(100, 100 + batch))
         for rid in rids:
             runner.add_request(rid)
@@ -183,7 +184,7 @@ def main() -> int:
             logits = runner.step([StepEntry(r, [t], [0]) for r, t in zip(rids, toks)])
             return sampler.argmax(logits).tolist()
 
-        for _ in range(warmup):
+        for _ in range(prep + warmup):
             toks = one(toks)
         sync()
         t = time.perf_counter()

@@ -319,7 +319,7 @@ def test_decode_graph_replays_equal_launch_by_launch(name, n_req, dtype, model_d
     feed = {i: harness.random_prompt(rng, 40, vocab) for i in prompts}
 
     def run(use_graphs):
-        runner = ModelRunner(model, page, 16 * (n_req + 2), n_req + 2, use_graphs=use_graphs)
+        runner = ModelRunner(model, page, 16 * (n_req + 2), n_req + 2, use_graphs=use_graphs, graph_after=1)
         out = []
         live = list(range(n_req))
         for i in live:
@@ -345,6 +345,19 @@ def test_decode_graph_replays_equal_launch_by_launch(name, n_req, dtype, model_d
     assert len(want) == len(got)
     for k, (a, b) in enumerate(zip(want, got)):
         assert a.shape == b.shape and torch.equal(a, b), f"step {k} differs between graph and launches"
+
+
+def test_a_batch_size_is_recorded_the_third_time_it_is_seen(model_dirs):
+    from xinfer_amd.engine import ModelRunner, StepEntry, load_model
+    runner = ModelRunner(load_model(model_dirs["A"], "bfloat16", DEV), 16, 8, 2)
+    runner.add_request(0)
+    runner.add_request(1)
+    for step in range(5):
+        runner.step([StepEntry(0, [step], [0]), StepEntry(1, [step + 7], [0])])
+        assert (len(runner._graphs), runner.graph_replays) == ((0, 0) if step < 2 else (1, step - 1))
+    runner.release(1)
+    runner.step([StepEntry(0, [9], [0])])                      # another batch size: first sighting
+    assert (len(runner._graphs), runner.graph_replays) == (1, 3)
 
 
 def test_model_with_a_part_that_reads_the_host_is_not_recorded(model_dirs):

@@ -88,9 +88,12 @@ class _DecodeGraph:
 
 class ModelRunner:
     def __init__(self, model: CausalLM, page_size: int, num_pages, max_requests: int,
-                 use_graphs: bool = True, graph_max_batch: int = 64):
+                 use_graphs: bool = True, graph_max_batch: int = 64, graph_after: int = 3):
         """`num_pages`: pages of every group's pool, or a list with one count per group.
-        `use_graphs`: record decode steps of up to `graph_max_batch` requests as HIP graphs."""
+        `use_graphs`: record decode steps of up to `graph_max_batch` requests as HIP graphs; a
+        (batch size, context bucket) is recorded the `graph_after`-th time it is seen, so that
+        batch sizes that merely pass by (requests finishing one after the other) do not pay
+        for a recording."""
         if not torch.cuda.is_available():
             raise RuntimeError("xinfer_amd runs on an AMD GPU only: no HIP device is visible")
         self.model = model
@@ -125,7 +128,9 @@ class ModelRunner:
         self._staging = _Staging(self.device)
         self.use_graphs = bool(use_graphs) and model.graph_safe
         self.graph_max_batch = int(graph_max_batch)
+        self.graph_after = max(1, int(graph_after))
         self._graphs: Dict[Tuple[int, int], _DecodeGraph] = {}
+        self._seen: Dict[Tuple[int, int], int] = {}
         self._graph_pool = None
         # widest block table a request can have: the fixed width of a recorded step's tables
         self._max_table = max(1, -(-model.spec.max_positions // self.page_size))
@@ -243,6 +248,10 @@ class ModelRunner:
         all_rows[:rows32.size] = rows32
         g = self._graphs.get(key)
         if g is None:
+            self._seen[key] = self._seen.get(key, 0) + 1
+            if self._seen[key] < self.graph_after:         # not yet: launch by launch
+                ctx, ids, want_rows, _, _ = self._context(a, ids32, rows32)
+                return self.model.forward(ids, ctx, self.layer_caches, want_rows)
             ctx, ids, want, d32, d64 = self._context(a, ids32, all_rows, max_ctx_len=bucket, host_lengths=False)
             every_row = torch.arange(B, dtype=torch.int32, device=self.device)
             cur = torch.cuda.current_stream(self.device)
