@@ -128,13 +128,16 @@ def test_linear_skinny(M, N, K, out_dtype):
     tol = 2.0 ** -8 if out_dtype == torch.bfloat16 else 1e-5
     xd, wd = x.to(DEV), w.to(DEV)
     outs = {}
-    for rt, nw in [(0, 0), (1, 8), (2, 8), (4, 8), (1, 16), (2, 16)]:
+    shapes = [(0, 0), (1, 8), (2, 8), (3, 8), (4, 8), (6, 8), (1, 16), (2, 16)] + ([(8, 8)] if M <= 32 else [])
+    for rt, nw in shapes:
         y = kernels.linear_skinny(xd, wd, out_dtype, row_tiles=rt, waves=nw)
         assert y.dtype == out_dtype and y.shape == (M, N)
         err = (y.cpu().double() - ref).abs().max() / ref.abs().max()
         assert err < tol, (rt, nw, err)
         outs[(rt, nw)] = y.cpu()
-    assert torch.equal(outs[(1, 8)], outs[(2, 8)]) and torch.equal(outs[(1, 8)], outs[(4, 8)])
+    for rt, nw in shapes:
+        if nw == 8:
+            assert torch.equal(outs[(1, 8)], outs[(rt, 8)]), rt
     assert torch.equal(outs[(1, 16)], outs[(2, 16)])
     r = M // 2
     for nw in (8, 16):
@@ -181,10 +184,15 @@ def test_linear_skinny_gated(M, I, K):
     w = _rand((2 * I, K), torch.bfloat16, g, 0.1)
     gu = x.double() @ w.double().T
     ref = plain.swiglu(gu[:, :I], gu[:, I:])
-    y = kernels.linear_skinny(x.to(DEV), w.to(DEV), gated=True)
-    assert y.shape == (M, I)
-    err = (y.cpu().double() - ref).abs().max() / ref.abs().max()
-    assert err < 2.0 ** -8, err
+    outs = []
+    for rt in (0, 2, 4, 6) + ((8,) if M <= 32 else ()):
+        y = kernels.linear_skinny(x.to(DEV), w.to(DEV), gated=True, row_tiles=rt, waves=8 if rt else 0)
+        assert y.shape == (M, I)
+        err = (y.cpu().double() - ref).abs().max() / ref.abs().max()
+        assert err < 2.0 ** -8, (rt, err)
+        outs.append(y.cpu())
+    for y in outs[2:]:
+        assert torch.equal(y, outs[1])     # the row tiles of a workgroup do not change a sum
 
 
 def test_linear_skinny_refuses():
@@ -197,8 +205,12 @@ def test_linear_skinny_refuses():
         kernels.linear_skinny(x[:4, :60].contiguous(), w[:, :60].contiguous())
     with pytest.raises(kernels.KernelError, match="bfloat16"):
         kernels.linear_skinny(x[:4].float(), w.float())
-    with pytest.raises(kernels.KernelError, match="LDS"):
+    with pytest.raises(kernels.KernelError, match="no kernel of 4 row tiles, 16 waves"):
         kernels.linear_skinny(x[:4].contiguous(), w, row_tiles=4, waves=16)
+    with pytest.raises(kernels.KernelError, match="no kernel of 5 row tiles"):
+        kernels.linear_skinny(x[:4].contiguous(), w, row_tiles=5, waves=8)
+    with pytest.raises(kernels.KernelError, match="no kernel of 8 row tiles"):
+        kernels.linear_skinny(x[:40].contiguous(), w, row_tiles=8, waves=8)
 
 
 def _rope_ref(x, pos, cos, sin, rot, interleaved):

@@ -108,12 +108,20 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_vec_kernel(float* __restrict__
       s[v] = load4(x + 4 * i);
       wv[v] = load4(w + 4 * i);
       if (yr) {
-        for (int p = 0; p < parts; ++p) {
-          const float4 yy = load4(yr + p * part_stride + 4 * i);
-          s[v].x += yy.x;
-          s[v].y += yy.y;
-          s[v].z += yy.z;
-          s[v].w += yy.w;
+        // up to 4 parts at a time: their loads are issued together, the sums run in order
+        for (int p0 = 0; p0 < parts; p0 += 4) {
+          float4 yy[4];
+#pragma unroll
+          for (int p = 0; p < 4; ++p)
+            yy[p] = p0 + p < parts ? load4(yr + (p0 + p) * part_stride + 4 * i) : float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int p = 0; p < 4; ++p)
+            if (p0 + p < parts) {
+              s[v].x += yy[p].x;
+              s[v].y += yy[p].y;
+              s[v].z += yy[p].z;
+              s[v].w += yy[p].w;
+            }
         }
       }
     } else {

@@ -21,6 +21,7 @@
 // Reference call sites: candle matmul in /root/reference/src/models/layers/linear.rs:76-124
 // (vendor BLAS); fused gate/up + silu_and_mul in /root/reference/src/models/layers/mlp.rs:613-633.
 #include "common.h"
+#include <cmath>
 #include <type_traits>
 
 namespace xi {
@@ -50,8 +51,14 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16* __re
                                                                 TO* __restrict__ y, int M, int N, int K,
                                                                 int steps_per_slice) {
   static_assert(!GATED || RT % 2 == 0, "the gated form pairs gate tiles with up tiles");
-  static_assert((NW / 2) * RT * MT <= 64, "the merge buffer must fit in 64 KB of LDS");
-  __shared__ float red[(NW / 2) * RT * MT * 256];
+  // The waves' sums are merged through LDS a chunk of PC output tiles (gated: pairs of a gate
+  // and an up tile) at a time, so that the buffer stays within 64 KB whatever RT and MT are.
+  constexpr int H = NW / 2;                      // waves whose sums are left after the first round
+  constexpr int TP = GATED ? 2 : 1;              // tiles of w per output tile
+  constexpr int PAIRS = RT / TP;
+  static_assert(H * TP * MT <= 64, "one output tile's sums must fit in 64 KB of LDS");
+  constexpr int PC = (64 / (H * TP * MT)) < PAIRS ? (64 / (H * TP * MT)) : PAIRS;
+  __shared__ float red[H * PC * TP * MT * 256];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, j = lane >> 4;
   const int n0 = blockIdx.x * (GATED ? 16 * (RT / 2) : 16 * RT);
@@ -111,6 +118,41 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16* __re
           acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], b[m][u], acc[t][m], 0, 0, 0);
     s += UU;
   };
+  // The main part keeps U steps of loads in flight all the time: a step's registers are loaded
+  // again, U steps ahead, right after its products.  The sums run in the same order as in
+  // `block`, so the result does not depend on which of the two forms ran.
+  if (s + 2 * U <= s_fast) {
+    bf16x8 a[RT][U], b[MT][U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int t = 0; t < RT; ++t) a[t][u] = ldg8(wp[t] + 32 * (s + u));
+#pragma unroll
+      for (int m = 0; m < MT; ++m) b[m][u] = ldg8(xp[m] + 32 * (s + u));
+    }
+    for (; s + 2 * U <= s_fast; s += U) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int t = 0; t < RT; ++t)
+#pragma unroll
+          for (int m = 0; m < MT; ++m)
+            acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], b[m][u], acc[t][m], 0, 0, 0);
+#pragma unroll
+        for (int t = 0; t < RT; ++t) a[t][u] = ldg8(wp[t] + 32 * (s + U + u));
+#pragma unroll
+        for (int m = 0; m < MT; ++m) b[m][u] = ldg8(xp[m] + 32 * (s + U + u));
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+          acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][u], b[m][u], acc[t][m], 0, 0, 0);
+    s += U;
+  }
   while (s + U <= s_fast) block(std::integral_constant<int, U>{});
   if constexpr (U >= 8) {
     if (s + 4 <= s_fast) block(std::integral_constant<int, 4>{});
@@ -133,48 +175,58 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16* __re
 
   // merge the waves in a fixed order: wave w + NW/2 hands its sums to wave w, then all threads
   // add the NW/2 sums that are left, in wave order, and store.  A lane's 4 values of a tile:
-  // token r, features 4j..4j+3.
-  constexpr int H = NW / 2;
-  if (wave >= H) {
-#pragma unroll
-    for (int t = 0; t < RT; ++t)
-#pragma unroll
-      for (int m = 0; m < MT; ++m)
-        *reinterpret_cast<f32x4*>(&red[(((wave - H) * RT + t) * MT + m) * 256 + lane * 4]) = acc[t][m];
-  }
-  __syncthreads();
-  if (wave < H) {
-#pragma unroll
-    for (int t = 0; t < RT; ++t)
-#pragma unroll
-      for (int m = 0; m < MT; ++m) {
-        f32x4* slot = reinterpret_cast<f32x4*>(&red[((wave * RT + t) * MT + m) * 256 + lane * 4]);
-        const f32x4 o = *slot;
-        f32x4 sum = acc[t][m];
-        sum[0] += o[0];
-        sum[1] += o[1];
-        sum[2] += o[2];
-        sum[3] += o[3];
-        *slot = sum;      // the same lane wrote and reads this slot: no barrier in between
-      }
-  }
-  __syncthreads();
-
+  // token r, features 4j..4j+3.  Slot of (wave wv, output tile q of the chunk, part tp, token
+  // tile m): ((wv * PC + q) * TP + tp) * MT + m.
   TO* yk = y + (size_t)ks * M * N;   // this slice's partial sums (ks is 0 without slices)
-  constexpr int PAIRS = GATED ? RT / 2 : RT;
-  for (int idx = threadIdx.x; idx < PAIRS * MT * 256; idx += NW * 64) {
-    const int tile = idx >> 8, e = idx & 255;
-    const int p = tile / MT, m = tile - p * MT;
-    const int ln = e >> 2, v = e & 3;
-    const int token = 16 * m + (ln & 15), n = n0 + 16 * p + 4 * (ln >> 4) + v;
-    float a0 = 0.f, a1 = 0.f;
 #pragma unroll
-    for (int wv = 0; wv < H; ++wv) {
-      a0 += red[((wv * RT + p) * MT + m) * 256 + e];
-      if (GATED) a1 += red[((wv * RT + RT / 2 + p) * MT + m) * 256 + e];
+  for (int p0 = 0; p0 < PAIRS; p0 += PC) {
+    if (p0 > 0) __syncthreads();     // the chunk before has been read
+    if (wave >= H) {
+#pragma unroll
+      for (int q = 0; q < PC; ++q)
+#pragma unroll
+        for (int tp = 0; tp < TP; ++tp)
+#pragma unroll
+          for (int m = 0; m < MT; ++m)
+            if (p0 + q < PAIRS)
+              *reinterpret_cast<f32x4*>(&red[((((wave - H) * PC + q) * TP + tp) * MT + m) * 256 + lane * 4]) =
+                  acc[tp * PAIRS + (p0 + q < PAIRS ? p0 + q : 0)][m];
     }
-    if (token < M && n < N)
-      yk[(size_t)token * N + n] = from_float<TO>(GATED ? a0 / (1.f + __expf(-a0)) * a1 : a0);
+    __syncthreads();
+    if (wave < H) {
+#pragma unroll
+      for (int q = 0; q < PC; ++q)
+#pragma unroll
+        for (int tp = 0; tp < TP; ++tp)
+#pragma unroll
+          for (int m = 0; m < MT; ++m)
+            if (p0 + q < PAIRS) {
+              f32x4* slot = reinterpret_cast<f32x4*>(&red[(((wave * PC + q) * TP + tp) * MT + m) * 256 + lane * 4]);
+              const f32x4 o = *slot;
+              f32x4 sum = acc[tp * PAIRS + (p0 + q < PAIRS ? p0 + q : 0)][m];
+              sum[0] += o[0];
+              sum[1] += o[1];
+              sum[2] += o[2];
+              sum[3] += o[3];
+              *slot = sum;      // the same lane wrote and reads this slot: no barrier in between
+            }
+    }
+    __syncthreads();
+    const int pairs_here = PAIRS - p0 < PC ? PAIRS - p0 : PC;
+    for (int idx = threadIdx.x; idx < pairs_here * MT * 256; idx += NW * 64) {
+      const int tile = idx >> 8, e = idx & 255;
+      const int q = tile / MT, m = tile - q * MT;
+      const int ln = e >> 2, v = e & 3;
+      const int token = 16 * m + (ln & 15), n = n0 + 16 * (p0 + q) + 4 * (ln >> 4) + v;
+      float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < H; ++wv) {
+        a0 += red[(((wv * PC + q) * TP) * MT + m) * 256 + e];
+        if (GATED) a1 += red[(((wv * PC + q) * TP + 1) * MT + m) * 256 + e];
+      }
+      if (token < M && n < N)
+        yk[(size_t)token * N + n] = from_float<TO>(GATED ? a0 / (1.f + __expf(-a0)) * a1 : a0);
+    }
   }
 }
 
@@ -184,39 +236,53 @@ struct SkinnyPlan {
   int rt;    // row tiles per workgroup
 };
 
+// Shapes that are built: 16 waves leave registers for 2 row tiles, 8 row tiles for 32 tokens.
+static bool skinny_shape_ok(int rt, int nw, int mt, bool gated) {
+  if (gated ? !(rt == 2 || rt == 4 || rt == 6 || rt == 8) : !(rt == 1 || rt == 2 || rt == 3 || rt == 4 || rt == 6 || rt == 8))
+    return false;
+  if (nw == 16 && rt > 2) return false;
+  if (rt == 8 && mt > 2) return false;
+  return true;
+}
+
 // ks and nw fix the order of the sums: they come from (N, K) and the caller's wish alone.
-// rt only says which workgroup computes what; it grows with M (reuse of the x operands) as
-// long as enough workgroups remain.
+// rt only says which workgroup computes what, and is chosen for speed.  Measured on MI355X:
+// a workgroup reads its x operands from L2 once per 16 * rt rows of w, and such a read costs
+// about 0.6 of a read of w from memory, so more row tiles pay with more rows of x; the
+// stream of w itself slows by about 4% per further row tile; and a grid that is no multiple of
+// the 256 compute units leaves some of them idle at the end.
 static SkinnyPlan plan_skinny(int M, int N, int K, bool gated, bool allow_split) {
   SkinnyPlan p;
-  const int tiles = (N + 15) / 16;
+  const int tiles = (N + 15) / 16;       // output tiles (gated: each a gate tile and an up tile)
   p.ks = 1;
   if (allow_split && !gated) {
     p.ks = (1024 + tiles - 1) / tiles;
     if (p.ks > 4) p.ks = 4;
     while (p.ks > 1 && K / p.ks < 512) --p.ks;
   }
-  p.nw = (gated || tiles * p.ks >= 1024) ? 8 : 16;
+  p.nw = 8;
   const int mt = (M + 15) / 16;
-  if (gated) {
-    p.rt = (mt >= 2 && tiles / 2 >= 256) ? 4 : 2;
-  } else {
-    int rt_max = M <= 4 ? 1 : (mt == 1 ? 2 : 4);
-    if (p.nw == 16 && rt_max > 2) rt_max = 2;
-    const int enough = mt >= 3 ? 256 : 512;      // workgroups that still fill the chip
-    p.rt = 1;
-    for (int rt = rt_max; rt > 1; rt >>= 1)
-      if ((tiles + rt - 1) / rt * p.ks >= enough) {
-        p.rt = rt;
-        break;
-      }
+  const int per = gated ? 2 : 1;         // tiles of w per output tile
+  double best = 0.;
+  p.rt = per;
+  for (int q = 1; q <= 8; ++q) {         // output tiles per workgroup
+    const int rt = q * per;
+    if (rt > 8 || !skinny_shape_ok(rt, p.nw, mt, gated)) continue;
+    const double g = (double)((tiles + q - 1) / q) * p.ks / 256.;
+    const double idle = g >= 1. ? ceil(g) / g : pow(g, -0.6);
+    const double cost = idle * (1. + 0.04 * (rt - 1) + 0.6 * (M / 16.) / rt);
+    if (best == 0. || cost < best * 0.999) {
+      best = cost;
+      p.rt = rt;
+    }
   }
   return p;
 }
 
 template <int MT, int RT, int NW, bool GATED, typename TO>
 static void launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, int ks, hipStream_t stream) {
-  constexpr int U = (RT + MT <= 2) ? 8 : (RT + MT <= 4 ? 4 : 2);
+  // steps of loads in flight, by the registers a wave has (16 waves: 128, 8 waves: 256)
+  constexpr int U = (RT + MT <= 2) ? 8 : (RT + MT <= (NW == 16 ? 4 : 7) ? 4 : 2);
   const int rows_per_wg = GATED ? 16 * (RT / 2) : 16 * RT;
   const int steps = (K + 31) / 32;
   const int sps = (steps + ks - 1) / ks;
@@ -230,7 +296,7 @@ static void launch_skinny_mt(int mt, const void* x, const void* w, void* y, int 
                              hipStream_t stream) {
   if (mt == 1) launch_skinny<1, RT, NW, GATED, TO>(x, w, y, M, N, K, ks, stream);
   else if (mt == 2) launch_skinny<2, RT, NW, GATED, TO>(x, w, y, M, N, K, ks, stream);
-  else launch_skinny<4, RT, NW, GATED, TO>(x, w, y, M, N, K, ks, stream);   // 33..64 rows
+  else if constexpr (RT <= 6) launch_skinny<4, RT, NW, GATED, TO>(x, w, y, M, N, K, ks, stream);   // 33..64 rows
 }
 
 }  // namespace xi
@@ -246,6 +312,11 @@ int xi_linear_skinny_max_rows() { return 64; }
 // its output when greater than 1).
 int xi_linear_skinny_slices(int N, int K, int gated, int allow_split) {
   return plan_skinny(1, N, K, gated != 0, allow_split != 0).ks;
+}
+
+// The row tiles of w a workgroup takes for these sizes (it does not change any sum).
+int xi_linear_skinny_row_tiles(int M, int N, int K, int gated, int allow_split) {
+  return plan_skinny(M, N, K, gated != 0, allow_split != 0).rt;
 }
 
 // x [M, K] bf16, w [N, K] bf16 -> y [M, N] in out_dtype (bf16 or float32); with
@@ -266,9 +337,9 @@ int xi_linear_skinny(const void* x, const void* w, void* y, int M, int N, int K,
   if (force_nw) p.nw = force_nw;
   if (force_rt) p.rt = force_rt;
   XI_CHECK(p.nw == 8 || p.nw == 16, "linear_skinny: %d waves (8 or 16)", p.nw);
-  XI_CHECK(gated ? (p.rt == 2 || p.rt == 4) : (p.rt == 1 || p.rt == 2 || p.rt == 4), "linear_skinny: %d row tiles", p.rt);
-  XI_CHECK(p.nw * p.rt <= 32, "linear_skinny: %d waves of %d row tiles do not fit in LDS", p.nw, p.rt);
   const int mt = (M + 15) / 16;
+  XI_CHECK(skinny_shape_ok(p.rt, p.nw, mt, gated != 0), "linear_skinny: no kernel of %d row tiles, %d waves for %d rows%s",
+           p.rt, p.nw, M, gated ? " (gated)" : "");
 #define XI_SK_PLAIN(RT, NW)                                                       \
   do {                                                                            \
     if (out_dtype == kBF16)                                                       \
@@ -280,14 +351,19 @@ int xi_linear_skinny(const void* x, const void* w, void* y, int M, int N, int K,
   if (gated) {
     if (p.nw == 16) XI_SK_GATED(2, 16);
     else if (p.rt == 2) XI_SK_GATED(2, 8);
-    else XI_SK_GATED(4, 8);
+    else if (p.rt == 4) XI_SK_GATED(4, 8);
+    else if (p.rt == 6) XI_SK_GATED(6, 8);
+    else XI_SK_GATED(8, 8);
   } else if (p.nw == 16) {
     if (p.rt == 1) XI_SK_PLAIN(1, 16);
     else XI_SK_PLAIN(2, 16);
   } else {
     if (p.rt == 1) XI_SK_PLAIN(1, 8);
     else if (p.rt == 2) XI_SK_PLAIN(2, 8);
-    else XI_SK_PLAIN(4, 8);
+    else if (p.rt == 3) XI_SK_PLAIN(3, 8);
+    else if (p.rt == 4) XI_SK_PLAIN(4, 8);
+    else if (p.rt == 6) XI_SK_PLAIN(6, 8);
+    else XI_SK_PLAIN(8, 8);
   }
 #undef XI_SK_PLAIN
 #undef XI_SK_GATED

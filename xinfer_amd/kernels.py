@@ -376,7 +376,9 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx
 
 SKINNY_MAX_ROWS = 64      # most rows the streaming kernel takes
 SKINNY_ROWS = 8           # up to this many rows it is faster than the vendor library (measured)
-SKINNY_GATED_ROWS = 16    # the same for the fused gate/up/silu form, which also saves a kernel
+SKINNY_SPLIT_ROWS = 64    # the same where the consumer takes partial sums over slices of K,
+SKINNY_SPLIT_FROM = 17    # which pays from this many rows on (fewer rows: the unsplit product)
+SKINNY_GATED_ROWS = 32    # the same for the fused gate/up/silu form, which also saves a kernel
 
 
 def linear_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
@@ -417,13 +419,19 @@ def linear_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dt
 def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
                 skinny_rows: int = SKINNY_ROWS, allow_split: bool = False) -> torch.Tensor:
     """bfloat16 x @ w.T with float32 accumulation, rounded once to `out_dtype` (bfloat16 or
-    float32).  Up to `skinny_rows` rows (decode): the hand-written streaming kernel.  More
+    float32).  Up to `skinny_rows` rows (decode): the hand-written streaming kernel, which with
+    `allow_split` may answer with float32 partial sums [slices, M, N] for a narrow output.  More
     rows: the vendor library (hipBLASLt through torch), which the reference's engine also
     uses for its matrix products."""
     _dev(x, w)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError("linear_bf16: operands must be bfloat16")
     out_dtype = out_dtype or torch.bfloat16
+    if (allow_split and x.shape[1] % 8 == 0 and x.shape[0] >= SKINNY_SPLIT_FROM
+            and int(lib().xi_linear_skinny_slices(w.shape[0], w.shape[1], 0, 1)) > 1):
+        skinny_rows = max(skinny_rows, SKINNY_SPLIT_ROWS)
+    else:
+        allow_split = False
     if 0 < x.shape[0] <= min(skinny_rows, SKINNY_MAX_ROWS) and x.shape[1] % 8 == 0:
         return linear_skinny(x, w, out_dtype, allow_split=allow_split)
     if out_dtype == torch.float32:

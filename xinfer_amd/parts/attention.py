@@ -92,4 +92,4 @@ class PagedAttention(Mixer):
             pos.interleaved if pos is not None else False,
             ctx.positions, slots, cache.k, cache.v, self.nq, self.nkv, self.d, v_transposed=vt)
         a = kernels.attention(q, cache.k, cache.v, ctx, cache.group, self.scale, self.window, v_transposed=vt)
-        return self.o(a, out_dtype=self.dtype)
+        return self.o(a, out_dtype=self.dtype, allow_split=True)     # the next norm adds the parts

@@ -53,4 +53,4 @@ class GatedMLP(FeedForward):
             m = kernels.linear_skinny(x, w, gated=True)        # gate, up and silu*mul in one pass
         else:
             m = kernels.silu_mul(self.gate_up(x, out_dtype=self.dtype))
-        return self.down(m, out_dtype=self.dtype)
+        return self.down(m, out_dtype=self.dtype, allow_split=True)  # the next norm adds the parts
