@@ -43,151 +43,24 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
-struct PagedKV {
-  const bf16* k;    // [pages, nkv, page, d]
-  const bf16* vt;   // [pages, nkv, d, page]
-  const int* bt;    // this sequence's block table
-  int page, nkv, d, kvh;
-};
-
-// Per-wave attention state for NQT column tiles and up to DT*16 output dims.
-template <int KC, int DT, int NQT>
-struct WaveAttn {
-  bf16x8 qb[NQT][KC];   // Q^T operands
-  f32x4 acc[DT][NQT];   // O^T accumulators
-  float m[NQT], l[NQT]; // running max (log2 domain) and per-lane partial sums
-  int qpos[NQT];        // position of this lane's query column (-1: no query)
-  int qlo[NQT];         // first key the query sees
-
-  __device__ __forceinline__ void init() {
-#pragma unroll
-    for (int ct = 0; ct < NQT; ++ct) {
-      m[ct] = -INFINITY;
-      l[ct] = 0.f;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) acc[dt][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
-  }
-
-  // q_row: pointer to this lane's query row (d elements) per column tile, or null.
-  __device__ __forceinline__ void load_q(const bf16* const* q_rows, int d, int j) {
-#pragma unroll
-    for (int ct = 0; ct < NQT; ++ct)
-#pragma unroll
-      for (int c = 0; c < KC; ++c) {
-        const int off = 32 * c + 8 * j;
-        qb[ct][c] = (q_rows[ct] && off < d) ? load8(q_rows[ct] + off) : zero8();
-      }
-  }
-
-  // Keys k_base .. k_base+31 (k_base a multiple of 32).  k_last: last key of the sequence
-  // that exists in the cache (addresses are clamped to it).  masked: some key of the step
-  // may be hidden from some query (else the mask arithmetic is skipped).
-  __device__ __forceinline__ void step(const PagedKV& kv, int k_base, int k_last, float scale_log2,
-                                       bool masked, int r, int j) {
-    const int d = kv.d;
-    // ---- K operands: tile 0 row r <-> key k_base + 8*(r/4) + r%4, tile 1 that + 4
-    int kgrp = k_base + 8 * (r >> 2);
-    if (kgrp > k_last) kgrp = k_last & ~7;
-    const int kpage = kv.bt[kgrp / kv.page];
-    const bf16* kp = kv.k + (((size_t)kpage * kv.nkv + kv.kvh) * kv.page + (kgrp % kv.page) + (r & 3)) * d;
-    bf16x8 ka[2][KC];
-#pragma unroll
-    for (int c = 0; c < KC; ++c) {
-      const int off = 32 * c + 8 * j;
-      if (off < d) {
-        ka[0][c] = load8(kp + off);
-        ka[1][c] = load8(kp + 4 * d + off);
-      } else {
-        ka[0][c] = zero8();
-        ka[1][c] = zero8();
-      }
-    }
-    // ---- V^T operands: row 16*dt + r, keys k_base + 8j .. +7
-    int vgrp = k_base + 8 * j;
-    if (vgrp > k_last) vgrp = k_last & ~7;
-    const int vpage = kv.bt[vgrp / kv.page];
-    const bf16* vp = kv.vt + (((size_t)vpage * kv.nkv + kv.kvh) * d + r) * kv.page + (vgrp % kv.page);
-    bf16x8 va[DT];
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) va[dt] = (16 * dt < d) ? load8(vp + (size_t)16 * dt * kv.page) : zero8();
-
-    bf16x8 pb[NQT];
-#pragma unroll
-    for (int ct = 0; ct < NQT; ++ct) {
-      f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int c = 0; c < KC; ++c) {
-        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[0][c], qb[ct][c], s0, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[1][c], qb[ct][c], s1, 0, 0, 0);
-      }
-      float s[8];
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        s[v] = s0[v] * scale_log2;
-        s[4 + v] = s1[v] * scale_log2;
-      }
-      if (masked) {
-        const int key0 = k_base + 8 * j;
-#pragma unroll
-        for (int v = 0; v < 8; ++v) {
-          const int key = key0 + v;
-          if (key > qpos[ct] || key < qlo[ct]) s[v] = -INFINITY;
-        }
-      }
-      float mx = s[0];
-#pragma unroll
-      for (int v = 1; v < 8; ++v) mx = fmaxf(mx, s[v]);
-      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-      const float m_new = fmaxf(m[ct], mx);
-      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-      const float corr = __builtin_amdgcn_exp2f(m[ct] - m_safe);
-      float psum = 0.f;
-#pragma unroll
-      for (int v = 0; v < 8; ++v) {
-        const float p = __builtin_amdgcn_exp2f(s[v] - m_safe);
-        psum += p;
-        pb[ct][v] = (__bf16)p;
-      }
-      l[ct] = l[ct] * corr + psum;
-      m[ct] = m_new;
-#pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        acc[dt][ct][0] *= corr;
-        acc[dt][ct][1] *= corr;
-        acc[dt][ct][2] *= corr;
-        acc[dt][ct][3] *= corr;
-      }
-    }
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-      for (int ct = 0; ct < NQT; ++ct)
-        acc[dt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt], pb[ct], acc[dt][ct], 0, 0, 0);
-  }
-
-  // Sum of a column's per-lane partial sums over the four lane groups.
-  __device__ __forceinline__ float total_l(int ct) const {
-    float t = l[ct] + __shfl_xor(l[ct], 16, kWave);
-    return t + __shfl_xor(t, 32, kWave);
-  }
-};
-
 // =====================================================================================
 // Decode: every sequence has one query token.  Workgroup (split, kv head, sequence): the
-// query heads of the kv group are the columns of one tile; the workgroup's four waves
-// take alternate 32-key steps of its chunk of `keys_per_wg` keys and merge through LDS.
-// Partial results (O * 2^-m normalised sums and m, l) go to a workspace, combined by the
-// second kernel in split order.
+// query heads of the kv group are the columns of one tile; each of the workgroup's four
+// waves takes a quarter of its chunk of `keys_per_wg` keys, 32 keys a step, and the waves
+// merge through LDS.  A wave keeps loads in flight all the time: the K operands of the next
+// step are asked for as soon as the scores of this one are computed, the V operands as soon
+// as this step's have been used, into the same registers.  The page numbers of the chunk
+// are read once into LDS, so that no step waits for the block table.  Partial results
+// (sums scaled by 2^-m, with m and l) go to a workspace, combined by the second kernel in
+// split order.
 // =====================================================================================
 template <int KC, int DT>
-__global__ __launch_bounds__(256) void attn_decode_split_kernel(
+__global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ vt_cache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ ctx_lens,
     float* __restrict__ part_o, float* __restrict__ part_ml, int max_splits, float scale_log2, int window,
     int page, int nq, int nkv, int d, int keys_per_wg) {
-  extern __shared__ float lds[];  // [4 waves][g][d] + [4][g][2]
+  extern __shared__ float lds[];  // [4 waves][g][d] + [4][g][2] + page numbers of the chunk
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, j = lane >> 4;
   const int split = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
@@ -199,34 +72,138 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(
   if (k_begin > pos) return;  // no keys for this split (the combine kernel knows)
   const int k_end = min(pos + 1, k_begin + keys_per_wg);  // exclusive
 
-  PagedKV kv{k_cache, vt_cache, block_tables + (size_t)seq * max_pages, page, nkv, d, kvh};
-  WaveAttn<KC, DT, 1> w;
-  w.init();
+  float* lds_o = lds;                                        // [4][g][d]
+  float* lds_ml = lds + 4 * g * d;                           // [4][g][2]
+  int* pages = reinterpret_cast<int*>(lds_ml + 4 * g * 2);   // [keys_per_wg / page + 1]
+  const int page_shift = __ffs(page) - 1;                    // the page size is a power of two
+  const int first_page = k_begin >> page_shift;
+  const int n_pages = ((k_end - 1) >> page_shift) - first_page + 1;
+  const int* bt = block_tables + (size_t)seq * max_pages;
+  for (int i = threadIdx.x; i < n_pages; i += 256) pages[i] = bt[first_page + i];
+
+  // this lane's query column: head kvh*g + r of the sequence, or none
   const bool col = r < g;
-  w.qpos[0] = col ? pos : -1;
-  w.qlo[0] = lo;
-  const bf16* q_rows[1] = {col ? q + ((size_t)seq * nq + kvh * g + r) * d : nullptr};
-  w.load_q(q_rows, d, j);
-  for (int kb = k_begin + 32 * wave; kb < k_end; kb += 128) {
-    const bool masked = (kb + 31 > pos) || (kb < lo);
-    w.step(kv, kb, pos, scale_log2, masked, r, j);
+  bf16x8 qb[KC];
+  {
+    const bf16* qrow = q + ((size_t)seq * nq + kvh * g + (col ? r : 0)) * d;
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+      const int off = 32 * c + 8 * j;
+      qb[c] = (col && off < d) ? load8(qrow + off) : zero8();
+    }
   }
-  const float lt = w.total_l(0);
-  float* lds_o = lds;                    // [4][g][d]
-  float* lds_ml = lds + 4 * g * d;       // [4][g][2]
+  __syncthreads();
+
+  // the four waves take alternate steps: the two halves of a 128-byte line of V^T (64 keys) are
+  // then asked for at about the same time
+  const int kb0 = k_begin + 32 * wave;
+  const int kb1 = k_end;
+
+  bf16x8 ka[2][KC], va[DT];
+  // K operands of keys k_base..k_base+31: tile 0 row r <-> key k_base + 8*(r/4) + r%4, tile 1
+  // that + 4.  Keys past the sequence are read from its last group of 8 (and masked).
+  auto load_k = [&](int k_base) {
+    int kgrp = k_base + 8 * (r >> 2);
+    if (kgrp > pos) kgrp = pos & ~7;
+    const int kpage = pages[(kgrp >> page_shift) - first_page];
+    const bf16* kp = k_cache + (((size_t)kpage * nkv + kvh) * page + (kgrp & (page - 1)) + (r & 3)) * d;
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+      const int off = 32 * c + 8 * j;
+      if (off < d) {
+        ka[0][c] = load8(kp + off);
+        ka[1][c] = load8(kp + 4 * d + off);
+      } else {
+        ka[0][c] = zero8();
+        ka[1][c] = zero8();
+      }
+    }
+  };
+  // V^T operands: row 16*dt + r, keys k_base + 8j .. +7
+  auto load_v = [&](int k_base) {
+    int vgrp = k_base + 8 * j;
+    if (vgrp > pos) vgrp = pos & ~7;
+    const int vpage = pages[(vgrp >> page_shift) - first_page];
+    const bf16* vp = vt_cache + (((size_t)vpage * nkv + kvh) * d + r) * page + (vgrp & (page - 1));
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) va[dt] = (16 * dt < d) ? load8(vp + (size_t)16 * dt * page) : zero8();
+  };
+
+  f32x4 acc[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;   // running max (log2 domain) and this lane's part of the sum
+  if (kb0 < kb1) {
+    load_k(kb0);
+    load_v(kb0);
+  }
+  for (int kb = kb0; kb < kb1; kb += 128) {
+    const bool more = kb + 128 < kb1;
+    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+      s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[0][c], qb[c], s0, 0, 0, 0);
+      s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[1][c], qb[c], s1, 0, 0, 0);
+    }
+    if (more) load_k(kb + 128);
+    float sc[8];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      sc[v] = s0[v] * scale_log2;
+      sc[4 + v] = s1[v] * scale_log2;
+    }
+    if (kb + 31 > pos || kb < lo) {   // some key of the step is hidden from the query
+      const int key0 = kb + 8 * j;
+#pragma unroll
+      for (int v = 0; v < 8; ++v) {
+        const int key = key0 + v;
+        if (key > pos || key < lo) sc[v] = -INFINITY;
+      }
+    }
+    float mx = sc[0];
+#pragma unroll
+    for (int v = 1; v < 8; ++v) mx = fmaxf(mx, sc[v]);
+    mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    const float m_new = fmaxf(m_run, mx);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float corr = __builtin_amdgcn_exp2f(m_run - m_safe);
+    float psum = 0.f;
+    bf16x8 pb;
+#pragma unroll
+    for (int v = 0; v < 8; ++v) {
+      const float p = __builtin_amdgcn_exp2f(sc[v] - m_safe);
+      psum += p;
+      pb[v] = (__bf16)p;
+    }
+    l_run = l_run * corr + psum;
+    m_run = m_new;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      acc[dt][0] *= corr;
+      acc[dt][1] *= corr;
+      acc[dt][2] *= corr;
+      acc[dt][3] *= corr;
+      acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt], pb, acc[dt], 0, 0, 0);
+    }
+    if (more) load_v(kb + 128);
+  }
+  // the column's sum over the four lane groups
+  float lt = l_run + __shfl_xor(l_run, 16, kWave);
+  lt += __shfl_xor(lt, 32, kWave);
   if (col) {
     if (j == 0) {
-      lds_ml[(wave * g + r) * 2] = w.m[0];
+      lds_ml[(wave * g + r) * 2] = m_run;
       lds_ml[(wave * g + r) * 2 + 1] = lt;
     }
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       if (16 * dt >= d) break;
       float* o = lds_o + ((size_t)wave * g + r) * d + 16 * dt + 4 * j;
-      o[0] = w.acc[dt][0][0];
-      o[1] = w.acc[dt][0][1];
-      o[2] = w.acc[dt][0][2];
-      o[3] = w.acc[dt][0][3];
+      o[0] = acc[dt][0];
+      o[1] = acc[dt][1];
+      o[2] = acc[dt][2];
+      o[3] = acc[dt][3];
     }
   }
   __syncthreads();
@@ -317,7 +294,7 @@ int xi_attention_decode_bf16(const void* q, const void* k_cache, const void* vt_
   XI_CHECK(keys_per_wg > 0 && keys_per_wg % 128 == 0, "attention_decode: keys_per_wg %d must be a multiple of 128", keys_per_wg);
   XI_CHECK(max_splits > 0 && nkv <= 65535 && n_seq <= 65535, "attention_decode: bad grid");
   XI_CHECK((size_t)max_splits * sizeof(float) <= 48 * 1024, "attention_decode: %d splits are too many", max_splits);
-  const size_t lds = (size_t)(4 * g * d + 4 * g * 2) * sizeof(float);
+  const size_t lds = (size_t)(4 * g * d + 4 * g * 2) * sizeof(float) + (size_t)(keys_per_wg / page + 2) * sizeof(int);
   XI_CHECK(lds <= 64 * 1024, "attention_decode: group %d x head_dim %d needs too much LDS", g, d);
   if (n_seq == 0) return 0;
   dim3 grid(max_splits, nkv, n_seq);
