@@ -45,9 +45,8 @@ __device__ __forceinline__ bf16x8 zero8() {
 
 // =====================================================================================
 // Decode: every sequence has one query token.  Workgroup (split, kv head, sequence): the
-// query heads of the kv group are the columns of one tile; each of the workgroup's four
-// waves takes a quarter of its chunk of `keys_per_wg` keys, 32 keys a step, and the waves
-// merge through LDS.  A wave keeps loads in flight all the time: the K operands of the next
+// query heads of the kv group are the columns of one tile; the workgroup's four waves take
+// alternate 32-key steps of its chunk of `keys_per_wg` keys and merge through LDS.  A wave keeps loads in flight all the time: the K operands of the next
 // step are asked for as soon as the scores of this one are computed, the V operands as soon
 // as this step's have been used, into the same registers.  The page numbers of the chunk
 // are read once into LDS, so that no step waits for the block table.  Partial results
