@@ -565,3 +565,148 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
     for what, steps in (("whole", harness.trace_whole(reqs)), ("mixed", harness.trace_mixed(reqs, 1, max_live=2)),
                         ("portions", harness.trace_portions(reqs))):
         harness.compare(run(steps), ref, harness.TOL["float32"], f"toy {what}")
+
+
+# ---- a toy feed-forward with routing and a toy position encoding, registered from here --------------------
+def test_toy_routed_feed_forward_and_position_encoding(tmp_path):
+    """Two more part kinds defined in this test: a feed-forward that routes every token to the
+    one of three gated experts whose router logit (float32) is largest, and a position encoding
+    that rotates interleaved pairs of a part of the head by the position divided by a factor.  An
+    architecture that uses them beside the built-in parts (the routed feed-forward in one layer,
+    a dense one in the other) is registered, written, loaded and stepped in every way of cutting,
+    without a change to the framework's files."""
+    from dataclasses import dataclass
+    from xinfer_amd.config.spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+    from xinfer_amd.engine import ModelRunner, load_model
+    from xinfer_amd.models import ModelFamily, register_architecture
+    from xinfer_amd.parts import FeedForward, PositionEncoding, register_feed_forward, register_position_encoding
+    from xinfer_amd.weights import TensorDecl, write_random_model
+    from xinfer_amd import kernels
+
+    E, H, I, D, ROT, FACTOR, THETA = 3, 40, 24, 16, 8, 4.0, 500.0
+
+    @register_feed_forward("top1_experts")
+    class Top1Experts(FeedForward):
+        def __init__(self, spec, dtype):
+            super().__init__(spec, dtype)
+            self.h, self.i, self.e = int(spec["hidden_size"]), int(spec["intermediate_size"]), int(spec["experts"])
+
+        @classmethod
+        def declare(cls, spec, prefix):
+            h, i = int(spec["hidden_size"]), int(spec["intermediate_size"])
+            out = [TensorDecl(f"{prefix}.router.weight", (int(spec["experts"]), h))]
+            for e in range(int(spec["experts"])):
+                out += [TensorDecl(f"{prefix}.experts.{e}.gate_proj.weight", (i, h)),
+                        TensorDecl(f"{prefix}.experts.{e}.up_proj.weight", (i, h)),
+                        TensorDecl(f"{prefix}.experts.{e}.down_proj.weight", (h, i))]
+            return out
+
+        def load(self, store, prefix, device):
+            self.router = store.get(f"{prefix}.router.weight", torch.float32, device)
+            self.w = [tuple(store.get(f"{prefix}.experts.{e}.{n}_proj.weight", torch.float32, device)
+                            for n in ("gate", "up", "down")) for e in range(self.e)]
+
+        def forward(self, x, ctx):
+            xf = x.float()
+            choice = kernels.gemm_tn(xf, self.router).argmax(dim=1)           # router logits in float32
+            out = torch.zeros_like(xf)
+            for e, (g, u, d) in enumerate(self.w):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel():
+                    xe = xf[rows].contiguous()
+                    a = kernels.silu_mul(torch.cat([kernels.gemm_tn(xe, g), kernels.gemm_tn(xe, u)], dim=1).contiguous())
+                    out[rows] = kernels.gemm_tn(a, d)
+            return out.to(self.dtype)
+
+    @register_position_encoding("scaled_pairs")
+    class ScaledPairs(PositionEncoding):
+        """What the attention mixer reads of a position encoding: `cos` and `sin`
+        [max_positions, rotary_dim / 2] float32, `rotary_dim`, `interleaved`."""
+
+        def __init__(self, spec, dtype):
+            super().__init__(spec, dtype)
+            self.rotary_dim, self.interleaved = int(spec["rotary_dim"]), True
+            self.theta, self.factor, self.max_positions = float(spec["theta"]), float(spec["factor"]), int(spec["max_positions"])
+            self.cos = self.sin = None
+
+        def load(self, store, prefix, device):
+            inv = 1.0 / (self.theta ** (torch.arange(0, self.rotary_dim, 2, dtype=torch.float64) / self.rotary_dim))
+            ang = (torch.arange(self.max_positions, dtype=torch.float64) / self.factor)[:, None] * inv[None, :]
+            self.cos, self.sin = ang.cos().float().contiguous().to(device), ang.sin().float().contiguous().to(device)
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        vocab_size: int
+        architecture: str = "ToyRoutedForCausalLM"
+
+        @classmethod
+        def from_dict(cls, raw, where="config.json"):
+            return cls(int(raw["vocab_size"]))
+
+        def to_dict(self):
+            return {"architectures": [self.architecture], "vocab_size": self.vocab_size}
+
+    def toy_spec(cfg):
+        norm = PartSpec("rmsnorm", dict(dim=H, eps=1e-5))
+        pos = PartSpec("scaled_pairs", dict(rotary_dim=ROT, theta=THETA, factor=FACTOR, max_positions=256))
+        attn = PartSpec("attention", dict(hidden_size=H, num_heads=3, num_kv_heads=1, head_dim=D, qk_norm=False,
+                                          window=None, position=pos, scale=0.3))
+        routed = PartSpec("top1_experts", dict(hidden_size=H, intermediate_size=I, experts=E))
+        dense = PartSpec("gated_mlp", dict(hidden_size=H, intermediate_size=I, activation="silu"))
+        norms = {"input_layernorm": norm, "post_attention_layernorm": norm}
+        layers = (LayerSpec("model.layers.0", "prenorm", attn, routed, norms),
+                  LayerSpec("model.layers.1", "prenorm", attn, dense, norms))
+        return ModelSpec(
+            architecture=cfg.architecture, vocab_size=cfg.vocab_size, hidden_size=H, max_positions=256,
+            embedding=PartSpec("embedding", dict(name="model.embed_tokens.weight", vocab_size=cfg.vocab_size, dim=H)),
+            layers=layers, schedule=(ScheduleEntry(0), ScheduleEntry(1)),
+            final_norm=PartSpec("rmsnorm", dict(dim=H, eps=1e-5, name="model.norm.weight")),
+            head=PartSpec("lm_head", dict(name="lm_head.weight", tied=False, vocab_size=cfg.vocab_size, dim=H)))
+
+    register_architecture("ToyRoutedForCausalLM", ModelFamily("toy_routed", ToyConfig, toy_spec))
+    d = write_random_model(str(tmp_path / "toy"), {"architectures": ["ToyRoutedForCausalLM"], "vocab_size": 61},
+                           seed=5, linear_std=0.15)
+    model = load_model(d, "float32", DEV)
+
+    # the same model written out plainly, whole sequences, float64
+    W = {k: v.double() for k, v in plain.read_weights(d).items()}
+    inv = 1.0 / (THETA ** (torch.arange(0, ROT, 2, dtype=torch.float64) / ROT))
+
+    def rotate(x, T):      # x [T, heads, D]: pairs (2i, 2i+1) of the first ROT dims, angle = p / FACTOR * inv[i]
+        ang = (torch.arange(T, dtype=torch.float64) / FACTOR)[:, None] * inv[None, :]
+        c, s = ang.cos()[:, None, :], ang.sin()[:, None, :]
+        y = x.clone()
+        a, b = x[..., 0:ROT:2], x[..., 1:ROT:2]
+        y[..., 0:ROT:2], y[..., 1:ROT:2] = a * c - b * s, a * s + b * c
+        return y
+
+    used = set()
+
+    def toy_logits(ids):
+        T = len(ids)
+        x = W["model.embed_tokens.weight"][torch.tensor(ids)]
+        for i in range(2):
+            p = f"model.layers.{i}"
+            h = plain.rms_norm(x, W[f"{p}.input_layernorm.weight"], 1e-5)
+            q = rotate((h @ W[f"{p}.self_attn.q_proj.weight"].T).reshape(T, 3, D), T)
+            k = rotate((h @ W[f"{p}.self_attn.k_proj.weight"].T).reshape(T, 1, D), T)
+            v = (h @ W[f"{p}.self_attn.v_proj.weight"].T).reshape(T, 1, D)
+            r = x + plain.attention(q, k, v, scale=0.3).reshape(T, 3 * D) @ W[f"{p}.self_attn.o_proj.weight"].T
+            h = plain.rms_norm(r, W[f"{p}.post_attention_layernorm.weight"], 1e-5)
+            if i == 0:
+                choice = (h @ W[f"{p}.mlp.router.weight"].T).argmax(dim=1)
+                used.update(choice.tolist())
+                m = torch.stack([plain.mlp_block(h[t:t + 1], W, f"{p}.mlp.experts.{int(choice[t])}")[0] for t in range(T)])
+            else:
+                m = plain.mlp_block(h, W, f"{p}.mlp")
+            x = r + m
+        return (plain.rms_norm(x, W["model.norm.weight"], 1e-5) @ W["lm_head.weight"].T).float()
+
+    rng = random.Random(10)
+    reqs = {f"q{i}": harness.random_prompt(rng, n, 61) for i, n in enumerate([23, 41, 9, 30])}
+    ref = {rid: toy_logits(t) for rid, t in reqs.items()}
+    assert used == set(range(E))           # every expert takes part
+    for what, steps in (("whole", harness.trace_whole(reqs)), ("mixed", harness.trace_mixed(reqs, 1, max_live=2)),
+                        ("portions", harness.trace_portions(reqs))):
+        runner = ModelRunner(model, page_size=8, num_pages=14, max_requests=2)
+        harness.compare(harness.replay(runner, steps), ref, harness.TOL["float32"], f"toy routed {what}")

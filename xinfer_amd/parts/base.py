@@ -137,7 +137,10 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
-    pass
+    """What a mixer reads of it is between the two.  The built-in attention mixer reads a
+    rotation: `cos` and `sin`, float32 tables [max_positions, rotary_dim / 2] on the device
+    (made in `load`), `rotary_dim` (even, at most the head size) and `interleaved` (pairs
+    (2i, 2i+1) instead of (i, i + rotary_dim / 2)); its kernels apply them to q and k."""
 
 
 class Block:
