@@ -195,6 +195,51 @@ def test_linear_skinny_gated(M, I, K):
         assert torch.equal(y, outs[1])     # the row tiles of a workgroup do not change a sum
 
 
+@pytest.mark.parametrize("M", [1, 5, 16])
+@pytest.mark.parametrize("N,K,N2", [(4096, 4096, 12288), (320, 136, 176), (1000, 1408, 509), (102 * 8, 96, 77)])
+def test_linear_folded_norm(M, N, K, N2):
+    """A norm between two products folded into them: the first adds into the float32 stream and
+    hands on round(stream * g) with the rows' sums of squares in parts, the second scales its rows.
+    Against add + RMSNorm + product in float64; the stream itself to float32 rounding."""
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(13)
+    x = _rand((M, K), torch.bfloat16, g)
+    w1 = _rand((N, K), torch.bfloat16, g, 0.05)
+    resid = _rand((M, N), torch.float32, g, 2.0)
+    gn = 1 + 0.2 * torch.randn(N, generator=g)
+    eps = 1e-6
+    r_dev = resid.to(DEV).clone()
+    xg, ss = kernels.linear_fold_out(x.to(DEV), w1.to(DEV), r_dev, gn.to(DEV))
+    want_r = resid.double() + x.double() @ w1.double().T
+    assert (r_dev.cpu().double() - want_r).abs().max() / want_r.abs().max() < 1e-5
+    assert ((ss.cpu().double().sum(1) - (want_r ** 2).sum(1)).abs() / (want_r ** 2).sum(1)).max() < 1e-5
+    normed = plain.rms_norm(want_r, gn.double(), eps)
+    for gated in (False, True):
+        w2 = _rand(((2 if gated else 1) * N2, N), torch.bfloat16, g, 0.05)
+        y = kernels.linear_fold_in(xg, ss, eps, w2.to(DEV), gated=gated)
+        full = normed @ w2.double().T
+        ref = plain.swiglu(full[:, :N2], full[:, N2:]) if gated else full
+        err = (y.cpu().double() - ref).abs().max() / ref.abs().max()
+        assert y.shape == (M, N2) and err < 2.0 ** -6, (gated, err)
+    y32 = kernels.linear_fold_in(xg, ss, eps, w2[:N2].contiguous().to(DEV), out_dtype=torch.float32)
+    ref = normed @ w2[:N2].double().T
+    assert y32.dtype == torch.float32 and (y32.cpu().double() - ref).abs().max() / ref.abs().max() < 2.0 ** -6
+
+
+def test_linear_folded_norm_refuses():
+    from xinfer_amd import kernels
+    x = torch.zeros((17, 64), dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros((32, 64), dtype=torch.bfloat16, device=DEV)
+    r = torch.zeros((17, 32), dtype=torch.float32, device=DEV)
+    gw = torch.ones(32, device=DEV)
+    with pytest.raises(kernels.KernelError, match="1..16"):
+        kernels.linear_fold_out(x, w, r, gw)
+    with pytest.raises(kernels.KernelError, match="do not match"):
+        kernels.linear_fold_out(x[:4].contiguous(), w, r[:3].contiguous(), gw)
+    with pytest.raises(kernels.KernelError, match="256 parts"):
+        kernels.linear_fold_in(x[:4].contiguous(), torch.zeros((4, 300), device=DEV), 1e-6, w)
+
+
 def test_linear_skinny_refuses():
     from xinfer_amd import kernels
     x = torch.zeros((65, 64), dtype=torch.bfloat16, device=DEV)

@@ -45,12 +45,33 @@ __device__ __forceinline__ int tile_row0(int t, int n0, int N) {
   return t < RT / 2 ? n0 + 16 * t : N + n0 + 16 * (t - RT / 2);
 }
 
-template <int MT, int RT, int NW, int U, bool GATED, typename TO>
+// A norm folded into the two products around it (few rows, MT = 1).  The product before the
+// norm (MODE 1, kFoldOut) adds its result into the float32 residual stream, writes
+// xg = round(stream * g) with the norm's weight g, and the sum of squares of its part of every
+// row, one per workgroup.  The product after the norm (MODE 2, kFoldIn) takes xg as its x and
+// multiplies each row of its result by rsqrt(sum of the parts / H + eps): the same value as
+// norming first, up to where the one rounding to bfloat16 happens, and without the norm's own
+// kernel between two kernels that stream weights.
+struct SkinnyFold {
+  float* resid;         // kFoldOut: [M, N] float32, updated in place
+  const float* g;       // kFoldOut: [N] weight of the norm that follows
+  bf16* xg;             // kFoldOut: [M, N]
+  float* ss_out;        // kFoldOut: [M, gridDim.x]
+  const float* ss_in;   // kFoldIn: [M, parts]
+  int parts;            // kFoldIn
+  float eps;            // kFoldIn
+  float inv_h;          // kFoldIn: 1 / length of the normed rows
+};
+constexpr int kFoldNone = 0, kFoldOut = 1, kFoldIn = 2;
+
+template <int MT, int RT, int NW, int U, bool GATED, typename TO, int MODE>
 __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16* __restrict__ x,
                                                                 const bf16* __restrict__ w,
                                                                 TO* __restrict__ y, int M, int N, int K,
-                                                                int steps_per_slice) {
+                                                                int steps_per_slice, SkinnyFold fold) {
   static_assert(!GATED || RT % 2 == 0, "the gated form pairs gate tiles with up tiles");
+  static_assert(MODE == kFoldNone || (MT == 1 && NW == 8), "a folded norm: up to 16 rows, 8 waves");
+  static_assert(MODE != kFoldOut || !GATED, "the product before a norm is a plain one");
   // The waves' sums are merged through LDS a chunk of PC output tiles (gated: pairs of a gate
   // and an up tile) at a time, so that the buffer stays within 64 KB whatever RT and MT are.
   constexpr int H = NW / 2;                      // waves whose sums are left after the first round
@@ -59,8 +80,21 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16* __re
   static_assert(H * TP * MT <= 64, "one output tile's sums must fit in 64 KB of LDS");
   constexpr int PC = (64 / (H * TP * MT)) < PAIRS ? (64 / (H * TP * MT)) : PAIRS;
   __shared__ float red[H * PC * TP * MT * 256];
+  static_assert(MODE != kFoldOut || PC == PAIRS, "the product before a norm stores in one pass");
+  __shared__ float fold_lds[MODE == kFoldOut ? 16 * 16 * RT : 16];   // squares [token][n], or 1/rms [token]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, j = lane >> 4;
+  // kFoldIn: 32 threads per row add up the parts of its sum of squares; the loads start now, the
+  // sum is taken after the products
+  float ss_mine[8];
+  if constexpr (MODE == kFoldIn) {
+    const int token = threadIdx.x >> 5, sub = threadIdx.x & 31;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int p = sub + 32 * i;
+      ss_mine[i] = (token < M && p < fold.parts) ? fold.ss_in[(size_t)token * fold.parts + p] : 0.f;
+    }
+  }
   const int n0 = blockIdx.x * (GATED ? 16 * (RT / 2) : 16 * RT);
   const int ks = blockIdx.y;
   const int w_rows = GATED ? 2 * N : N;
@@ -178,6 +212,14 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16* __re
   // token r, features 4j..4j+3.  Slot of (wave wv, output tile q of the chunk, part tp, token
   // tile m): ((wv * PC + q) * TP + tp) * MT + m.
   TO* yk = y + (size_t)ks * M * N;   // this slice's partial sums (ks is 0 without slices)
+  if constexpr (MODE == kFoldIn) {   // read after the barriers of the merge below
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) t += ss_mine[i];
+#pragma unroll
+    for (int o = 16; o; o >>= 1) t += __shfl_xor(t, o, kWave);
+    if ((threadIdx.x & 31) == 0) fold_lds[threadIdx.x >> 5] = rsqrtf(t * fold.inv_h + fold.eps);
+  }
 #pragma unroll
   for (int p0 = 0; p0 < PAIRS; p0 += PC) {
     if (p0 > 0) __syncthreads();     // the chunk before has been read
@@ -224,8 +266,32 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16* __re
         a0 += red[(((wv * PC + q) * TP) * MT + m) * 256 + e];
         if (GATED) a1 += red[(((wv * PC + q) * TP + 1) * MT + m) * 256 + e];
       }
-      if (token < M && n < N)
-        yk[(size_t)token * N + n] = from_float<TO>(GATED ? a0 / (1.f + __expf(-a0)) * a1 : a0);
+      if constexpr (MODE == kFoldIn) {
+        const float inv = fold_lds[token];
+        a0 *= inv;
+        a1 *= inv;
+      }
+      if constexpr (MODE == kFoldOut) {
+        float sq = 0.f;
+        if (token < M && n < N) {
+          const float rr = fold.resid[(size_t)token * N + n] + a0;
+          fold.resid[(size_t)token * N + n] = rr;
+          fold.xg[(size_t)token * N + n] = from_float<bf16>(rr * fold.g[n]);
+          sq = rr * rr;
+        }
+        fold_lds[token * (16 * RT) + (n - n0)] = sq;
+      } else {
+        if (token < M && n < N)
+          yk[(size_t)token * N + n] = from_float<TO>(GATED ? a0 / (1.f + __expf(-a0)) * a1 : a0);
+      }
+    }
+  }
+  if constexpr (MODE == kFoldOut) {   // a row's squares summed in the order of n
+    __syncthreads();
+    if (threadIdx.x < 16 && (int)threadIdx.x < M) {
+      float t = 0.f;
+      for (int i = 0; i < 16 * RT; ++i) t += fold_lds[threadIdx.x * (16 * RT) + i];
+      fold.ss_out[(size_t)threadIdx.x * gridDim.x + blockIdx.x] = t;
     }
   }
 }
@@ -279,16 +345,32 @@ static SkinnyPlan plan_skinny(int M, int N, int K, bool gated, bool allow_split)
   return p;
 }
 
-template <int MT, int RT, int NW, bool GATED, typename TO>
-static void launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, int ks, hipStream_t stream) {
+template <int MT, int RT, int NW, bool GATED, typename TO, int MODE = kFoldNone>
+static void launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, int ks, hipStream_t stream,
+                          const SkinnyFold& fold = SkinnyFold{}) {
   // steps of loads in flight, by the registers a wave has (16 waves: 128, 8 waves: 256)
   constexpr int U = (RT + MT <= 2) ? 8 : (RT + MT <= (NW == 16 ? 4 : 7) ? 4 : 2);
   const int rows_per_wg = GATED ? 16 * (RT / 2) : 16 * RT;
   const int steps = (K + 31) / 32;
   const int sps = (steps + ks - 1) / ks;
   dim3 grid((unsigned)((N + rows_per_wg - 1) / rows_per_wg), (unsigned)ks);
-  linear_skinny_kernel<MT, RT, NW, U, GATED, TO><<<grid, NW * 64, 0, stream>>>(
-      (const bf16*)x, (const bf16*)w, (TO*)y, M, N, K, sps);
+  linear_skinny_kernel<MT, RT, NW, U, GATED, TO, MODE><<<grid, NW * 64, 0, stream>>>(
+      (const bf16*)x, (const bf16*)w, (TO*)y, M, N, K, sps, fold);
+}
+
+// The folded forms exist for up to 16 rows and 8 waves; rt as the plan says.
+template <bool GATED, typename TO, int MODE>
+static bool launch_skinny_fold(int rt, const void* x, const void* w, void* y, int M, int N, int K, hipStream_t stream,
+                               const SkinnyFold& fold) {
+  if constexpr (!GATED) {
+    if (rt == 1) { launch_skinny<1, 1, 8, false, TO, MODE>(x, w, y, M, N, K, 1, stream, fold); return true; }
+    if (rt == 3) { launch_skinny<1, 3, 8, false, TO, MODE>(x, w, y, M, N, K, 1, stream, fold); return true; }
+  }
+  if (rt == 2) { launch_skinny<1, 2, 8, GATED, TO, MODE>(x, w, y, M, N, K, 1, stream, fold); return true; }
+  if (rt == 4) { launch_skinny<1, 4, 8, GATED, TO, MODE>(x, w, y, M, N, K, 1, stream, fold); return true; }
+  if (rt == 6) { launch_skinny<1, 6, 8, GATED, TO, MODE>(x, w, y, M, N, K, 1, stream, fold); return true; }
+  if (rt == 8) { launch_skinny<1, 8, 8, GATED, TO, MODE>(x, w, y, M, N, K, 1, stream, fold); return true; }
+  return false;
 }
 
 template <int RT, int NW, bool GATED, typename TO>
@@ -317,6 +399,53 @@ int xi_linear_skinny_slices(int N, int K, int gated, int allow_split) {
 // The row tiles of w a workgroup takes for these sizes (it does not change any sum).
 int xi_linear_skinny_row_tiles(int M, int N, int K, int gated, int allow_split) {
   return plan_skinny(M, N, K, gated != 0, allow_split != 0).rt;
+}
+
+// The product before a norm, for M <= 16 rows: resid [M, N] float32 += x [M, K] @ w [N, K]^T;
+// xg [M, N] bf16 = round(resid * g) with the norm's weight g [N]; ss [M, parts] float32 = the
+// sum of squares of each row of resid, in parts = xi_linear_skinny_fold_parts(M, N, K), one per
+// workgroup.  The product after the norm then takes xg and ss (xi_linear_skinny_fold_in).
+int xi_linear_skinny_fold_parts(int M, int N, int K) {
+  const SkinnyPlan p = plan_skinny(M, N, K, false, false);
+  return (N + 16 * p.rt - 1) / (16 * p.rt);
+}
+
+int xi_linear_skinny_fold_out(const void* x, const void* w, int M, int N, int K, float* resid, const float* g, void* xg,
+                              float* ss, hipStream_t stream) {
+  XI_CHECK(M > 0 && M <= 16 && N > 0 && K > 0 && K % 8 == 0, "linear_skinny_fold_out: bad sizes M=%d N=%d K=%d", M, N, K);
+  const SkinnyPlan p = plan_skinny(M, N, K, false, false);
+  SkinnyFold f{};
+  f.resid = resid;
+  f.g = g;
+  f.xg = (bf16*)xg;
+  f.ss_out = ss;
+  const bool ok = launch_skinny_fold<false, bf16, kFoldOut>(p.rt, x, w, nullptr, M, N, K, stream, f);
+  XI_CHECK(ok, "linear_skinny_fold_out: no kernel of %d row tiles", p.rt);
+  XI_LAUNCH_CHECK("linear_skinny_fold_out");
+  return 0;
+}
+
+// The product after a norm whose first half ran in xi_linear_skinny_fold_out: xg [M, K] bf16,
+// ss [M, parts] float32 (parts <= 256), y [M, N] = (xg @ w^T) * rsqrt(sum(ss[row]) / K + eps) per
+// row, rounded once; gated as in xi_linear_skinny (then y is bfloat16).
+int xi_linear_skinny_fold_in(const void* xg, const void* w, void* y, int M, int N, int K, int out_dtype, int gated,
+                             const float* ss, int parts, float eps, hipStream_t stream) {
+  XI_CHECK(M > 0 && M <= 16 && N > 0 && K > 0 && K % 8 == 0, "linear_skinny_fold_in: bad sizes M=%d N=%d K=%d", M, N, K);
+  XI_CHECK(parts > 0 && parts <= 256, "linear_skinny_fold_in: %d parts of a row's sum of squares (at most 256)", parts);
+  XI_CHECK(out_dtype == kBF16 || (out_dtype == kF32 && !gated), "linear_skinny_fold_in: output dtype %d", out_dtype);
+  const SkinnyPlan p = plan_skinny(M, N, K, gated != 0, false);
+  SkinnyFold f{};
+  f.ss_in = ss;
+  f.parts = parts;
+  f.eps = eps;
+  f.inv_h = 1.f / (float)K;
+  bool ok;
+  if (gated) ok = launch_skinny_fold<true, bf16, kFoldIn>(p.rt, xg, w, y, M, N, K, stream, f);
+  else if (out_dtype == kBF16) ok = launch_skinny_fold<false, bf16, kFoldIn>(p.rt, xg, w, y, M, N, K, stream, f);
+  else ok = launch_skinny_fold<false, float, kFoldIn>(p.rt, xg, w, y, M, N, K, stream, f);
+  XI_CHECK(ok, "linear_skinny_fold_in: no kernel of %d row tiles", p.rt);
+  XI_LAUNCH_CHECK("linear_skinny_fold_in");
+  return 0;
 }
 
 // x [M, K] bf16, w [N, K] bf16 -> y [M, N] in out_dtype (bf16 or float32); with

@@ -107,13 +107,21 @@ class CausalLM:
         """ids int32 [T]; caches: layer index -> the cache that layer owns; want_rows int32
         [R].  Returns float32 logits [R, vocab]."""
         stream = Stream(self.embedding.forward(ids), None)
-        for e in self.spec.schedule:
+        schedule = self.spec.schedule
+        for i, e in enumerate(schedule):
             owner = e.layer if e.cache_of is None else e.cache_of
             c = caches.get(owner)
             if c is None:
                 c = LayerCache()
             elif e.cache_of is not None:
                 c = LayerCache(c.group, c.k, c.v, c.state, write=False)
-            stream = self.blocks[e.layer].forward(stream, ctx, c)
+            blk = self.blocks[e.layer]
+            if getattr(blk, "folds", False):
+                # the block that runs next may let this one half do its first norm
+                nxt = self.blocks[schedule[i + 1].layer] if i + 1 < len(schedule) else None
+                next_norm = nxt.first_norm() if getattr(nxt, "folds", False) else None
+                stream = blk.forward(stream, ctx, c, next_norm=next_norm)
+            else:
+                stream = blk.forward(stream, ctx, c)
         h = self.final_norm.forward(stream.resid, stream.pending, self.dtype, rows=want_rows)
         return self.head.forward(h)

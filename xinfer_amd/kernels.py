@@ -416,6 +416,70 @@ def linear_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dt
     return out
 
 
+FOLD_ROWS = 16            # most rows of the products that carry a folded norm between them
+FOLD_PARTS = 256          # most parts of a row's sum of squares the product after the norm adds up
+
+
+def linear_fold_parts(M: int, N: int, K: int) -> int:
+    """The parts in which `linear_fold_out` hands on each row's sum of squares for these sizes."""
+    return int(lib().xi_linear_skinny_fold_parts(int(M), int(N), int(K)))
+
+
+def linear_fold_out(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, norm_weight: torch.Tensor):
+    """The product before an RMSNorm, for up to FOLD_ROWS rows: resid [M, N] float32 += x [M, K] @
+    w [N, K]^T in place; returns (xg, ss): xg [M, N] bfloat16 = round(resid * norm_weight), ss
+    [M, parts] float32 the sums of squares of the rows of resid in parts.  `linear_fold_in` is the
+    product after the norm; between them no norm kernel runs."""
+    _dev(x, w, resid, norm_weight)
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError("linear_fold_out: operands must be bfloat16")
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
+        raise KernelError(f"linear_fold_out: x {tuple(x.shape)} and w {tuple(w.shape)} do not match")
+    M, K = x.shape
+    N = w.shape[0]
+    if not (0 < M <= FOLD_ROWS) or K % 8:
+        raise KernelError(f"linear_fold_out: M={M} must be 1..{FOLD_ROWS} and K={K} a multiple of 8")
+    _want(resid, torch.float32, "linear_fold_out: resid")
+    _want(norm_weight, torch.float32, "linear_fold_out: norm weight")
+    if tuple(resid.shape) != (M, N) or tuple(norm_weight.shape) != (N,) or not resid.is_contiguous():
+        raise KernelError(f"linear_fold_out: resid {tuple(resid.shape)} / norm weight {tuple(norm_weight.shape)} "
+                          f"do not match [M={M}, N={N}]")
+    parts = linear_fold_parts(M, N, K)
+    xg = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    ss = torch.empty((M, parts), dtype=torch.float32, device=x.device)
+    _ok(lib().xi_linear_skinny_fold_out(_p(x), _p(w), M, N, K, _p(resid), _p(norm_weight), _p(xg), _p(ss), _stream()))
+    return xg, ss
+
+
+def linear_fold_in(xg: torch.Tensor, ss: torch.Tensor, eps: float, w: torch.Tensor,
+                   out_dtype: Optional[torch.dtype] = None, gated: bool = False) -> torch.Tensor:
+    """The product after an RMSNorm whose first half `linear_fold_out` did: (xg @ w^T) with each
+    row multiplied by rsqrt(sum(ss[row]) / K + eps), one rounding; `gated` as in `linear_skinny`."""
+    _dev(xg, ss, w)
+    if xg.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError("linear_fold_in: operands must be bfloat16")
+    if xg.dim() != 2 or w.dim() != 2 or xg.shape[1] != w.shape[1]:
+        raise KernelError(f"linear_fold_in: x {tuple(xg.shape)} and w {tuple(w.shape)} do not match")
+    M, K = xg.shape
+    N = w.shape[0]
+    if gated:
+        if N % 2:
+            raise KernelError("linear_fold_in: a gated weight must be [2N, K]")
+        N //= 2
+    _want(ss, torch.float32, "linear_fold_in: ss")
+    if not (0 < M <= FOLD_ROWS) or K % 8 or ss.dim() != 2 or ss.shape[0] != M or not (0 < ss.shape[1] <= 256) \
+            or not ss.is_contiguous():
+        raise KernelError(f"linear_fold_in: M={M} (1..{FOLD_ROWS}), K={K} (multiple of 8), ss {tuple(ss.shape)} "
+                          f"([M, up to 256 parts])")
+    out_dtype = out_dtype or torch.bfloat16
+    if gated and out_dtype != torch.bfloat16:
+        raise KernelError("linear_fold_in: the gated form writes bfloat16")
+    y = torch.empty((M, N), dtype=out_dtype, device=xg.device)
+    _ok(lib().xi_linear_skinny_fold_in(_p(xg), _p(w), _p(y), M, N, K, _code(y, "linear_fold_in"), int(bool(gated)),
+                                       _p(ss), int(ss.shape[1]), ctypes.c_float(eps), _stream()))
+    return y
+
+
 def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
                 skinny_rows: int = SKINNY_ROWS, allow_split: bool = False) -> torch.Tensor:
     """bfloat16 x @ w.T with float32 accumulation, rounded once to `out_dtype` (bfloat16 or

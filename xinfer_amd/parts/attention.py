@@ -79,7 +79,11 @@ class PagedAttention(Mixer):
         return KVNeed(self.nkv, self.d, self.window, v_transposed=self.dtype == torch.bfloat16)
 
     # ---- step ----------------------------------------------------------------
-    def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> torch.Tensor:
+    takes_sink = True
+    takes_folded = True
+
+    def forward(self, x, ctx: StepContext, cache: LayerCache, sink=None):
+        """`x`: rows or a `Folded`; `sink`: see `Part.takes_sink`."""
         qkv = self.qkv(x, out_dtype=self.dtype)
         pos = self.position
         slots = ctx.slots[cache.group] if cache.write else ctx.no_slots
@@ -92,4 +96,4 @@ class PagedAttention(Mixer):
             pos.interleaved if pos is not None else False,
             ctx.positions, slots, cache.k, cache.v, self.nq, self.nkv, self.d, v_transposed=vt)
         a = kernels.attention(q, cache.k, cache.v, ctx, cache.group, self.scale, self.window, v_transposed=vt)
-        return self.o(a, out_dtype=self.dtype, allow_split=True)     # the next norm adds the parts
+        return self.o(a, out_dtype=self.dtype, allow_split=True, sink=sink)     # the next norm adds the parts

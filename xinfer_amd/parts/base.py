@@ -87,12 +87,39 @@ class StepContext:
 
 
 @dataclass
+class NormSink:
+    """Given to the part that runs before a norm: "add your result into `resid` yourself and
+    prepare `norm`'s input".  A part that can (its last product, for few rows) answers with a
+    `Folded`; it may always answer with its plain result instead."""
+    resid: torch.Tensor                        # float32 [T, H], the residual stream
+    norm: "Norm"
+
+
+@dataclass
+class Folded:
+    """Rows whose norm is half done by the product before it: the stream already holds the sum,
+    `xg` = round(stream * norm.weight) [T, H], `ss` [T, parts] float32 the parts of each row's
+    sum of squares.  The product after the norm takes it in place of normed rows and scales its
+    own rows by rsqrt(sum(ss) / H + eps) (`kernels.linear_fold_in`)."""
+    xg: torch.Tensor
+    ss: torch.Tensor
+    norm: "Norm"
+
+    def rows(self, dtype: torch.dtype) -> torch.Tensor:
+        """The normed rows themselves, for a consumer without the folded product."""
+        inv = torch.rsqrt(self.ss.sum(dim=1) / self.xg.shape[1] + self.norm.eps)
+        return (self.xg.float() * inv[:, None]).to(dtype)
+
+
+@dataclass
 class Stream:
     """The residual stream between blocks: `resid` float32 [T, H], and a branch output
     `pending` that has not been added to it yet (the next norm adds it in the same
-    kernel that norms)."""
+    kernel that norms), or `folded`: the branch output is already added and the next
+    norm (`folded.norm`) half done."""
     resid: torch.Tensor
     pending: Optional[torch.Tensor] = None
+    folded: Optional[Folded] = None
 
 
 class Part:
@@ -101,6 +128,13 @@ class Part:
     # decode step can be recorded once as a HIP graph and replayed.  Parts that do not say so
     # keep the whole model on the launch-by-launch path.
     graph_safe = False
+    # Folding a norm into the products around it (see `Folded`): a mixer or feed-forward whose
+    # `forward` takes a keyword `sink: Optional[NormSink]` says `takes_sink`; one whose `forward`
+    # takes a `Folded` in place of its input rows says `takes_folded`; a norm that can be folded
+    # (a weight vector `weight` in float32, `eps`, `dim`) says `foldable`.
+    takes_sink = False
+    takes_folded = False
+    foldable = False
 
     def __init__(self, spec: PartSpec, dtype: torch.dtype):
         self.spec = spec

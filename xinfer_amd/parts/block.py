@@ -14,7 +14,7 @@ import torch
 
 from ..config.spec import LayerSpec
 from ..weights.store import TensorDecl, WeightStore
-from .base import (Block, KVNeed, LayerCache, StateNeed, StepContext, Stream,
+from .base import (Block, Folded, KVNeed, LayerCache, NormSink, StateNeed, StepContext, Stream,
                    feed_forward_class, mixer_class, norm_class, register_block)
 
 # tensor-name infixes of a pre-norm decoder layer's parts (HF naming, qwen3.rs:41,54,81,93)
@@ -61,9 +61,31 @@ class PreNormBlock(Block):
     def state_need(self) -> Optional[StateNeed]:
         return self.mixer.state_need()
 
-    def forward(self, stream: Stream, ctx: StepContext, cache: LayerCache) -> Stream:
-        h = self.norm1.forward(stream.resid, stream.pending, self.dtype)
-        a = self.mixer.forward(h, ctx, cache)
-        h2 = self.norm2.forward(stream.resid, a, self.dtype)
-        m = self.ffn.forward(h2, ctx)
+    # ---- folding norms into the products around them (parts.base.Folded) ---------------------
+    folds = True         # `forward` takes `next_norm` and a stream with `folded`
+
+    def first_norm(self):
+        """The norm that a block before this one may half do, or None."""
+        return self.norm1 if (self.norm1.foldable and self.mixer.takes_folded) else None
+
+    def forward(self, stream: Stream, ctx: StepContext, cache: LayerCache, next_norm=None) -> Stream:
+        """`next_norm`: the first norm of the block that runs next, if that block lets this
+        one's feed-forward half do it."""
+        if stream.folded is not None:
+            if stream.folded.norm is not self.norm1:
+                raise RuntimeError("the stream carries a half-done norm of another block")
+            h = stream.folded
+        else:
+            h = self.norm1.forward(stream.resid, stream.pending, self.dtype)
+        if self.mixer.takes_sink and self.ffn.takes_folded and self.norm2.foldable:
+            a = self.mixer.forward(h, ctx, cache, sink=NormSink(stream.resid, self.norm2))
+        else:
+            a = self.mixer.forward(h, ctx, cache)
+        h2 = a if isinstance(a, Folded) else self.norm2.forward(stream.resid, a, self.dtype)
+        if next_norm is not None and self.ffn.takes_sink:
+            m = self.ffn.forward(h2, ctx, sink=NormSink(stream.resid, next_norm))
+        else:
+            m = self.ffn.forward(h2, ctx)
+        if isinstance(m, Folded):
+            return Stream(stream.resid, None, m)
         return Stream(stream.resid, m)

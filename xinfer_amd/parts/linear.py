@@ -16,6 +16,7 @@ from typing import Optional
 import torch
 
 from .. import kernels
+from .base import Folded, NormSink
 
 
 class Linear:
@@ -25,15 +26,37 @@ class Linear:
         self.weight = weight.contiguous()
         self.out_features, self.in_features = weight.shape
 
-    def __call__(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
-                 skinny_rows: Optional[int] = None, allow_split: bool = False) -> torch.Tensor:
-        """`allow_split`: the caller hands the result to a norm, which also takes a stack
+    def __call__(self, x, out_dtype: Optional[torch.dtype] = None, skinny_rows: Optional[int] = None,
+                 allow_split: bool = False, sink: Optional[NormSink] = None, gated: bool = False):
+        """`x`: rows, or a `Folded` (the norm before this product is half done: this product
+        finishes it).  `sink`: the norm after this product may be folded: if the sizes allow
+        (bfloat16, up to `kernels.FOLD_ROWS` rows) the result is added into the stream here and a
+        `Folded` comes back instead of rows.  `gated`: the weight is [gate; up] and the result
+        silu(gate) * up, where the fused kernel takes the sizes (else None: the caller does it
+        in two steps).
+        `allow_split`: the caller hands the result to a norm, which also takes a stack
         [P, T, out] of float32 partial sums; few rows and a narrow output then come back so.
         A workgroup of the split product takes more rows of the weight per read of x, which
         on an MI355X pays from about 16 rows on (o and down projections at Qwen3 sizes)."""
         if skinny_rows is None:
             skinny_rows = kernels.SKINNY_ROWS
         w = self.weight
+        if isinstance(x, Folded):
+            if w.dtype == torch.bfloat16 and x.xg.shape[1] % 8 == 0 and (not gated or out_dtype in (None, torch.bfloat16)):
+                return kernels.linear_fold_in(x.xg, x.ss, x.norm.eps, w, out_dtype or torch.bfloat16, gated=gated)
+            x = x.rows(torch.bfloat16 if w.dtype == torch.bfloat16 else torch.float32)
+        if gated:
+            if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+                    and 0 < x.shape[0] <= kernels.SKINNY_GATED_ROWS and x.shape[1] % 8 == 0):
+                return kernels.linear_skinny(x, w, gated=True)        # gate, up and silu*mul in one pass
+            return None
+        if (sink is not None and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2
+                and 0 < x.shape[0] <= kernels.FOLD_ROWS and x.shape[1] % 8 == 0 and w.shape[0] % 8 == 0
+                and sink.norm.foldable and sink.norm.weight.shape[0] == w.shape[0]
+                and sink.resid.dtype == torch.float32 and sink.resid.is_contiguous()
+                and kernels.linear_fold_parts(x.shape[0], w.shape[0], w.shape[1]) <= kernels.FOLD_PARTS):
+            xg, ss = kernels.linear_fold_out(x, w, sink.resid, sink.norm.weight)
+            return Folded(xg, ss, sink.norm)
         out_dtype = out_dtype or x.dtype
         if w.dtype == torch.float32:
             xf = x if x.dtype == torch.float32 else x.float()

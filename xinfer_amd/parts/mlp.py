@@ -46,11 +46,12 @@ class GatedMLP(FeedForward):
         self.gate_up = Linear(torch.cat([g.to(common), u.to(common)], dim=0))
         self.down = Linear(lin(f"{prefix}.down_proj.weight"))
 
-    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
-        w = self.gate_up.weight
-        if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
-                and 0 < x.shape[0] <= kernels.SKINNY_GATED_ROWS and x.shape[1] % 8 == 0):
-            m = kernels.linear_skinny(x, w, gated=True)        # gate, up and silu*mul in one pass
-        else:
+    takes_sink = True
+    takes_folded = True
+
+    def forward(self, x, ctx: StepContext, sink=None):
+        """`x`: rows or a `Folded`; `sink`: see `Part.takes_sink`."""
+        m = self.gate_up(x, out_dtype=self.dtype, gated=True)         # gate, up and silu*mul in one pass
+        if m is None:
             m = kernels.silu_mul(self.gate_up(x, out_dtype=self.dtype))
-        return self.down(m, out_dtype=self.dtype, allow_split=True)  # the next norm adds the parts
+        return self.down(m, out_dtype=self.dtype, allow_split=True, sink=sink)   # the next norm adds the parts

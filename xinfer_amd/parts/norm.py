@@ -20,6 +20,7 @@ from .base import Norm, register_norm
 @register_norm("rmsnorm")
 class RMSNorm(Norm):
     graph_safe = True
+    foldable = True      # the products around it can carry it (parts.base.Folded)
 
     def __init__(self, spec: PartSpec, dtype: torch.dtype):
         super().__init__(spec, dtype)
