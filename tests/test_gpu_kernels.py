@@ -543,6 +543,27 @@ def test_attention_decode_mfma(nq, nkv, d, page, window, seqs):
     assert err < _tol(torch.bfloat16, 2), err
 
 
+@pytest.mark.parametrize("window", [0, 100])
+def test_attention_decode_one_split_per_sequence(window):
+    """Many sequences of about the same length: a workgroup takes a whole sequence and writes the
+    result itself (no partial results, no second kernel).  256 (sequence, kv head) pairs."""
+    from xinfer_amd import kernels
+    nq, nkv, d, page = 8, 8, 32, 16
+    g = torch.Generator().manual_seed(23)
+    seqs = [(290 + (7 * b) % 30, 1) for b in range(32)]
+    assert kernels.decode_keys_per_workgroup(32 * nkv, 320, similar=True) > 320
+    assert kernels.decode_keys_per_workgroup(32 * nkv, 320, similar=False) == 256
+    assert kernels.decode_keys_per_workgroup(48 * nkv, 320, similar=True) == 256     # 384 pairs leave units idle
+    case = _paged_case(g, torch.bfloat16, nq, nkv, d, page, seqs)
+    scale = 1.0 / math.sqrt(d)
+    ref = _attention_ref(case, seqs, window, scale)
+    q, kc, vt, bt = _mfma_inputs(case)
+    _, ctx = _cu_ctx(seqs)
+    out = kernels.attention_decode_bf16(q, kc, vt, bt, ctx.to(DEV), int(ctx.max()), scale, window, similar=True)
+    err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
+    assert err < _tol(torch.bfloat16, 2), err
+
+
 def test_attention_mfma_far_key_and_page_edges():
     """One key is made to win the softmax, placed in turn at a page's first and last offset,
     at the first key, and just before the query: decode and prefill kernels must return its

@@ -51,14 +51,14 @@ __device__ __forceinline__ bf16x8 zero8() {
 // as this step's have been used, into the same registers.  The page numbers of the chunk
 // are read once into LDS, so that no step waits for the block table.  Partial results
 // (sums scaled by 2^-m, with m and l) go to a workspace, combined by the second kernel in
-// split order.
+// split order; with one split for every sequence the kernel writes the result itself.
 // =====================================================================================
 template <int KC, int DT>
 __global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ vt_cache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ ctx_lens,
-    float* __restrict__ part_o, float* __restrict__ part_ml, int max_splits, float scale_log2, int window,
-    int page, int nq, int nkv, int d, int keys_per_wg) {
+    float* __restrict__ part_o, float* __restrict__ part_ml, bf16* __restrict__ out, int max_splits, float scale_log2,
+    int window, int page, int nq, int nkv, int d, int keys_per_wg) {
   extern __shared__ float lds[];  // [4 waves][g][d] + [4][g][2] + page numbers of the chunk
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, j = lane >> 4;
@@ -220,6 +220,10 @@ __global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
       o += lds_o[((size_t)wv * g + h) * d + i] * f;
       ll += lds_ml[(wv * g + h) * 2 + 1] * f;
     }
+    if (max_splits == 1) {   // the only split of every sequence: the result itself
+      out[((size_t)seq * nq + kvh * g + h) * d + i] = __float2bfloat16(o / ll);
+      continue;
+    }
     const size_t pidx = ((size_t)seq * nq + kvh * g + h) * max_splits + split;
     part_o[pidx * d + i] = o;
     if (i == 0) {
@@ -301,12 +305,13 @@ int xi_attention_decode_bf16(const void* q, const void* k_cache, const void* vt_
 #define XI_DC(KC, DT)                                                                              \
   attn_decode_split_kernel<KC, DT><<<grid, 256, lds, stream>>>(                                    \
       (const bf16*)q, (const bf16*)k_cache, (const bf16*)vt_cache, block_tables, max_pages, ctx_lens, \
-      part_o, part_ml, max_splits, sl, window, page, nq, nkv, d, keys_per_wg)
+      part_o, part_ml, (bf16*)out, max_splits, sl, window, page, nq, nkv, d, keys_per_wg)
   if (d <= 64) XI_DC(2, 4);
   else if (d <= 128) XI_DC(4, 8);
   else XI_DC(8, 16);
 #undef XI_DC
   XI_LAUNCH_CHECK("attention_decode_split");
+  if (max_splits == 1) return 0;   // the split kernel has written the result
   attn_decode_combine_kernel<<<dim3(nq, n_seq), 64, max_splits * sizeof(float), stream>>>(part_o, part_ml, ctx_lens, (bf16*)out,
                                                                   max_splits, window, nq, d, keys_per_wg);
   XI_LAUNCH_CHECK("attention_decode_combine");

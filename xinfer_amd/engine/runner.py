@@ -37,6 +37,12 @@ class StepError(ValueError):
     pass
 
 
+def _similar(ctx_lens: np.ndarray) -> bool:
+    """The sequences of a step are about equally long (kernels may then give each a workgroup of
+    its own instead of cutting all into equal pieces)."""
+    return bool(ctx_lens.size) and float(ctx_lens.mean()) >= 0.9 * float(ctx_lens.max())
+
+
 class _Staging:
     """Pinned host buffers through which a step's index arrays reach the device: one copy
     for the 32-bit arrays and one for the 64-bit ones."""
@@ -129,8 +135,8 @@ class ModelRunner:
         self.use_graphs = bool(use_graphs) and model.graph_safe
         self.graph_max_batch = int(graph_max_batch)
         self.graph_after = max(1, int(graph_after))
-        self._graphs: Dict[Tuple[int, int], _DecodeGraph] = {}
-        self._seen: Dict[Tuple[int, int], int] = {}
+        self._graphs: Dict[Tuple[int, int, bool], _DecodeGraph] = {}
+        self._seen: Dict[Tuple[int, int, bool], int] = {}
         self._graph_pool = None
         # widest block table a request can have: the fixed width of a recorded step's tables
         self._max_table = max(1, -(-model.spec.max_positions // self.page_size))
@@ -229,6 +235,7 @@ class ModelRunner:
             ctx_lens_host=a.ctx_lens.tolist() if host_lengths else (),
             max_q_len=int(q_lens.max()),
             max_ctx_len=int(a.ctx_lens.max()) if max_ctx_len is None else int(max_ctx_len),
+            similar_lengths=_similar(a.ctx_lens),
             no_slots=d64[o64[2]:o64[2] + T], empty_f32=self._empty_f32)
         return ctx, v32(0, T), v32(5, rows32.size), d32, d64
 
@@ -243,7 +250,7 @@ class ModelRunner:
         bucket = 1024
         while bucket < longest:
             bucket *= 4
-        key = (B, bucket)
+        key = (B, bucket, _similar(a.ctx_lens))     # what kernels choose their shapes from
         all_rows = np.zeros(B, dtype=np.int32)
         all_rows[:rows32.size] = rows32
         g = self._graphs.get(key)

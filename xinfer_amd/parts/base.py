@@ -81,6 +81,7 @@ class StepContext:
     ctx_lens_host: Sequence[int] = ()
     max_q_len: int = 0
     max_ctx_len: int = 0
+    similar_lengths: bool = False              # host: the mean cached length is at least 0.9 of the longest
     no_slots: Optional[torch.Tensor] = None    # int64 [T] of -1: "store nothing"
     empty_f32: Optional[torch.Tensor] = None   # float32 [1, 0]: tables of "no rotation"
     scratch: Dict[Any, Any] = field(default_factory=dict)   # per-step data that kernels derive once
