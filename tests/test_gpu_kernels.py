@@ -236,8 +236,8 @@ def test_linear_folded_norm_refuses():
         kernels.linear_fold_out(x, w, r, gw)
     with pytest.raises(kernels.KernelError, match="do not match"):
         kernels.linear_fold_out(x[:4].contiguous(), w, r[:3].contiguous(), gw)
-    with pytest.raises(kernels.KernelError, match="256 parts"):
-        kernels.linear_fold_in(x[:4].contiguous(), torch.zeros((4, 300), device=DEV), 1e-6, w)
+    with pytest.raises(kernels.KernelError, match="512 parts"):
+        kernels.linear_fold_in(x[:4].contiguous(), torch.zeros((4, 600), device=DEV), 1e-6, w)
 
 
 def test_linear_skinny_refuses():

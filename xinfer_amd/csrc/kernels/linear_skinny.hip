@@ -37,14 +37,6 @@ __device__ __forceinline__ bf16x8 zeros8() {
   return z;
 }
 
-// Row of w that tile t of the workgroup at n0 reads.  Plain: tiles are consecutive blocks of
-// 16 rows.  Gated: tiles 0..RT/2-1 are gate rows, tiles RT/2..RT-1 the matching up rows.
-template <int RT, bool GATED>
-__device__ __forceinline__ int tile_row0(int t, int n0, int N) {
-  if (!GATED) return n0 + 16 * t;
-  return t < RT / 2 ? n0 + 16 * t : N + n0 + 16 * (t - RT / 2);
-}
-
 // A norm folded into the two products around it (few rows, MT = 1).  The product before the
 // norm (MODE 1, kFoldOut) adds its result into the float32 residual stream, writes
 // xg = round(stream * g) with the norm's weight g, and the sum of squares of its part of every
@@ -68,7 +60,7 @@ template <int MT, int RT, int NW, int U, bool GATED, typename TO, int MODE>
 __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16* __restrict__ x,
                                                                 const bf16* __restrict__ w,
                                                                 TO* __restrict__ y, int M, int N, int K,
-                                                                int steps_per_slice, SkinnyFold fold) {
+                                                                int steps_per_slice, int R, SkinnyFold fold) {
   static_assert(!GATED || RT % 2 == 0, "the gated form pairs gate tiles with up tiles");
   static_assert(MODE == kFoldNone || (MT == 1 && NW == 8), "a folded norm: up to 16 rows, 8 waves");
   static_assert(MODE != kFoldOut || !GATED, "the product before a norm is a plain one");
@@ -86,27 +78,31 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16* __re
   const int r = lane & 15, j = lane >> 4;
   // kFoldIn: 32 threads per row add up the parts of its sum of squares; the loads start now, the
   // sum is taken after the products
-  float ss_mine[8];
+  constexpr int kSsLoads = 16;   // 32 threads x 16 loads: up to 512 parts of a row's sum
+  float ss_mine[kSsLoads];
   if constexpr (MODE == kFoldIn) {
     const int token = threadIdx.x >> 5, sub = threadIdx.x & 31;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < kSsLoads; ++i) {
       const int p = sub + 32 * i;
       ss_mine[i] = (token < M && p < fold.parts) ? fold.ss_in[(size_t)token * fold.parts + p] : 0.f;
     }
   }
-  const int n0 = blockIdx.x * (GATED ? 16 * (RT / 2) : 16 * RT);
+  // The workgroup owns output features n0 .. n0 + R - 1 (R <= 16 * PAIRS, any number: the grid
+  // can then be a multiple of the compute units whatever N is).  Lanes past its last feature
+  // read that feature's row again (the same address in one instruction costs nothing) and their
+  // results are dropped.
+  const int n0 = blockIdx.x * R;
   const int ks = blockIdx.y;
-  const int w_rows = GATED ? 2 * N : N;
+  const int n_last = min(n0 + R, N) - 1;
 
-  // rows of w and x this lane loads; rows past the end are clamped (their results are dropped)
   const bf16* wp[RT];
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
-    int row = tile_row0<RT, GATED>(t, n0, N) + r;
-    const int last = GATED ? (t < RT / 2 ? N - 1 : 2 * N - 1) : N - 1;
-    if (row > last) row = last;
-    if (row > w_rows - 1) row = w_rows - 1;
+    const int tl = GATED ? (t < RT / 2 ? t : t - RT / 2) : t;     // tile among the workgroup's features
+    int n = n0 + 16 * tl + r;
+    if (n > n_last) n = n_last;
+    const int row = (GATED && t >= RT / 2) ? N + n : n;
     wp[t] = w + (size_t)row * K + 8 * j;
   }
   const bf16* xp[MT];
@@ -215,7 +211,7 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16* __re
   if constexpr (MODE == kFoldIn) {   // read after the barriers of the merge below
     float t = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) t += ss_mine[i];
+    for (int i = 0; i < kSsLoads; ++i) t += ss_mine[i];
 #pragma unroll
     for (int o = 16; o; o >>= 1) t += __shfl_xor(t, o, kWave);
     if ((threadIdx.x & 31) == 0) fold_lds[threadIdx.x >> 5] = rsqrtf(t * fold.inv_h + fold.eps);
@@ -271,9 +267,10 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16* __re
         a0 *= inv;
         a1 *= inv;
       }
+      const bool mine = n <= n_last;      // a feature of this workgroup that exists
       if constexpr (MODE == kFoldOut) {
         float sq = 0.f;
-        if (token < M && n < N) {
+        if (token < M && mine) {
           const float rr = fold.resid[(size_t)token * N + n] + a0;
           fold.resid[(size_t)token * N + n] = rr;
           fold.xg[(size_t)token * N + n] = from_float<bf16>(rr * fold.g[n]);
@@ -281,7 +278,7 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16* __re
         }
         fold_lds[token * (16 * RT) + (n - n0)] = sq;
       } else {
-        if (token < M && n < N)
+        if (token < M && mine)
           yk[(size_t)token * N + n] = from_float<TO>(GATED ? a0 / (1.f + __expf(-a0)) * a1 : a0);
       }
     }
@@ -299,7 +296,8 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16* __re
 struct SkinnyPlan {
   int ks;    // slices of K across workgroups
   int nw;    // waves per workgroup
-  int rt;    // row tiles per workgroup
+  int rt;    // row tiles of w per workgroup (the kernel's shape)
+  int rows;  // output features per workgroup, at most 16 * rt (gated: 8 * rt)
 };
 
 // Shapes that are built: 16 waves leave registers for 2 row tiles, 8 row tiles for 32 tokens.
@@ -312,11 +310,12 @@ static bool skinny_shape_ok(int rt, int nw, int mt, bool gated) {
 }
 
 // ks and nw fix the order of the sums: they come from (N, K) and the caller's wish alone.
-// rt only says which workgroup computes what, and is chosen for speed.  Measured on MI355X:
-// a workgroup reads its x operands from L2 once per 16 * rt rows of w, and such a read costs
-// about 0.6 of a read of w from memory, so more row tiles pay with more rows of x; the
+// rt and rows only say which workgroup computes what, and are chosen for speed.  Measured on
+// MI355X: a workgroup reads its x operands from L2 once for all its rows of w, and such a read
+// costs about 0.6 of a read of w from memory, so more rows of w pay with more rows of x; the
 // stream of w itself slows by about 4% per further row tile; and a grid that is no multiple of
-// the 256 compute units leaves some of them idle at the end.
+// the 256 compute units leaves some of them idle at the end, which is why a workgroup may own
+// a number of features that is no multiple of 16 (N = 5120: 20 each make 256 workgroups).
 static SkinnyPlan plan_skinny(int M, int N, int K, bool gated, bool allow_split) {
   SkinnyPlan p;
   const int tiles = (N + 15) / 16;       // output tiles (gated: each a gate tile and an up tile)
@@ -331,54 +330,66 @@ static SkinnyPlan plan_skinny(int M, int N, int K, bool gated, bool allow_split)
   const int per = gated ? 2 : 1;         // tiles of w per output tile
   double best = 0.;
   p.rt = per;
+  p.rows = 16;
   for (int q = 1; q <= 8; ++q) {         // output tiles per workgroup
     const int rt = q * per;
     if (rt > 8 || !skinny_shape_ok(rt, p.nw, mt, gated)) continue;
-    const double g = (double)((tiles + q - 1) / q) * p.ks / 256.;
-    const double idle = g >= 1. ? ceil(g) / g : pow(g, -0.6);
-    const double cost = idle * (1. + 0.04 * (rt - 1) + 0.6 * (M / 16.) / rt);
-    if (best == 0. || cost < best * 0.999) {
-      best = cost;
-      p.rt = rt;
+    const int cap = 16 * q;
+    const int g_full = (N + cap - 1) / cap;
+    // whole tiles, or the next grids that are multiples of 128 and of 256 workgroups
+    const int grids[3] = {g_full, (g_full * p.ks + 127) / 128 * 128 / p.ks, (g_full * p.ks + 255) / 256 * 256 / p.ks};
+    for (int c = 0; c < 3; ++c) {
+      if (grids[c] < g_full) continue;
+      const int rows = c == 0 ? cap : (N + grids[c] - 1) / grids[c];
+      if (rows < 1 || rows > cap) continue;
+      const double g = (double)((N + rows - 1) / rows) * p.ks / 256.;
+      const double idle = g >= 1. ? ceil(g) / g : pow(g, -0.6);
+      const double cost = idle * (1. + 0.04 * (rt - 1) + 0.6 * (double)M / (rows * per));
+      if (best == 0. || cost < best * 0.999) {
+        best = cost;
+        p.rt = rt;
+        p.rows = rows;
+      }
     }
   }
   return p;
 }
 
 template <int MT, int RT, int NW, bool GATED, typename TO, int MODE = kFoldNone>
-static void launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, int ks, hipStream_t stream,
-                          const SkinnyFold& fold = SkinnyFold{}) {
+static void launch_skinny(const void* x, const void* w, void* y, int M, int N, int K, int ks, int rows,
+                          hipStream_t stream, const SkinnyFold& fold = SkinnyFold{}) {
   // steps of loads in flight, by the registers a wave has (16 waves: 128, 8 waves: 256)
   constexpr int U = (RT + MT <= 2) ? 8 : (RT + MT <= (NW == 16 ? 4 : 7) ? 4 : 2);
-  const int rows_per_wg = GATED ? 16 * (RT / 2) : 16 * RT;
+  const int cap = GATED ? 16 * (RT / 2) : 16 * RT;
+  if (rows <= 0 || rows > cap) rows = cap;
   const int steps = (K + 31) / 32;
   const int sps = (steps + ks - 1) / ks;
-  dim3 grid((unsigned)((N + rows_per_wg - 1) / rows_per_wg), (unsigned)ks);
+  dim3 grid((unsigned)((N + rows - 1) / rows), (unsigned)ks);
   linear_skinny_kernel<MT, RT, NW, U, GATED, TO, MODE><<<grid, NW * 64, 0, stream>>>(
-      (const bf16*)x, (const bf16*)w, (TO*)y, M, N, K, sps, fold);
+      (const bf16*)x, (const bf16*)w, (TO*)y, M, N, K, sps, rows, fold);
 }
 
 // The folded forms exist for up to 16 rows and 8 waves; rt as the plan says.
 template <bool GATED, typename TO, int MODE>
-static bool launch_skinny_fold(int rt, const void* x, const void* w, void* y, int M, int N, int K, hipStream_t stream,
+static bool launch_skinny_fold(int rt, int rows, const void* x, const void* w, void* y, int M, int N, int K, hipStream_t stream,
                                const SkinnyFold& fold) {
   if constexpr (!GATED) {
-    if (rt == 1) { launch_skinny<1, 1, 8, false, TO, MODE>(x, w, y, M, N, K, 1, stream, fold); return true; }
-    if (rt == 3) { launch_skinny<1, 3, 8, false, TO, MODE>(x, w, y, M, N, K, 1, stream, fold); return true; }
+    if (rt == 1) { launch_skinny<1, 1, 8, false, TO, MODE>(x, w, y, M, N, K, 1, rows, stream, fold); return true; }
+    if (rt == 3) { launch_skinny<1, 3, 8, false, TO, MODE>(x, w, y, M, N, K, 1, rows, stream, fold); return true; }
   }
-  if (rt == 2) { launch_skinny<1, 2, 8, GATED, TO, MODE>(x, w, y, M, N, K, 1, stream, fold); return true; }
-  if (rt == 4) { launch_skinny<1, 4, 8, GATED, TO, MODE>(x, w, y, M, N, K, 1, stream, fold); return true; }
-  if (rt == 6) { launch_skinny<1, 6, 8, GATED, TO, MODE>(x, w, y, M, N, K, 1, stream, fold); return true; }
-  if (rt == 8) { launch_skinny<1, 8, 8, GATED, TO, MODE>(x, w, y, M, N, K, 1, stream, fold); return true; }
+  if (rt == 2) { launch_skinny<1, 2, 8, GATED, TO, MODE>(x, w, y, M, N, K, 1, rows, stream, fold); return true; }
+  if (rt == 4) { launch_skinny<1, 4, 8, GATED, TO, MODE>(x, w, y, M, N, K, 1, rows, stream, fold); return true; }
+  if (rt == 6) { launch_skinny<1, 6, 8, GATED, TO, MODE>(x, w, y, M, N, K, 1, rows, stream, fold); return true; }
+  if (rt == 8) { launch_skinny<1, 8, 8, GATED, TO, MODE>(x, w, y, M, N, K, 1, rows, stream, fold); return true; }
   return false;
 }
 
 template <int RT, int NW, bool GATED, typename TO>
-static void launch_skinny_mt(int mt, const void* x, const void* w, void* y, int M, int N, int K, int ks,
+static void launch_skinny_mt(int mt, const void* x, const void* w, void* y, int M, int N, int K, int ks, int rows,
                              hipStream_t stream) {
-  if (mt == 1) launch_skinny<1, RT, NW, GATED, TO>(x, w, y, M, N, K, ks, stream);
-  else if (mt == 2) launch_skinny<2, RT, NW, GATED, TO>(x, w, y, M, N, K, ks, stream);
-  else if constexpr (RT <= 6) launch_skinny<4, RT, NW, GATED, TO>(x, w, y, M, N, K, ks, stream);   // 33..64 rows
+  if (mt == 1) launch_skinny<1, RT, NW, GATED, TO>(x, w, y, M, N, K, ks, rows, stream);
+  else if (mt == 2) launch_skinny<2, RT, NW, GATED, TO>(x, w, y, M, N, K, ks, rows, stream);
+  else if constexpr (RT <= 6) launch_skinny<4, RT, NW, GATED, TO>(x, w, y, M, N, K, ks, rows, stream);   // 33..64 rows
 }
 
 }  // namespace xi
@@ -396,9 +407,13 @@ int xi_linear_skinny_slices(int N, int K, int gated, int allow_split) {
   return plan_skinny(1, N, K, gated != 0, allow_split != 0).ks;
 }
 
-// The row tiles of w a workgroup takes for these sizes (it does not change any sum).
+// The row tiles of w a workgroup takes for these sizes, and the output features it owns (they
+// do not change any sum).
 int xi_linear_skinny_row_tiles(int M, int N, int K, int gated, int allow_split) {
   return plan_skinny(M, N, K, gated != 0, allow_split != 0).rt;
+}
+int xi_linear_skinny_rows(int M, int N, int K, int gated, int allow_split) {
+  return plan_skinny(M, N, K, gated != 0, allow_split != 0).rows;
 }
 
 // The product before a norm, for M <= 16 rows: resid [M, N] float32 += x [M, K] @ w [N, K]^T;
@@ -407,7 +422,7 @@ int xi_linear_skinny_row_tiles(int M, int N, int K, int gated, int allow_split) 
 // workgroup.  The product after the norm then takes xg and ss (xi_linear_skinny_fold_in).
 int xi_linear_skinny_fold_parts(int M, int N, int K) {
   const SkinnyPlan p = plan_skinny(M, N, K, false, false);
-  return (N + 16 * p.rt - 1) / (16 * p.rt);
+  return (N + p.rows - 1) / p.rows;
 }
 
 int xi_linear_skinny_fold_out(const void* x, const void* w, int M, int N, int K, float* resid, const float* g, void* xg,
@@ -419,19 +434,19 @@ int xi_linear_skinny_fold_out(const void* x, const void* w, int M, int N, int K,
   f.g = g;
   f.xg = (bf16*)xg;
   f.ss_out = ss;
-  const bool ok = launch_skinny_fold<false, bf16, kFoldOut>(p.rt, x, w, nullptr, M, N, K, stream, f);
+  const bool ok = launch_skinny_fold<false, bf16, kFoldOut>(p.rt, p.rows, x, w, nullptr, M, N, K, stream, f);
   XI_CHECK(ok, "linear_skinny_fold_out: no kernel of %d row tiles", p.rt);
   XI_LAUNCH_CHECK("linear_skinny_fold_out");
   return 0;
 }
 
 // The product after a norm whose first half ran in xi_linear_skinny_fold_out: xg [M, K] bf16,
-// ss [M, parts] float32 (parts <= 256), y [M, N] = (xg @ w^T) * rsqrt(sum(ss[row]) / K + eps) per
+// ss [M, parts] float32 (parts <= 512), y [M, N] = (xg @ w^T) * rsqrt(sum(ss[row]) / K + eps) per
 // row, rounded once; gated as in xi_linear_skinny (then y is bfloat16).
 int xi_linear_skinny_fold_in(const void* xg, const void* w, void* y, int M, int N, int K, int out_dtype, int gated,
                              const float* ss, int parts, float eps, hipStream_t stream) {
   XI_CHECK(M > 0 && M <= 16 && N > 0 && K > 0 && K % 8 == 0, "linear_skinny_fold_in: bad sizes M=%d N=%d K=%d", M, N, K);
-  XI_CHECK(parts > 0 && parts <= 256, "linear_skinny_fold_in: %d parts of a row's sum of squares (at most 256)", parts);
+  XI_CHECK(parts > 0 && parts <= 512, "linear_skinny_fold_in: %d parts of a row's sum of squares (at most 512)", parts);
   XI_CHECK(out_dtype == kBF16 || (out_dtype == kF32 && !gated), "linear_skinny_fold_in: output dtype %d", out_dtype);
   const SkinnyPlan p = plan_skinny(M, N, K, gated != 0, false);
   SkinnyFold f{};
@@ -440,9 +455,9 @@ int xi_linear_skinny_fold_in(const void* xg, const void* w, void* y, int M, int 
   f.eps = eps;
   f.inv_h = 1.f / (float)K;
   bool ok;
-  if (gated) ok = launch_skinny_fold<true, bf16, kFoldIn>(p.rt, xg, w, y, M, N, K, stream, f);
-  else if (out_dtype == kBF16) ok = launch_skinny_fold<false, bf16, kFoldIn>(p.rt, xg, w, y, M, N, K, stream, f);
-  else ok = launch_skinny_fold<false, float, kFoldIn>(p.rt, xg, w, y, M, N, K, stream, f);
+  if (gated) ok = launch_skinny_fold<true, bf16, kFoldIn>(p.rt, p.rows, xg, w, y, M, N, K, stream, f);
+  else if (out_dtype == kBF16) ok = launch_skinny_fold<false, bf16, kFoldIn>(p.rt, p.rows, xg, w, y, M, N, K, stream, f);
+  else ok = launch_skinny_fold<false, float, kFoldIn>(p.rt, p.rows, xg, w, y, M, N, K, stream, f);
   XI_CHECK(ok, "linear_skinny_fold_in: no kernel of %d row tiles", p.rt);
   XI_LAUNCH_CHECK("linear_skinny_fold_in");
   return 0;
@@ -464,7 +479,10 @@ int xi_linear_skinny(const void* x, const void* w, void* y, int M, int N, int K,
   XI_CHECK(p.ks == 1 || out_dtype == kF32, "linear_skinny: partial sums of %d slices must be float32", p.ks);
   XI_CHECK(!gated || out_dtype == kBF16, "linear_skinny: the gated form writes bfloat16");
   if (force_nw) p.nw = force_nw;
-  if (force_rt) p.rt = force_rt;
+  if (force_rt) {
+    p.rt = force_rt;
+    p.rows = 0;          // whole tiles
+  }
   XI_CHECK(p.nw == 8 || p.nw == 16, "linear_skinny: %d waves (8 or 16)", p.nw);
   const int mt = (M + 15) / 16;
   XI_CHECK(skinny_shape_ok(p.rt, p.nw, mt, gated != 0), "linear_skinny: no kernel of %d row tiles, %d waves for %d rows%s",
@@ -472,11 +490,11 @@ int xi_linear_skinny(const void* x, const void* w, void* y, int M, int N, int K,
 #define XI_SK_PLAIN(RT, NW)                                                       \
   do {                                                                            \
     if (out_dtype == kBF16)                                                       \
-      launch_skinny_mt<RT, NW, false, bf16>(mt, x, w, y, M, N, K, p.ks, stream);  \
+      launch_skinny_mt<RT, NW, false, bf16>(mt, x, w, y, M, N, K, p.ks, p.rows, stream);  \
     else                                                                          \
-      launch_skinny_mt<RT, NW, false, float>(mt, x, w, y, M, N, K, p.ks, stream); \
+      launch_skinny_mt<RT, NW, false, float>(mt, x, w, y, M, N, K, p.ks, p.rows, stream); \
   } while (0)
-#define XI_SK_GATED(RT, NW) launch_skinny_mt<RT, NW, true, bf16>(mt, x, w, y, M, N, K, p.ks, stream)
+#define XI_SK_GATED(RT, NW) launch_skinny_mt<RT, NW, true, bf16>(mt, x, w, y, M, N, K, p.ks, p.rows, stream)
   if (gated) {
     if (p.nw == 16) XI_SK_GATED(2, 16);
     else if (p.rt == 2) XI_SK_GATED(2, 8);

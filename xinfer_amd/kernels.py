@@ -427,7 +427,7 @@ def linear_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dt
 
 
 FOLD_ROWS = 16            # most rows of the products that carry a folded norm between them
-FOLD_PARTS = 256          # most parts of a row's sum of squares the product after the norm adds up
+FOLD_PARTS = 512          # most parts of a row's sum of squares the product after the norm adds up
 
 
 def linear_fold_parts(M: int, N: int, K: int) -> int:
@@ -477,10 +477,10 @@ def linear_fold_in(xg: torch.Tensor, ss: torch.Tensor, eps: float, w: torch.Tens
             raise KernelError("linear_fold_in: a gated weight must be [2N, K]")
         N //= 2
     _want(ss, torch.float32, "linear_fold_in: ss")
-    if not (0 < M <= FOLD_ROWS) or K % 8 or ss.dim() != 2 or ss.shape[0] != M or not (0 < ss.shape[1] <= 256) \
+    if not (0 < M <= FOLD_ROWS) or K % 8 or ss.dim() != 2 or ss.shape[0] != M or not (0 < ss.shape[1] <= FOLD_PARTS) \
             or not ss.is_contiguous():
         raise KernelError(f"linear_fold_in: M={M} (1..{FOLD_ROWS}), K={K} (multiple of 8), ss {tuple(ss.shape)} "
-                          f"([M, up to 256 parts])")
+                          f"([M, up to {FOLD_PARTS} parts])")
     out_dtype = out_dtype or torch.bfloat16
     if gated and out_dtype != torch.bfloat16:
         raise KernelError("linear_fold_in: the gated form writes bfloat16")
