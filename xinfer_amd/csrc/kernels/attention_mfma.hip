@@ -235,41 +235,61 @@ __global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
 
 // One wave per (head, sequence).  Lanes first share out the splits to find the common
 // maximum and each split's weight, then every lane sums its output dims over the splits in
-// split order.
+// split order.  The kernel lives on latency, so whatever can be asked for at once is: the
+// sequence's length, the first 64 splits' (m, l) and the first kEarly splits' sums all start
+// before anything is known about them (what lies past the sequence's last split is dropped).
 __global__ __launch_bounds__(64) void attn_decode_combine_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ ctx_lens,
     bf16* __restrict__ out, int max_splits, int window, int nq, int d, int keys_per_wg) {
   extern __shared__ float f_s[];  // [max_splits] weight of each split
+  constexpr int kEarly = 16;
   const int head = blockIdx.x, seq = blockIdx.y, lane = threadIdx.x;
-  const int pos = ctx_lens[seq] - 1;
+  const size_t base = ((size_t)seq * nq + head) * max_splits;
+  const float* po = part_o + base * d;
+  const int ctx = ctx_lens[seq];
+  float2 ml0 = {-INFINITY, 0.f};
+  if (lane < max_splits) ml0 = *reinterpret_cast<const float2*>(part_ml + (base + lane) * 2);
+  float early[2][kEarly];          // output dims lane and lane + 64 of the first splits
+#pragma unroll
+  for (int c = 0; c < 2; ++c)
+#pragma unroll
+    for (int e = 0; e < kEarly; ++e)
+      early[c][e] = (e < max_splits && lane + 64 * c < d) ? po[(size_t)e * d + lane + 64 * c] : 0.f;
+  const int pos = ctx - 1;
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int n_splits = (pos - (lo & ~31)) / keys_per_wg + 1;
-  const size_t base = ((size_t)seq * nq + head) * max_splits;
-  float mm = -INFINITY;
-  for (int s = lane; s < n_splits; s += kWave) mm = fmaxf(mm, part_ml[(base + s) * 2]);
+  float mm = lane < n_splits ? ml0.x : -INFINITY;
+  for (int s = lane + kWave; s < n_splits; s += kWave) mm = fmaxf(mm, part_ml[(base + s) * 2]);
   mm = wave_max(mm);
   float ll = 0.f;
   for (int s = lane; s < n_splits; s += kWave) {
-    const float f = __builtin_amdgcn_exp2f(part_ml[(base + s) * 2] - mm);
+    const float ms = s == lane ? ml0.x : part_ml[(base + s) * 2];
+    const float ls = s == lane ? ml0.y : part_ml[(base + s) * 2 + 1];
+    const float f = __builtin_amdgcn_exp2f(ms - mm);
     f_s[s] = f;
-    ll += part_ml[(base + s) * 2 + 1] * f;
+    ll += ls * f;
   }
   ll = wave_sum(ll);
   __syncthreads();
   const float inv = 1.f / ll;
-  for (int i = lane; i < d; i += kWave) {
-    const float* po = part_o + base * d + i;
+  for (int i = lane, c = 0; i < d; i += kWave, ++c) {
     float o = 0.f;
     int s = 0;
+    if (c < 2) {
+#pragma unroll
+      for (int e = 0; e < kEarly; ++e)
+        if (e < n_splits) o += (c == 0 ? early[0][e] : early[1][e]) * f_s[e];
+      s = n_splits < kEarly ? n_splits : kEarly;
+    }
     for (; s + 4 <= n_splits; s += 4) {
-      const float a0 = po[(size_t)s * d], a1 = po[(size_t)(s + 1) * d], a2 = po[(size_t)(s + 2) * d],
-                  a3 = po[(size_t)(s + 3) * d];
+      const float a0 = po[(size_t)s * d + i], a1 = po[(size_t)(s + 1) * d + i], a2 = po[(size_t)(s + 2) * d + i],
+                  a3 = po[(size_t)(s + 3) * d + i];
       o += a0 * f_s[s];
       o += a1 * f_s[s + 1];
       o += a2 * f_s[s + 2];
       o += a3 * f_s[s + 3];
     }
-    for (; s < n_splits; ++s) o += po[(size_t)s * d] * f_s[s];
+    for (; s < n_splits; ++s) o += po[(size_t)s * d + i] * f_s[s];
     out[((size_t)seq * nq + head) * d + i] = __float2bfloat16(o * inv);
   }
 }

@@ -256,39 +256,66 @@ __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, const float* _
     for (int i = lane; i < d; i += kWave) dst[i] = src[i];
     return;
   }
+  // The kernel lives on latency: everything that can be asked for at once is.  A lane holds
+  // pairs lane and lane + 64 of the rotated part and up to 4 elements of the rest (head_dim <=
+  // 256); the position's row of the tables is asked for as soon as the position is there,
+  // while the sum of squares is still being taken.
+  const int half = rot / 2;
+  const int pos = positions[t];
+  float xa[2], xb[2], wa[2], wb[2], xt[4], wt[4];
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    const int i = lane + kWave * p;
+    const bool ok = i < half;
+    const int ia = interleaved ? 2 * i : i;
+    const int ib = interleaved ? 2 * i + 1 : i + half;
+    xa[p] = ok ? to_float(src[ia]) : 0.f;
+    xb[p] = ok ? to_float(src[ib]) : 0.f;
+    wa[p] = (ok && w) ? w[ia] : 1.f;
+    wb[p] = (ok && w) ? w[ib] : 1.f;
+  }
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const int i = rot + lane + kWave * p;
+    const bool ok = i < d;
+    xt[p] = ok ? to_float(src[i]) : 0.f;
+    wt[p] = (ok && w) ? w[i] : 1.f;
+  }
+  const float* c = cos_t + (size_t)pos * half;
+  const float* sn_row = sin_t + (size_t)pos * half;
+  float cs[2], sn[2];
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    const int i = lane + kWave * p;
+    cs[p] = i < half ? c[i] : 1.f;
+    sn[p] = i < half ? sn_row[i] : 0.f;
+  }
   float inv = 1.f;
   if (w) {
     float ss = 0.f;
-    for (int i = lane; i < d; i += kWave) {
-      const float v = to_float(src[i]);
-      ss += v * v;
-    }
+#pragma unroll
+    for (int p = 0; p < 2; ++p) ss += xa[p] * xa[p] + xb[p] * xb[p];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) ss += xt[p] * xt[p];
     ss = wave_sum(ss);
     inv = rsqrtf(ss / (float)d + eps);
   }
-  const int half = rot / 2;
-  const int pos = positions[t];
-  const float* c = cos_t + (size_t)pos * half;
-  const float* s = sin_t + (size_t)pos * half;
-  for (int i = lane; i < half; i += kWave) {
-    const int ia = interleaved ? 2 * i : i;
-    const int ib = interleaved ? 2 * i + 1 : i + half;
-    float a = to_float(src[ia]) * inv;
-    float b = to_float(src[ib]) * inv;
-    if (w) {
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    const int i = lane + kWave * p;
+    if (i < half) {
       // the reference rounds the normed value to the activation type before rotating
       // (two kernels); here it stays in float32 until the single final rounding.
-      a *= w[ia];
-      b *= w[ib];
+      const float a = xa[p] * inv * wa[p];
+      const float b = xb[p] * inv * wb[p];
+      dst[interleaved ? 2 * i : i] = from_float<T>(a * cs[p] - b * sn[p]);
+      dst[interleaved ? 2 * i + 1 : i + half] = from_float<T>(a * sn[p] + b * cs[p]);
     }
-    const float cs = c[i], sn = s[i];
-    dst[ia] = from_float<T>(a * cs - b * sn);
-    dst[ib] = from_float<T>(a * sn + b * cs);
   }
-  for (int i = rot + lane; i < d; i += kWave) {  // dims beyond the rotary part
-    float v = to_float(src[i]) * inv;
-    if (w) v *= w[i];
-    dst[i] = from_float<T>(v);
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {  // dims beyond the rotary part
+    const int i = rot + lane + kWave * p;
+    if (i < d) dst[i] = from_float<T>(xt[p] * inv * wt[p]);
   }
 }
 
@@ -512,6 +539,7 @@ int xi_qk_norm_rope_kv(const void* qkv, int dtype, const float* qw, const float*
   XI_CHECK(n_tok >= 0 && nq > 0 && nkv > 0 && d > 0 && page_size > 0,
            "qk_norm_rope_kv: bad sizes T=%d nq=%d nkv=%d d=%d page=%d", n_tok, nq, nkv, d, page_size);
   XI_CHECK(rot >= 0 && rot <= d && rot % 2 == 0, "qk_norm_rope_kv: rotary_dim %d must be even and <= head_dim %d", rot, d);
+  XI_CHECK(d <= 256, "qk_norm_rope_kv: head_dim %d exceeds 256", d);
   XI_CHECK((qw == nullptr) == (kw == nullptr), "qk_norm_rope_kv: q and k norm weights must both be given or both absent");
   if (n_tok == 0) return 0;
   // Many tokens (prompt portions): the vectorized form.  Few (decode steps): one wave per
