@@ -116,6 +116,7 @@ def serve(workload: str, layers) -> int:
 
 
 def main() -> int:
+    global CONTEXT, PREFILL_TOKENS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
@@ -125,6 +126,10 @@ def main() -> int:
     ap.add_argument("--workload", choices=["decode"] + sorted(WORKLOADS), default="decode",
                     help="decode: the contract's run (default); the others: a serving workload end to end")
     ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=CONTEXT,
+                    help="context length at the end of the decode run (default: the contract's)")
+    ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
+                    help="length of the prefilled prompt (default: the contract's)")
     ap.add_argument("--skip-points", action="store_true", help="only the default decode run")
     ap.add_argument("--only", choices=["all", "decode", "prefill"], default="all",
                     help="run one phase only (for profiling); the JSON line then lacks the other")
@@ -136,6 +141,7 @@ def main() -> int:
         return serve(args.workload, args.layers)
     if args.layers is None:
         args.layers = FULL_LAYERS
+    CONTEXT, PREFILL_TOKENS = args.context, args.prefill_tokens     # the sizes of this run
 
     import torch
     from xinfer_amd.engine import ModelRunner, StepEntry, build_model
