@@ -59,6 +59,9 @@ def _bind(lib):
         "xi_cm_check": (i, [vp, ctypes.c_char_p, i]),
         "xi_cm_last_error": (ctypes.c_char_p, [vp]),
         "xi_cm_max_table_len": (i, [vp, i, _I64P]),
+        "xi_cm_lengths": (None, [vp, i, _I64P, _I64P]),
+        "xi_cm_reserve_many": (i, [vp, i, _I64P, _I32P]),
+        "xi_cm_commit_many": (i, [vp, i, _I64P, _I32P]),
         "xi_cm_build_batch": (i, [vp, i, _I64P, _I32P, _I32P, _I32P, _I32P, _I32P, _I32P,
                                   _I64P, _I32P, i, i]),
     }
@@ -168,6 +171,29 @@ class PagedCacheManager:
             raise CacheError(self._lib.xi_cm_last_error(self._h).decode())
         return r
 
+    # ---- a step's worth in one call ------------------------------------------
+    def lengths(self, rids: np.ndarray) -> np.ndarray:
+        """Cached lengths of the requests `rids` (int64 array); -1 where a request is not live."""
+        out = np.empty(rids.size, np.int64)
+        self._lib.xi_cm_lengths(self._h, int(rids.size), rids.ctypes.data_as(_I64P), out.ctypes.data_as(_I64P))
+        return out
+
+    def reserve_many(self, rids: np.ndarray, counts: np.ndarray) -> None:
+        """`reserve` for every request in turn (rids int64, counts int32); the first that
+        cannot be served raises as `reserve` does, the ones before it keep their pages."""
+        b = self._lib.xi_cm_reserve_many(self._h, int(rids.size), rids.ctypes.data_as(_I64P),
+                                         counts.ctypes.data_as(_I32P))
+        if b >= 0:
+            msg = self._lib.xi_cm_last_error(self._h).decode()
+            if not self.has(int(rids[b])):
+                raise CacheError(msg)
+            raise OutOfPages(f"request {int(rids[b])} needs pages for {int(counts[b])} more tokens: {msg}")
+
+    def commit_many(self, rids: np.ndarray, counts: np.ndarray) -> None:
+        if self._lib.xi_cm_commit_many(self._h, int(rids.size), rids.ctypes.data_as(_I64P),
+                                       counts.ctypes.data_as(_I32P)) != 0:
+            raise CacheError(self._lib.xi_cm_last_error(self._h).decode())
+
     def release(self, rid: int) -> int:
         r = self._lib.xi_cm_release(self._h, rid)
         if r < 0:
@@ -178,14 +204,14 @@ class PagedCacheManager:
     def build_batch(self, rids: Sequence[int], n_tokens: Sequence[int],
                     max_pages: Optional[int] = None) -> BatchArrays:
         B = len(rids)
-        T = int(sum(n_tokens))
+        T = int(np.sum(n_tokens)) if isinstance(n_tokens, np.ndarray) else int(sum(n_tokens))
         G = len(self.groups)
-        ids = np.asarray(rids, dtype=np.int64)
+        ids = rids if isinstance(rids, np.ndarray) and rids.dtype == np.int64 else np.asarray(rids, dtype=np.int64)
         if max_pages is None:
             max_pages = self._lib.xi_cm_max_table_len(self._h, B, ids.ctypes.data_as(_I64P))
             if max_pages < 0:
                 raise CacheError("cannot build the batch: a request is not live")
-        nt = np.asarray(n_tokens, dtype=np.int32)
+        nt = n_tokens if isinstance(n_tokens, np.ndarray) and n_tokens.dtype == np.int32 else np.asarray(n_tokens, dtype=np.int32)
         out = BatchArrays(
             num_tokens=T, num_seqs=B, max_pages=int(max_pages),
             positions=np.empty(T, np.int32), tok_seq=np.empty(T, np.int32),

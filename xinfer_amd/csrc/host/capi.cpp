@@ -59,6 +59,26 @@ int xi_cm_check(CacheManager* cm, char* why, int cap) {
 }
 const char* xi_cm_last_error(CacheManager* cm) { return cm->last_error().c_str(); }
 
+// The same for many requests in one call (a step's worth): lengths (-1: not live); reserve until
+// one fails (returns its index, or -1 if all succeeded); commit all (returns 0, or -1 - index of
+// the first that failed, the ones before it committed).
+void xi_cm_lengths(CacheManager* cm, int B, const int64_t* ids, int64_t* out) {
+  for (int b = 0; b < B; ++b) {
+    const xi::RequestPages* r = cm->find(ids[b]);
+    out[b] = r ? r->length : -1;
+  }
+}
+int xi_cm_reserve_many(CacheManager* cm, int B, const int64_t* ids, const int32_t* counts) {
+  for (int b = 0; b < B; ++b)
+    if (!cm->reserve(ids[b], counts[b])) return b;
+  return -1;
+}
+int xi_cm_commit_many(CacheManager* cm, int B, const int64_t* ids, const int32_t* counts) {
+  for (int b = 0; b < B; ++b)
+    if (cm->commit(ids[b], counts[b]) < 0) return -1 - b;
+  return 0;
+}
+
 }  // extern "C"
 
 // ---- scheduler -----------------------------------------------------------------------

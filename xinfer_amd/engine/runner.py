@@ -163,38 +163,62 @@ class ModelRunner:
         spec = self.model.spec
         if not entries:
             return torch.empty((0, spec.vocab_size), dtype=torch.float32, device=self.device)
-        seen = set()
-        rids, counts, all_tokens, rows = [], [], [], []
-        base = 0
-        for e in entries:
-            n = len(e.tokens)
-            if n == 0:
-                raise StepError(f"request {e.request}: an entry needs at least one token")
-            if e.request in seen:
-                raise StepError(f"request {e.request} appears twice in one step")
-            seen.add(e.request)
-            if not self.cache.has(e.request):
-                raise StepError(f"request {e.request} is not live")
-            if self.cache.length(e.request) + n > spec.max_positions:
-                raise StepError(
-                    f"request {e.request}: {self.cache.length(e.request) + n} tokens exceed the "
-                    f"model's {spec.max_positions} positions")
-            for w in e.want:
-                if not (0 <= w < n):
-                    raise StepError(f"request {e.request}: wanted place {w} is outside its {n} tokens")
-                rows.append(base + int(w))
-            rids.append(e.request)
-            counts.append(n)
-            all_tokens.extend(int(t) for t in e.tokens)
-            base += n
-        ids_host = np.asarray(all_tokens, dtype=np.int64)
+        B = len(entries)
+        if all(len(e.tokens) == 1 for e in entries):
+            # a step of single tokens (the hot path of decoding): checked and reserved in a few
+            # calls for all entries together
+            rid_arr = np.fromiter((e.request for e in entries), np.int64, B)
+            counts_arr = np.ones(B, np.int32)
+            ids_host = np.fromiter((e.tokens[0] for e in entries), np.int64, B)
+            if len(set(rid_arr.tolist())) != B:
+                raise StepError("a request appears twice in one step")
+            lengths = self.cache.lengths(rid_arr)
+            if lengths.min() < 0:
+                raise StepError(f"request {int(rid_arr[int(lengths.argmin())])} is not live")
+            if lengths.max() + 1 > spec.max_positions:
+                b = int(lengths.argmax())
+                raise StepError(f"request {int(rid_arr[b])}: {int(lengths[b]) + 1} tokens exceed the "
+                                f"model's {spec.max_positions} positions")
+            rows = []
+            for b, e in enumerate(entries):
+                for w in e.want:
+                    if w != 0:
+                        raise StepError(f"request {e.request}: wanted place {w} is outside its 1 tokens")
+                    rows.append(b)
+        else:
+            seen = set()
+            rids, counts, all_tokens, rows = [], [], [], []
+            base = 0
+            for e in entries:
+                n = len(e.tokens)
+                if n == 0:
+                    raise StepError(f"request {e.request}: an entry needs at least one token")
+                if e.request in seen:
+                    raise StepError(f"request {e.request} appears twice in one step")
+                seen.add(e.request)
+                if not self.cache.has(e.request):
+                    raise StepError(f"request {e.request} is not live")
+                if self.cache.length(e.request) + n > spec.max_positions:
+                    raise StepError(
+                        f"request {e.request}: {self.cache.length(e.request) + n} tokens exceed the "
+                        f"model's {spec.max_positions} positions")
+                for w in e.want:
+                    if not (0 <= w < n):
+                        raise StepError(f"request {e.request}: wanted place {w} is outside its {n} tokens")
+                    rows.append(base + int(w))
+                rids.append(e.request)
+                counts.append(n)
+                all_tokens.extend(int(t) for t in e.tokens)
+                base += n
+            rid_arr = np.asarray(rids, dtype=np.int64)
+            counts_arr = np.asarray(counts, dtype=np.int32)
+            ids_host = np.asarray(all_tokens, dtype=np.int64)
         if ids_host.min() < 0 or ids_host.max() >= spec.vocab_size:
             raise StepError(f"a token id is outside the vocabulary of {spec.vocab_size}")
         if not reserved:
-            for rid, n in zip(rids, counts):
-                self.cache.reserve(rid, n)      # OutOfPages leaves every request's length as it was
-        decode = self.use_graphs and max(counts) == 1 and len(rids) <= self.graph_max_batch
-        arrays = self.cache.build_batch(rids, counts, max_pages=self._max_table if decode else None)
+            self.cache.reserve_many(rid_arr, counts_arr)   # OutOfPages leaves every request's length as it was
+        decode = self.use_graphs and int(counts_arr.max()) == 1 and B <= self.graph_max_batch
+        arrays = self.cache.build_batch(rid_arr, counts_arr, max_pages=self._max_table if decode else None)
         ids32 = ids_host.astype(np.int32)
         rows32 = np.asarray(rows, dtype=np.int32)
         if decode:
@@ -203,8 +227,7 @@ class ModelRunner:
             ctx, ids, want_rows, _, _ = self._context(arrays, ids32, rows32)
             logits = self.model.forward(ids, ctx, self.layer_caches, want_rows)
         if not reserved:
-            for rid, n in zip(rids, counts):
-                self.cache.commit(rid, n)
+            self.cache.commit_many(rid_arr, counts_arr)
         return logits
 
     # ---- index arrays on the device -------------------------------------------------
@@ -215,12 +238,7 @@ class ModelRunner:
         dev = self.device
         G = len(self.cache.groups)
         T, B = a.num_tokens, a.num_seqs
-        no_slots = np.full(T, -1, dtype=np.int64)
-        parts32 = [ids32, a.positions, a.tok_seq, a.cu_q, a.ctx_lens, rows32, a.block_tables]
-        parts64 = [a.state_slots.astype(np.int64), a.slots, no_slots]
-        d32, o32 = self._staging.upload(parts32, torch.int32, dst32)
-        d64, o64 = self._staging.upload(parts64, torch.int64, dst64)
-        self._staging.mark()
+        d32, o32, d64, o64 = self._upload(a, ids32, rows32, dst32, dst64)
         v32 = lambda i, n: d32[o32[i]:o32[i] + n]
         P = a.max_pages
         tables = v32(6, G * B * P).view(G, B, P)
@@ -238,6 +256,17 @@ class ModelRunner:
             similar_lengths=_similar(a.ctx_lens),
             no_slots=d64[o64[2]:o64[2] + T], empty_f32=self._empty_f32)
         return ctx, v32(0, T), v32(5, rows32.size), d32, d64
+
+    def _upload(self, a: BatchArrays, ids32: np.ndarray, rows32: np.ndarray, dst32=None, dst64=None):
+        """The step's arrays to the device in two copies (into the fixed buffers of a recorded
+        step if given); returns both buffers with the offsets of their parts."""
+        no_slots = np.full(a.num_tokens, -1, dtype=np.int64)
+        parts32 = [ids32, a.positions, a.tok_seq, a.cu_q, a.ctx_lens, rows32, a.block_tables]
+        parts64 = [a.state_slots.astype(np.int64), a.slots, no_slots]
+        d32, o32 = self._staging.upload(parts32, torch.int32, dst32)
+        d64, o64 = self._staging.upload(parts64, torch.int64, dst64)
+        self._staging.mark()
+        return d32, o32, d64, o64
 
     # ---- decode steps as HIP graphs ---------------------------------------------------
     def _replay_decode(self, a: BatchArrays, ids32: np.ndarray, rows32: np.ndarray) -> torch.Tensor:
@@ -276,8 +305,7 @@ class ModelRunner:
             g = _DecodeGraph(graph, d32, d64, logits, want, keep=(every_row, ctx, ids))
             self._graphs[key] = g
         else:
-            self._context(a, ids32, all_rows, dst32=g.dev32, dst64=g.dev64, max_ctx_len=bucket,
-                          host_lengths=False)
+            self._upload(a, ids32, all_rows, g.dev32, g.dev64)
         g.graph.replay()
         self.graph_replays += 1
         if rows32.size == B and np.array_equal(rows32, np.arange(B)):
