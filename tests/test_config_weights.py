@@ -191,3 +191,16 @@ def test_command_line_options_follow_the_reference():
     a = build_parser().parse_args(["--m", "x", "--prompts", "a|b", "--max-num-seqs", "4", "--top-k", "5", "--top-p", "0.9",
                                    "--temperature", "0.5", "--kv-fraction", "0.3", "--disable-cuda-graph"])
     assert a.prompts == "a|b" and a.max_num_seqs == 4 and a.top_k == 5 and a.kv_fraction == 0.3 and a.disable_cuda_graph
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The measurement script runs on one GPU: for more it prints one line that says so and
+    exits with 2, before anything touches a GPU."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 2
+    lines = [l for l in r.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1 and "one GPU" in lines[0]
