@@ -187,7 +187,8 @@ def test_command_line_options_follow_the_reference():
     a = build_parser().parse_args([])
     assert (a.m, a.w, a.dtype, a.max_num_seqs, a.max_tokens, a.prefill_chunk_size) == (None, None, "bf16", 1, 16384, 8192)
     assert a.max_model_len is None and a.temperature is None and a.top_k is None and a.top_p is None
-    assert not a.ignore_eos and not a.disable_cuda_graph and a.seed is None and a.batch is None
+    assert not a.ignore_eos and not a.disable_cuda_graph and a.seed is None and a.batch is None and not a.interactive
+    assert build_parser().parse_args(["--i"]).interactive
     a = build_parser().parse_args(["--m", "x", "--prompts", "a|b", "--max-num-seqs", "4", "--top-k", "5", "--top-p", "0.9",
                                    "--temperature", "0.5", "--kv-fraction", "0.3", "--disable-cuda-graph"])
     assert a.prompts == "a|b" and a.max_num_seqs == 4 and a.top_k == 5 and a.kv_fraction == 0.3 and a.disable_cuda_graph

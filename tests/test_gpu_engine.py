@@ -242,6 +242,35 @@ def test_command_line(model_dirs, capsys):
     assert cli.main([]) == 2
 
 
+def test_command_line_interactive_chat(model_dirs, monkeypatch, capsys):
+    """`--i`: lines from the input are the user's turns of one conversation; the second answer
+    has the first exchange in its context; the end of the input clears the history, a second
+    end exits.  Greedy, so the first answer equals the one `generate_stream` gives for the
+    same chat."""
+    from xinfer_amd import Engine, EngineConfig, Message, SamplingParams, cli
+    lines = iter(["Hello there", "", "And again"])
+
+    def fake_input():
+        try:
+            return next(lines)
+        except StopIteration:
+            raise EOFError
+
+    monkeypatch.setattr("builtins.input", fake_input)
+    rc = cli.main(["--m", model_dirs["A"], "--i", "--max-tokens", "5", "--max-model-len", "128", "--temperature", "0",
+                   "--ignore-eos", "--page-size", "16", "--num-pages", "16", "--dtype", "f32"])
+    out = capsys.readouterr().out
+    assert rc == 0
+    assert out.count("Enter a new prompt") == 2 and out.count("Enter another prompt") == 3
+    assert "No prompt was given." in out and "Chat history cleared" in out and out.rstrip().endswith("Exiting.")
+    left = [int(l.split(":")[1]) for l in out.splitlines() if l.startswith("Tokens left:")]
+    assert len(left) == 2 and left[1] < left[0] < 128
+    engine = Engine(EngineConfig(model_id=model_dirs["A"], max_model_len=128, max_tokens=5, page_size=16, num_pages=16), "f32")
+    _, _, stream = engine.generate_stream(SamplingParams(temperature=0.0, ignore_eos=True), [Message("user", "Hello there")])
+    first = "".join(it.data for it in stream if it.datatype == "TOKEN")
+    assert first in out
+
+
 # ---- long decoding and first tokens ----------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_one_by_one(dtype, model_dirs):

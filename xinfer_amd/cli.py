@@ -39,6 +39,8 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--prefill-chunk-size", type=int, default=8192,
                    help="most prompt tokens of one request in a step")
     p.add_argument("--disable-cuda-graph", action="store_true", help="disable HIP graph replay of decode steps")
+    p.add_argument("--i", dest="interactive", action="store_true",
+                   help="interactive chat: prompts are read line by line, the conversation so far is the context")
     p.add_argument("--page-size", type=int, default=64, help="tokens per cache page")
     p.add_argument("--num-pages", type=int, default=None, help="cache pages (default: from --kv-fraction)")
     return p
@@ -54,8 +56,14 @@ def run(args) -> int:
     if not (args.m or args.w):
         print("Must provide model folder (--m or --w)!", file=sys.stderr)
         return 2
-    if args.prompt_ids:
-        prompts: List = [[int(t) for t in part.split(",") if t.strip()] for part in args.prompt_ids.split("|")]
+    interactive = bool(args.interactive)
+    if interactive and args.batch:
+        print("interactive mode is ignored in batch performance test.", file=sys.stderr)   # main.rs:58-60
+        interactive = False
+    if interactive:
+        prompts: List = []
+    elif args.prompt_ids:
+        prompts = [[int(t) for t in part.split(",") if t.strip()] for part in args.prompt_ids.split("|")]
     elif args.prompts:
         prompts = args.prompts.split("|")
     else:
@@ -82,6 +90,8 @@ def run(args) -> int:
     params = SamplingParams(temperature=args.temperature, top_k=args.top_k, top_p=args.top_p,
                             frequency_penalty=args.frequency_penalty,
                             presence_penalty=args.presence_penalty, ignore_eos=args.ignore_eos)
+    if interactive:
+        return _chat(engine, params, max_num_seqs * max_model_len)
     print("Start inference with", len(prompts), "prompts")
     outputs = engine.generate(prompts, [params] * len(prompts))
     outputs.sort(key=lambda o: o.seq_id)
@@ -102,6 +112,61 @@ def run(args) -> int:
     print(f"Decoded tokens: {total_decoded} in {decode_time:.2f}s "
           f"({total_decoded / max(decode_time, 0.001):.2f} tokens/s)")
     return 0
+
+
+def _chat(engine, params, total_tokens: int, lines=None, out=None) -> int:
+    """The reference's interactive mode (main.rs:320-560): every line is a user turn of one
+    conversation whose history is the context; the answer is printed as its tokens arrive.  An
+    empty line asks again; end of input (or Ctrl+C) clears the history if there is one and
+    exits if there is none."""
+    from . import Message
+    out = out or sys.stdout
+    lines = iter(lines) if lines is not None else None
+    history: List = []
+    left = total_tokens
+    while True:
+        print("Enter a new prompt (Press Ctrl+C to exit):" if not history else
+              "Enter another prompt to continue current chat (Press Ctrl+C to start a new chat):", file=out, flush=True)
+        try:
+            line = next(lines) if lines is not None else input()
+        except (EOFError, KeyboardInterrupt, StopIteration):
+            if not history:
+                print("Exiting.", file=out, flush=True)
+                return 0
+            print("Chat history cleared. Start a new conversation.", file=out, flush=True)
+            history.clear()
+            left = total_tokens
+            continue
+        text = line.strip()
+        if not text:
+            print("No prompt was given.", file=out, flush=True)
+            continue
+        if left <= 0:
+            print("No tokens left, press Ctrl+C to start a new chat session!", file=out, flush=True)
+            continue
+        history.append(Message("user", text))
+        try:
+            seq_id, prompt_length, stream = engine.generate_stream(params, list(history))
+        except Exception as ex:          # the conversation no longer fits: start over, as the reference does
+            print(f"Session unexpectedly ended because: {ex}", file=out, flush=True)
+            print("Chat history cleared. Start a new conversation.", file=out, flush=True)
+            history.clear()
+            left = total_tokens
+            continue
+        pieces: List[str] = []
+        decoded = 0
+        for item in stream:
+            if item.datatype == "TOKEN":
+                pieces.append(item.data)
+                print(item.data, end="", file=out, flush=True)
+            elif item.datatype == "TOKEN_ID":
+                decoded += 1
+            elif item.datatype == "ERROR":
+                print(f"\n{item.data}", file=out, flush=True)
+        print(file=out, flush=True)
+        history.append(Message("assistant", "".join(pieces)))
+        left = total_tokens - prompt_length - decoded
+        print(f"Tokens left: {left}", file=out, flush=True)
 
 
 def main(argv: Optional[List[str]] = None) -> int:
