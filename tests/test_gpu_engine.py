@@ -271,6 +271,33 @@ def test_command_line_interactive_chat(model_dirs, monkeypatch, capsys):
     assert first in out
 
 
+def test_stop_sequences(model_dirs):
+    """Generation ends at the token that completes a stop sequence, which is not appended; the
+    first tokens of a longer stop sequence stay; a stop that never completes changes nothing."""
+    from xinfer_amd import Engine, EngineConfig, SamplingParams
+    cfg = EngineConfig(model_id=model_dirs["A"], max_model_len=64, max_num_seqs=4, page_size=16, num_pages=16)
+    engine = Engine(cfg, "f32")
+    prompt = [5, 17, 3, 9]
+    # sampled with a seed of the request's own: the same tokens in every run, and varied ones
+    greedy = dict(temperature=1.5, seed=7, ignore_eos=True, max_tokens=12)
+    full = engine.generate([prompt], SamplingParams(**greedy))[0].token_ids
+    assert len(full) == 12
+    k = next(i for i in range(2, 12) if full[i] not in full[:i])            # its first occurrence is at i
+    one = engine.generate([prompt], SamplingParams(stop_token_ids=[[full[k]]], **greedy))[0]
+    assert one.token_ids == full[:k] and one.finish_reason == "stop"
+    j = next(i for i in range(2, 12) if full[i - 1:i + 1] not in [full[a - 1:a + 1] for a in range(1, i)])
+    two = engine.generate([prompt], SamplingParams(stop_token_ids=[[full[j - 1], full[j]]], **greedy))[0]
+    assert two.token_ids == full[:j] and two.finish_reason == "stop"
+    never = engine.generate([prompt], SamplingParams(stop_token_ids=[[full[3], full[3] + 1 if full[4] != full[3] + 1 else full[3] + 2]],
+                                                      **greedy))[0]
+    assert never.token_ids == full and never.finish_reason == "length"
+    # as text: the byte tokenizer maps a character below 128 to the token of its code
+    low = [i for i in range(1, 12) if full[i] < 128 and full[i] not in full[:i] and chr(full[i]).isprintable()]
+    if low:
+        txt = engine.generate([prompt], SamplingParams(stop_sequences=["", chr(full[low[0]])], **greedy))[0]
+        assert txt.token_ids == full[:low[0]] and txt.finish_reason == "stop"
+
+
 # ---- long decoding and first tokens ----------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_one_by_one(dtype, model_dirs):

@@ -34,6 +34,11 @@ class SamplingParams:
     frequency_penalty: Optional[float] = None
     presence_penalty: Optional[float] = None
     seed: Optional[int] = None          # per-request seed; default: the engine's seed and the request id
+    # Generation ends when the new token completes one of these (config.rs:807-809): texts, tokenised
+    # at admission, and/or token id sequences.  The completing token is not appended (as with EOS);
+    # the earlier tokens of a longer stop sequence stay in the output, as in the reference.
+    stop_sequences: Optional[List[str]] = None
+    stop_token_ids: Optional[List[List[int]]] = None
 
 
 @dataclass
@@ -52,7 +57,7 @@ class GenerationOutput:
     decoded_length: int
     decode_output: str
     token_ids: List[int] = field(default_factory=list)     # the generated token ids
-    finish_reason: str = ""                                 # "eos", "length", "max_model_len"
+    finish_reason: str = ""                                 # "eos", "stop", "length", "max_model_len"
 
 
 @dataclass(frozen=True)

@@ -46,6 +46,7 @@ class _Request:
     decode_finish: int = 0
     finish_reason: str = ""
     preemptions: int = 0
+    stops: List[List[int]] = field(default_factory=list)    # token sequences that end the generation
 
     @property
     def generated(self) -> List[int]:
@@ -120,6 +121,12 @@ class LLMEngine:
             raise ValueError(f"a prompt token is outside the vocabulary of {vocab}")
         max_tokens = params.max_tokens or self.econfig.max_tokens or DEFAULT_MAX_TOKENS
         max_tokens = max(1, min(max_tokens, self.max_model_len - len(prompt)))   # engine.rs:650-678
+        stops: List[List[int]] = [[int(t) for t in ids] for ids in (params.stop_token_ids or []) if len(ids)]
+        for text in params.stop_sequences or []:           # engine.rs:693-721: empty ones are skipped
+            if text:
+                ids = self.tokenizer.encode(text)
+                if ids:
+                    stops.append([int(t) for t in ids])
         rid = self._next_id
         self._next_id += 1
         self.scheduler.add(rid, len(prompt), max_tokens)
@@ -128,7 +135,7 @@ class LLMEngine:
         seed, stream = (params.seed, 0) if params.seed is not None else (self.seed, rid)
         self._requests[rid] = _Request(
             rid, prompt, len(prompt), max_tokens, params,
-            resolve_strategy(params, self.generation_cfg), seed, stream, prompt_start=_now_ms())
+            resolve_strategy(params, self.generation_cfg), seed, stream, prompt_start=_now_ms(), stops=stops)
         return rid
 
     # ---- the loop ------------------------------------------------------------------------
@@ -163,7 +170,9 @@ class LLMEngine:
                 if not r.generated:
                     r.decode_start = now
                 reason = ""
-                if tok in self.eos_token_ids and not r.params.ignore_eos:
+                if _completes_a_stop(r.stops, r.generated, int(tok)):
+                    reason = "stop"
+                elif tok in self.eos_token_ids and not r.params.ignore_eos:
                     reason = "eos"
                 else:
                     r.tokens.append(int(tok))
@@ -238,6 +247,19 @@ class LLMEngine:
         is rendered with the chat template and completed."""
         prompts = [self.tokenizer.apply_chat_template(list(m)) for m in message_list]
         return self.generate(prompts, list(params))
+
+
+def _completes_a_stop(stops: List[List[int]], generated: Sequence[int], token: int) -> bool:
+    """Whether `token` after the tokens generated so far completes a stop sequence
+    (scheduler.rs:1459-1490: a one-token stop matches the token; a longer one needs its first
+    tokens at the end of the output)."""
+    for stop in stops:
+        if stop[-1] != token:
+            continue
+        n = len(stop) - 1
+        if n == 0 or (n <= len(generated) and list(generated[len(generated) - n:]) == stop[:-1]):
+            return True
+    return False
 
 
 class EngineStream:
