@@ -1,10 +1,12 @@
 // y[M,N] = x[M,K] @ w[N,K]^T in bfloat16 for few rows (decode batches, M <= 64): bound by
 // the one pass over w, so the kernel is a streaming read of w through the matrix cores.
 //
-// A workgroup owns 16*RT rows of w (output features) and one of KS slices of K.  Its NW
-// waves take consecutive parts of the slice and merge through LDS in a fixed order, so an
-// output element's value depends on (K, KS, NW) alone, never on M, on RT or on what else is
-// in the batch.  Per 32-wide k step a wave issues v_mfma_f32_16x16x32_bf16 with A = 16 rows
+// A workgroup owns R output features (rows of w; R <= 16*RT, any number, so that the grid can
+// be a multiple of the compute units) and one of KS slices of K.  Its NW waves take
+// consecutive parts of the slice and merge through LDS in a fixed order, so an output
+// element's value depends on (K, KS, NW) alone, never on M, on RT, on R or on what else is in
+// the batch.  A wave keeps U steps of loads in flight: a step's registers are loaded again, U
+// steps ahead, right after its products.  Per 32-wide k step a wave issues v_mfma_f32_16x16x32_bf16 with A = 16 rows
 // of w (lane l: row l%16, k group l/16, one 16-byte load) and B = x^T (lane l: token l%16,
 // same k group), for RT row tiles and MT tiles of 16 tokens: every x operand is used RT
 // times and every w operand MT times.  x is small and is read from L2.
