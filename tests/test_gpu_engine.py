@@ -766,3 +766,31 @@ def test_toy_routed_feed_forward_and_position_encoding(tmp_path):
                         ("portions", harness.trace_portions(reqs))):
         runner = ModelRunner(model, page_size=8, num_pages=14, max_requests=2)
         harness.compare(harness.replay(runner, steps), ref, harness.TOL["float32"], f"toy routed {what}")
+
+
+# ---- the measurement script -------------------------------------------------------------------------------
+def test_bench_line_keeps_its_contract():
+    """`bench.py` with two layers: one JSON line with the contract's fields, a flat `config` of at
+    most 20 keys that names both layer counts, the prefill and roofline records and the two points."""
+    import json
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--layers", "2", "--steps", "4", "--warmup", "1"],
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [l for l in r.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1
+    d = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+                "vs_baseline", "dtype", "data", "config", "prefill", "roofline", "points"):
+        assert key in d, key
+    assert d["n_gpus"] == 1 and d["steps"] == 4 and d["warmup"] == 1 and d["higher_is_better"] is True
+    assert d["value"] > 0 and abs(d["value"] - 8 / (d["ms_per_step"] / 1e3)) / d["value"] < 1e-3
+    cfg = d["config"]
+    assert len(cfg) <= 20 and all(not isinstance(v, (dict, list)) for v in cfg.values())
+    assert cfg["layers"] == 2 and cfg["layers_of_model"] == 36 and cfg["global_batch"] == 8 and cfg["seq_len"] == 4096
+    assert set(d["prefill"]) == {"value", "tokens", "ms", "frac"} and d["prefill"]["tokens"] == 2048
+    assert d["roofline"]["bound"] == "hbm" and d["roofline"]["peak"] == 8000.0 and d["roofline"]["unit"] == "GB/s"
+    assert abs(d["roofline"]["frac"] - d["roofline"]["achieved"] / 8000.0) < 1e-3
+    assert set(d["points"]) == {"decode_b1", "decode_b64"}
