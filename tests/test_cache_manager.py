@@ -5,7 +5,9 @@ import random
 
 import pytest
 
-from xinfer_amd.cache import CacheError, CacheGroup, OutOfPages, PagedCacheManager
+import numpy as np
+
+from xinfer_amd.cache import CacheError, CacheGroup, DecodeStepError, OutOfPages, PagedCacheManager
 
 
 def test_pages_slots_and_tables():
@@ -38,6 +40,53 @@ def test_pages_slots_and_tables():
     cm.reserve(6, 16 * 6)
     assert cm.block_table(6) == [4, 5, 6, 7, 0, 1]
     cm.check()
+
+
+def test_decode_step_in_one_call_matches_the_builder():
+    """The one-call preparation of a step of single tokens fills the two upload buffers with
+    what reserve + build_batch give, in the runner's order, and refuses what the step function
+    refuses."""
+    def manager():
+        cm = PagedCacheManager([CacheGroup(8, 12), CacheGroup(8, 12, window=10)], max_requests=3)
+        for rid, n in ((4, 13), (7, 1), (2, 24)):
+            cm.add_request(rid)
+            cm.reserve(rid, n)
+            cm.commit(rid, n)
+        return cm
+    a, b = manager(), manager()
+    rids = np.array([7, 2, 4], np.int64)
+    toks = np.array([3, 250, 0], np.int32)
+    B, G, P = 3, 2, 5
+    out32 = np.full(6 * B + 1 + G * B * P, -7, np.int32)
+    out64 = np.full((2 + G) * B, -7, np.int64)
+    longest, similar = a.decode_step(rids, toks, True, 256, 64, P, np.array([2, 0], np.int32), out32, out64)
+    b.reserve_many(rids, np.ones(B, np.int32))
+    w = b.build_batch(rids, np.ones(B, np.int32), max_pages=P)
+    assert longest == 25 and not similar and [a.block_table(r, g) for r in (7, 2, 4) for g in (0, 1)] == \
+        [b.block_table(r, g) for r in (7, 2, 4) for g in (0, 1)]
+    want32 = np.concatenate([toks, w.positions, w.tok_seq, w.cu_q, w.ctx_lens, [2, 0, 0], w.block_tables.reshape(-1)])
+    want64 = np.concatenate([w.state_slots.astype(np.int64), w.slots.reshape(-1), [-1, -1, -1]])
+    assert out32.tolist() == want32.tolist() and out64.tolist() == want64.tolist()
+    a.commit_many(rids, np.ones(B, np.int32))
+    assert a.lengths(np.array([4, 7, 2, 99], np.int64)).tolist() == [14, 2, 25, -1]
+    a.check()
+    assert a.decode_step(np.array([4, 7, 2], np.int64), toks, True, 256, 64, P, np.array([], np.int32), out32, out64)[1] is False
+    for bad_rids, bad_toks, max_pos, rows, kind, entry in (
+            ([7, 99, 4], [1, 1, 1], 64, [0], -1, 1), ([7, 2, 7], [1, 1, 1], 64, [0], -2, 2),
+            ([7, 2, 4], [1, 1, 1], 25, [0], -3, 1), ([7, 2, 4], [1, 256, 1], 64, [0], -4, 1),
+            ([7, 2, 4], [1, 1, 1], 64, [3], -6, 0)):
+        with pytest.raises(DecodeStepError) as e:
+            a.decode_step(np.array(bad_rids, np.int64), np.array(bad_toks, np.int32), True, 256, max_pos, P,
+                          np.array(rows, np.int32), out32, out64)
+        assert (e.value.kind, e.value.entry) == (kind, entry)
+    small = PagedCacheManager([CacheGroup(8, 1)], max_requests=2)
+    for rid in (0, 1):
+        small.add_request(rid)
+    small.reserve(0, 8)
+    small.commit(0, 8)
+    with pytest.raises(OutOfPages):
+        small.decode_step(np.array([0], np.int64), np.array([1], np.int32), True, 256, 64, 4, np.array([0], np.int32),
+                          np.zeros(11, np.int32), np.zeros(3, np.int64))
 
 
 def test_reserve_is_all_or_nothing():

@@ -1,1 +1,1 @@
-from .manager import BatchArrays, CacheError, CacheGroup, OutOfPages, PagedCacheManager
+from .manager import BatchArrays, CacheError, CacheGroup, DecodeStepError, OutOfPages, PagedCacheManager

@@ -60,6 +60,7 @@ def _bind(lib):
         "xi_cm_last_error": (ctypes.c_char_p, [vp]),
         "xi_cm_max_table_len": (i, [vp, i, _I64P]),
         "xi_cm_lengths": (None, [vp, i, _I64P, _I64P]),
+        "xi_cm_decode_step": (i, [vp, i, _I64P, _I32P, i, i, i64, i, _I32P, i, _I32P, _I64P, _I32P, _I32P]),
         "xi_cm_reserve_many": (i, [vp, i, _I64P, _I32P]),
         "xi_cm_commit_many": (i, [vp, i, _I64P, _I32P]),
         "xi_cm_build_batch": (i, [vp, i, _I64P, _I32P, _I32P, _I32P, _I32P, _I32P, _I32P,
@@ -86,6 +87,15 @@ class BatchArrays:
     state_slots: np.ndarray    # [B] int32
     slots: np.ndarray          # [G, T] int64
     block_tables: np.ndarray   # [G, B, max_pages] int32
+
+
+class DecodeStepError(Exception):
+    """`decode_step` refused entry `entry`: kind -1 not live, -2 twice, -3 past the model's
+    positions, -4 token outside the vocabulary, -6 a wanted row outside the step, -7 no batch."""
+
+    def __init__(self, kind: int, entry: int):
+        super().__init__(f"decode step: kind {kind}, entry {entry}")
+        self.kind, self.entry = kind, entry
 
 
 class PagedCacheManager:
@@ -193,6 +203,26 @@ class PagedCacheManager:
         if self._lib.xi_cm_commit_many(self._h, int(rids.size), rids.ctypes.data_as(_I64P),
                                        counts.ctypes.data_as(_I32P)) != 0:
             raise CacheError(self._lib.xi_cm_last_error(self._h).decode())
+
+    def decode_step(self, rids: np.ndarray, tokens: np.ndarray, reserve: bool, vocab: int, max_positions: int,
+                    max_pages: int, rows: np.ndarray, out32: np.ndarray, out64: np.ndarray):
+        """A step of one token per request prepared in one call (see xi_cm_decode_step): fills the
+        two upload buffers and returns (longest cached length, lengths are similar).  Raises
+        CacheError(kind, entry) for a request that cannot take part, OutOfPages if pages run out."""
+        stats = np.zeros(2, np.int32)
+        bad = np.zeros(1, np.int32)
+        rc = self._lib.xi_cm_decode_step(
+            self._h, int(rids.size), rids.ctypes.data_as(_I64P), tokens.ctypes.data_as(_I32P), int(bool(reserve)),
+            int(vocab), int(max_positions), int(max_pages), rows.ctypes.data_as(_I32P), int(rows.size),
+            out32.ctypes.data_as(_I32P), out64.ctypes.data_as(_I64P), stats.ctypes.data_as(_I32P),
+            bad.ctypes.data_as(_I32P))
+        if rc == 0:
+            return int(stats[0]), bool(stats[1])
+        b = int(bad[0])
+        if rc == -5:
+            msg = self._lib.xi_cm_last_error(self._h).decode()
+            raise OutOfPages(f"request {int(rids[b])} needs pages for 1 more tokens: {msg}")
+        raise DecodeStepError(rc, b)
 
     def release(self, rid: int) -> int:
         r = self._lib.xi_cm_release(self._h, rid)

@@ -21,7 +21,7 @@ from typing import Any, Dict, List, Optional, Sequence, Tuple
 import numpy as np
 import torch
 
-from ..cache import BatchArrays, CacheGroup, OutOfPages, PagedCacheManager
+from ..cache import DecodeStepError, BatchArrays, CacheGroup, OutOfPages, PagedCacheManager
 from ..parts import LayerCache, StepContext
 from .model import CausalLM
 
@@ -75,6 +75,24 @@ class _Staging:
             raise ValueError("staging: the fixed device buffer does not fit this step's arrays")
         dst.copy_(pin[:n], non_blocking=True)
         return dst, offsets
+
+    def pinned(self, dtype: torch.dtype, n: int) -> np.ndarray:
+        """The pinned buffer of `dtype` with room for n elements, free to be written (the copy
+        of the step before has left it)."""
+        pin = self._pin[dtype]
+        if pin is None or pin.numel() < n:
+            pin = torch.empty((max(1024, 1 << (n - 1).bit_length()),), dtype=dtype, pin_memory=True)
+            self._pin[dtype] = pin
+        if self._done is not None:
+            self._done.synchronize()
+            self._done = None
+        return pin.numpy()
+
+    def push(self, dtype: torch.dtype, n: int, dst: torch.Tensor) -> None:
+        """Copies the first n elements of the pinned buffer into `dst`."""
+        if dst.numel() != n or dst.dtype != dtype:
+            raise ValueError("staging: the fixed device buffer does not fit this step's arrays")
+        dst.copy_(self._pin[dtype][:n], non_blocking=True)
 
     def mark(self) -> None:
         self._done = torch.cuda.Event()
@@ -164,7 +182,12 @@ class ModelRunner:
         if not entries:
             return torch.empty((0, spec.vocab_size), dtype=torch.float32, device=self.device)
         B = len(entries)
-        if all(len(e.tokens) == 1 for e in entries):
+        single = all(len(e.tokens) == 1 for e in entries)
+        if single and self.use_graphs and B <= self.graph_max_batch and self._graphs:
+            logits = self._decode_recorded(entries, reserved)
+            if logits is not None:
+                return logits
+        if single:
             # a step of single tokens (the hot path of decoding): checked and reserved in a few
             # calls for all entries together
             rid_arr = np.fromiter((e.request for e in entries), np.int64, B)
@@ -229,6 +252,50 @@ class ModelRunner:
         if not reserved:
             self.cache.commit_many(rid_arr, counts_arr)
         return logits
+
+    def _decode_recorded(self, entries: Sequence[StepEntry], reserved: bool) -> Optional[torch.Tensor]:
+        """A step of single tokens whose graph is recorded already: one call into the cache
+        manager checks the requests, reserves their pages and writes the step's arrays straight
+        into the pinned buffers; two copies and a replay follow.  Returns None (nothing done
+        but, possibly, the reservation, which the general path repeats harmlessly) if the step
+        has no recorded graph yet."""
+        spec = self.model.spec
+        B = len(entries)
+        G = len(self.cache.groups)
+        P = self._max_table
+        rid_arr = np.fromiter((e.request for e in entries), np.int64, B)
+        tokens = np.fromiter((e.tokens[0] for e in entries), np.int32, B)
+        rows = np.fromiter((b for b, e in enumerate(entries) for _ in e.want), np.int32)
+        if any(w != 0 for e in entries for w in e.want):
+            raise StepError("a wanted place is outside an entry's 1 tokens")
+        n32, n64 = 6 * B + 1 + G * B * P, (2 + G) * B
+        host32 = self._staging.pinned(torch.int32, n32)
+        host64 = self._staging.pinned(torch.int64, n64)
+        try:
+            longest, similar = self.cache.decode_step(rid_arr, tokens, not reserved, spec.vocab_size,
+                                                      spec.max_positions, P, rows, host32, host64)
+        except DecodeStepError as ex:
+            rid = int(rid_arr[ex.entry]) if 0 <= ex.entry < B else -1
+            raise StepError({-1: f"request {rid} is not live", -2: f"request {rid} appears twice in one step",
+                             -3: f"request {rid}: its tokens exceed the model's {spec.max_positions} positions",
+                             -4: f"a token id is outside the vocabulary of {spec.vocab_size}"}.get(
+                                 ex.kind, f"the step could not be prepared ({ex.kind})")) from None
+        bucket = 1024
+        while bucket < longest:
+            bucket *= 4
+        g = self._graphs.get((B, bucket, similar))
+        if g is None:
+            return None
+        self._staging.push(torch.int32, n32, g.dev32)
+        self._staging.push(torch.int64, n64, g.dev64)
+        self._staging.mark()
+        g.graph.replay()
+        self.graph_replays += 1
+        if not reserved:
+            self.cache.commit_many(rid_arr, np.ones(B, np.int32))
+        if rows.size == B and np.array_equal(rows, np.arange(B)):
+            return g.logits.clone()
+        return g.logits.index_select(0, g.want[:rows.size])
 
     # ---- index arrays on the device -------------------------------------------------
     def _context(self, a: BatchArrays, ids32: np.ndarray, rows32: np.ndarray, dst32=None, dst64=None,
