@@ -240,6 +240,23 @@ def test_linear_folded_norm_refuses():
         kernels.linear_fold_in(x[:4].contiguous(), torch.zeros((4, 600), device=DEV), 1e-6, w)
 
 
+def test_linear_skinny_plan_fills_the_compute_units():
+    """The shapes the streaming product chooses: grids that are multiples of the 256 compute
+    units where the width allows (a workgroup may own a number of features that is no multiple
+    of 16), slices of K for narrow outputs only when asked, and the same slices for every M."""
+    from xinfer_amd import kernels
+    for (N, K, gated) in ((4096, 4096, False), (5120, 5120, False), (6144, 4096, False), (5120, 17408, False),
+                          (12288, 4096, True)):
+        for M in (1, 8, 16):
+            ks, rt, rows, wgs = kernels.linear_skinny_plan(M, N, K, gated)
+            assert ks == 1 and rows <= 16 * rt // (2 if gated else 1) and wgs % 256 == 0, (N, K, gated, M, rt, rows, wgs)
+    assert kernels.linear_skinny_plan(8, 5120, 5120)[2] == 20
+    assert kernels.linear_skinny_plan(16, 17408, 5120, gated=True)[3] == 512
+    for M in (1, 17, 64):
+        assert kernels.linear_skinny_plan(M, 4096, 12288, allow_split=True)[0] == 4
+        assert kernels.linear_skinny_plan(M, 151936, 4096, allow_split=True)[0] == 1
+
+
 def test_linear_skinny_refuses():
     from xinfer_amd import kernels
     x = torch.zeros((65, 64), dtype=torch.bfloat16, device=DEV)

@@ -412,6 +412,7 @@ def linear_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dt
         N //= 2
     if M > SKINNY_MAX_ROWS or K % 8:
         raise KernelError(f"linear_skinny: M={M} must be <= {SKINNY_MAX_ROWS} and K={K} a multiple of 8")
+    assert SKINNY_MAX_ROWS == int(lib().xi_linear_skinny_max_rows())
     slices = int(lib().xi_linear_skinny_slices(N, K, int(bool(gated)), int(bool(allow_split))))
     if slices > 1:
         out_dtype, shape = torch.float32, (slices, M, N)
@@ -424,6 +425,16 @@ def linear_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dt
     _ok(lib().xi_linear_skinny(_p(x), _p(w), _p(out), M, N, K, _code(out, "linear_skinny"), int(bool(gated)),
                                int(bool(allow_split)), int(row_tiles), int(waves), _stream()))
     return out
+
+
+def linear_skinny_plan(M: int, N: int, K: int, gated: bool = False, allow_split: bool = False):
+    """What `linear_skinny` chooses for these sizes: (slices of K, row tiles per workgroup, output
+    features per workgroup, workgroups).  Only the slices change a sum's order."""
+    L = lib()
+    ks = int(L.xi_linear_skinny_slices(N, K, int(bool(gated)), int(bool(allow_split))))
+    rt = int(L.xi_linear_skinny_row_tiles(M, N, K, int(bool(gated)), int(bool(allow_split))))
+    rows = int(L.xi_linear_skinny_rows(M, N, K, int(bool(gated)), int(bool(allow_split))))
+    return ks, rt, rows, -(-N // rows) * ks
 
 
 FOLD_ROWS = 16            # most rows of the products that carry a folded norm between them
