@@ -1,6 +1,7 @@
 """Tiny Qwen3 configurations for tests.  A and B differ in every size and option; W adds
-a sliding window on some layers (two cache groups) and a head size that is no power of
-two; all have widths and vocabularies that are no power of two where they can."""
+a sliding window on some layers (two cache groups), a head size that is no power of
+two and biases on the q, k and v projections; all have widths and vocabularies that are
+no power of two where they can."""
 
 def _cfg(**kw):
     base = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", hidden_act="silu")
@@ -23,7 +24,7 @@ TINY = {
         config=_cfg(num_hidden_layers=3, hidden_size=80, num_attention_heads=5, num_key_value_heads=5,
                     head_dim=48, intermediate_size=176, vocab_size=300, rope_theta=50000.0,
                     rms_norm_eps=1e-5, tie_word_embeddings=False, max_position_embeddings=320,
-                    sliding_window=24,
+                    sliding_window=24, attention_bias=True,
                     layer_types=["sliding_attention", "full_attention", "sliding_attention"]),
         seed=2, linear_std=0.05, norm_std=0.2, page_size=16),
 }

@@ -126,15 +126,21 @@ def swiglu(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
 
 def attention_block(x, W, prefix, c, positions, cos, sin, window):
     """q/k/v projections, per-head q_norm and k_norm before RoPE, RoPE on q and k, causal
-    GQA, o_proj; no biases.  /root/reference/src/models/layers/attention.rs:805-828
-    (projections), 709-748 (per-head norm on [T*heads, d]), 872-879 (RoPE), 947-958
-    (attention), 976 (o_proj)."""
+    GQA, o_proj.  With `attention_bias` q, k and v have a bias each, o_proj has none.
+    /root/reference/src/models/layers/attention.rs:805-828 (projections), 388-399 (the three
+    biases), 596-608 (o_proj without), 709-748 (per-head norm on [T*heads, d]), 872-879
+    (RoPE), 947-958 (attention), 976 (o_proj)."""
     T = x.shape[0]
     nq, nkv, d = c["num_attention_heads"], c["num_key_value_heads"], c["head_dim"]
     eps = c["rms_norm_eps"]
-    q = (x @ W[f"{prefix}.q_proj.weight"].T).reshape(T, nq, d)
-    k = (x @ W[f"{prefix}.k_proj.weight"].T).reshape(T, nkv, d)
-    v = (x @ W[f"{prefix}.v_proj.weight"].T).reshape(T, nkv, d)
+    q = x @ W[f"{prefix}.q_proj.weight"].T
+    k = x @ W[f"{prefix}.k_proj.weight"].T
+    v = x @ W[f"{prefix}.v_proj.weight"].T
+    if c.get("attention_bias"):
+        q = q + W[f"{prefix}.q_proj.bias"]
+        k = k + W[f"{prefix}.k_proj.bias"]
+        v = v + W[f"{prefix}.v_proj.bias"]
+    q, k, v = q.reshape(T, nq, d), k.reshape(T, nkv, d), v.reshape(T, nkv, d)
     q = rms_norm(q, W[f"{prefix}.q_norm.weight"], eps)
     k = rms_norm(k, W[f"{prefix}.k_norm.weight"], eps)
     q = apply_rope(q, positions, cos, sin)

@@ -103,7 +103,7 @@ def _engine(model_dir, name, dtype, **kw):
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_greedy_generation_tiny_a(dtype, model_dirs):
-    """BASELINE workload of tiny A: prompts of 5, 17 and 33 tokens, 16 greedy tokens each."""
+    """Workload of tiny configuration A: prompts of 5, 17 and 33 tokens, 16 greedy tokens each."""
     from xinfer_amd import SamplingParams
     rng = random.Random(0)
     prompts = [harness.random_prompt(rng, n, 256) for n in (5, 17, 33)]
@@ -126,7 +126,7 @@ def test_greedy_generation_tiny_a(dtype, model_dirs):
 
 
 def test_tiny_b_workload_chunked_and_sampled(model_dirs):
-    """BASELINE workload of tiny B: prompts 1, 9, 64, 130, 200, chunk 48 mixed with decode,
+    """Workload of tiny configuration B: prompts 1, 9, 64, 130, 200, chunk 48 mixed with decode,
     temperature 0.8 with a seed, 24 tokens each.  A request's tokens do not depend on what it was
     batched with: alone and together give the same tokens (float32)."""
     from xinfer_amd import SamplingParams

@@ -389,6 +389,45 @@ def test_qk_norm_rope_kv_many_tokens(nq, nkv, d, rot, interleaved):
     assert torch.equal(got_v, want_v)
 
 
+@pytest.mark.parametrize("dtype,T,nq,nkv,d,rot,interleaved", [
+    (torch.float32, 11, 3, 1, 48, 48, False), (torch.bfloat16, 11, 4, 2, 32, 16, True),
+    (torch.bfloat16, 150, 5, 5, 48, 48, False), (torch.bfloat16, 150, 2, 1, 128, 64, True)])
+def test_qk_norm_rope_kv_bias(dtype, T, nq, nkv, d, rot, interleaved):
+    """A bias on the packed projection is added before the norm (q, k) and before the store
+    (v), in float32: both kernels (one wave per head; 16 bytes per lane from 128 tokens on)
+    against norm(x + b) rotated, and v + b rounded once."""
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(23)
+    page, pages, eps = 8, 24, 1e-5
+    positions = torch.randint(0, 200, (T,), generator=g).to(torch.int32)
+    cos, sin = plain.rope_tables(10000.0, rot, 200)
+    width = (nq + 2 * nkv) * d
+    qkv = _rand((T, width), dtype, g)
+    bias = torch.randn(width, generator=g) * 0.5
+    qw, kw = 1 + 0.3 * torch.randn(d, generator=g), 1 + 0.3 * torch.randn(d, generator=g)
+    slots = torch.randperm(pages * page, generator=g)[:T].to(torch.int64)
+    vt_form = dtype == torch.bfloat16
+    kc = torch.zeros((pages, nkv, page, d), dtype=dtype, device=DEV)
+    vc = torch.zeros((pages, nkv, d, page) if vt_form else (pages, nkv, page, d), dtype=dtype, device=DEV)
+    q_out = kernels.qk_norm_rope_kv(qkv.to(DEV), qw.to(DEV), kw.to(DEV), eps, cos.to(DEV), sin.to(DEV), rot, interleaved,
+                                    positions.to(DEV), slots.to(DEV), kc, vc, nq, nkv, d, v_transposed=vt_form,
+                                    bias=bias.to(DEV))
+    x = (qkv.double() + bias.double()).reshape(T, nq + 2 * nkv, d)
+    q = _rope_ref(plain.rms_norm(x[:, :nq], qw.double(), eps), positions.long(), cos, sin, rot, interleaved)
+    k = _rope_ref(plain.rms_norm(x[:, nq:nq + nkv], kw.double(), eps), positions.long(), cos, sin, rot, interleaved)
+    v = (qkv.float() + bias).to(dtype).reshape(T, nq + 2 * nkv, d)[:, nq + nkv:]
+    tol = _tol(dtype)
+    assert (q_out.cpu().double() - q).abs().max() / q.abs().max() < tol
+    got_k = kc.cpu().double().permute(0, 2, 1, 3).reshape(pages * page, nkv, d)
+    got_v = (vc.cpu().permute(0, 3, 1, 2) if vt_form else vc.cpu().permute(0, 2, 1, 3)).reshape(pages * page, nkv, d)
+    assert (got_k[slots] - k).abs().max() / k.abs().max() < tol
+    assert torch.equal(got_v[slots], v)
+    with pytest.raises(kernels.KernelError, match="bias"):
+        kernels.qk_norm_rope_kv(qkv.to(DEV), qw.to(DEV), kw.to(DEV), eps, cos.to(DEV), sin.to(DEV), rot, interleaved,
+                                positions.to(DEV), slots.to(DEV), kc, vc, nq, nkv, d, v_transposed=vt_form,
+                                bias=bias[:-1].contiguous().to(DEV))
+
+
 def _paged_case(g, dtype, nq, nkv, d, page, seqs, extra_pages=3):
     """Random K/V of several sequences laid into a paged cache under a shuffled page map.
     `seqs` = list of (context length, number of query tokens at its end)."""

@@ -157,3 +157,28 @@ def test_layer_order_norm_before_mixer(tmp_path):
     want = plain.rms_norm(x, W["model.norm.weight"], 0.0) @ W["model.embed_tokens.weight"].T
     assert torch.allclose(a.double(), want, atol=1e-6)
     assert not torch.allclose(a, base, atol=1e-4)
+
+
+def test_bias_is_one_more_input_column(tmp_path):
+    """A bias on q, k and v is what a constant input of 1 with the bias as its weight column
+    gives: the attention block with `attention_bias` equals the block without, run on [x, 1]
+    with weights [W, b].  A bias added after the norm or the rotation, or one on o_proj, fails."""
+    pm = _tiny_weights("W", tmp_path)
+    c, W = pm.config, pm.weights
+    assert c["attention_bias"]
+    p = "model.layers.1.self_attn"
+    T, H = 9, c["hidden_size"]
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(T, H, generator=g, dtype=torch.float64)
+    W64 = {k: v.double() for k, v in W.items() if k.startswith(p)}
+    assert float(W64[f"{p}.k_proj.bias"].abs().max()) > 0
+    positions = torch.arange(3, 3 + T)
+    cos, sin = plain.rope_tables(c["rope_theta"], c["head_dim"], 64)
+    with_bias = plain.attention_block(x, W64, p, c, positions, cos, sin, None)
+    W1 = dict(W64)
+    for n in ("q", "k", "v"):
+        W1[f"{p}.{n}_proj.weight"] = torch.cat([W64[f"{p}.{n}_proj.weight"], W64[f"{p}.{n}_proj.bias"][:, None]], dim=1)
+    x1 = torch.cat([x, torch.ones(T, 1, dtype=torch.float64)], dim=1)
+    no_bias = plain.attention_block(x1, W1, p, dict(c, attention_bias=False), positions, cos, sin, None)
+    assert torch.allclose(with_bias, no_bias, atol=1e-12)
+    assert f"{p}.o_proj.bias" not in W

@@ -211,9 +211,13 @@ __global__ void silu_mul_vec8_kernel(const bf16* __restrict__ gu, bf16* __restri
 //   slot = page*page_size + offset (reference slot formula runner.rs:1344-1362); with
 //   v_transposed the V pool is [page, kv_head, d, offset] (what the MFMA attention reads).
 //   A negative slot means: do not store (the token's cache belongs to another run).
+//   `bias` (float32, one value per element of the packed row, or null) is the projections'
+//   bias: it is added here, in float32, to the product the row holds (q, k and v alike;
+//   reference attention.rs:819-828 adds it in the linear layer).
 // ---------------------------------------------------------------------------------
 template <typename T>
-__global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, const float* __restrict__ qw,
+__global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, const float* __restrict__ bias,
+                                       const float* __restrict__ qw,
                                        const float* __restrict__ kw, float eps,
                                        const float* __restrict__ cos_t,
                                        const float* __restrict__ sin_t, int rot, int interleaved,
@@ -228,6 +232,7 @@ __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, const float* _
   const int t = (int)(wid / heads);
   const int h = (int)(wid - (long long)t * heads);
   const T* src = qkv + (size_t)t * heads * d + (size_t)h * d;
+  const float* bs = bias ? bias + (size_t)h * d : nullptr;
 
   T* dst;
   const float* w = nullptr;
@@ -244,7 +249,8 @@ __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, const float* _
     const int kvh = is_k ? h - nq : h - nq - nkv;
     if (!is_k && v_transposed) {  // V kept as [page, kv_head, d, offset]
       T* vt = v_cache + ((size_t)page * nkv + kvh) * d * page_size + off;
-      for (int i = lane; i < d; i += kWave) vt[(size_t)i * page_size] = src[i];
+      for (int i = lane; i < d; i += kWave)
+        vt[(size_t)i * page_size] = bs ? from_float<T>(to_float(src[i]) + bs[i]) : src[i];
       return;
     }
     T* cache = is_k ? k_cache : v_cache;
@@ -253,7 +259,7 @@ __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, const float* _
     rotate = is_k;
   }
   if (!rotate) {  // v: plain copy
-    for (int i = lane; i < d; i += kWave) dst[i] = src[i];
+    for (int i = lane; i < d; i += kWave) dst[i] = bs ? from_float<T>(to_float(src[i]) + bs[i]) : src[i];
     return;
   }
   // The kernel lives on latency: everything that can be asked for at once is.  A lane holds
@@ -269,8 +275,8 @@ __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, const float* _
     const bool ok = i < half;
     const int ia = interleaved ? 2 * i : i;
     const int ib = interleaved ? 2 * i + 1 : i + half;
-    xa[p] = ok ? to_float(src[ia]) : 0.f;
-    xb[p] = ok ? to_float(src[ib]) : 0.f;
+    xa[p] = ok ? to_float(src[ia]) + (bs ? bs[ia] : 0.f) : 0.f;
+    xb[p] = ok ? to_float(src[ib]) + (bs ? bs[ib] : 0.f) : 0.f;
     wa[p] = (ok && w) ? w[ia] : 1.f;
     wb[p] = (ok && w) ? w[ib] : 1.f;
   }
@@ -278,7 +284,7 @@ __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, const float* _
   for (int p = 0; p < 4; ++p) {
     const int i = rot + lane + kWave * p;
     const bool ok = i < d;
-    xt[p] = ok ? to_float(src[i]) : 0.f;
+    xt[p] = ok ? to_float(src[i]) + (bs ? bs[i] : 0.f) : 0.f;
     wt[p] = (ok && w) ? w[i] : 1.f;
   }
   const float* c = cos_t + (size_t)pos * half;
@@ -331,7 +337,7 @@ __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, const float* _
 struct alignas(16) bf16x8v { bf16 v[8]; };
 
 __global__ __launch_bounds__(1024) void qk_norm_rope_kvt_bf16_kernel(
-    const bf16* __restrict__ qkv, const float* __restrict__ qw, const float* __restrict__ kw, float eps,
+    const bf16* __restrict__ qkv, const float* __restrict__ bias, const float* __restrict__ qw, const float* __restrict__ kw, float eps,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot, int interleaved,
     const int* __restrict__ positions, const long long* __restrict__ slots, bf16* __restrict__ q_out,
     bf16* __restrict__ k_cache, bf16* __restrict__ vt_cache, int page_size, int n_tok, int nq, int nkv, int d) {
@@ -354,7 +360,13 @@ __global__ __launch_bounds__(1024) void qk_norm_rope_kvt_bf16_kernel(
     bf16* vs = reinterpret_cast<bf16*>(smem_raw);  // [tpw][d + 2]
     const int vstride = d + 2;                      // an odd number of 32-bit words per row
     if (on) {
-      const uint4 raw = *reinterpret_cast<const uint4*>(qkv + ((size_t)t * heads + h) * d + 8 * c);
+      uint4 raw = *reinterpret_cast<const uint4*>(qkv + ((size_t)t * heads + h) * d + 8 * c);
+      if (bias) {
+        bf16x8v x = *reinterpret_cast<const bf16x8v*>(&raw);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x.v[e] = from_float<bf16>(to_float(x.v[e]) + bias[(size_t)h * d + 8 * c + e]);
+        raw = *reinterpret_cast<const uint4*>(&x);
+      }
       unsigned* dst = reinterpret_cast<unsigned*>(vs + tl * vstride + 8 * c);
       dst[0] = raw.x;
       dst[1] = raw.y;
@@ -381,7 +393,7 @@ __global__ __launch_bounds__(1024) void qk_norm_rope_kvt_bf16_kernel(
     bf16x8v x;
     if (on) x = *reinterpret_cast<const bf16x8v*>(qkv + ((size_t)t * heads + h) * d + 8 * c);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = on ? to_float(x.v[e]) : 0.f;
+    for (int e = 0; e < 8; ++e) v[e] = on ? to_float(x.v[e]) + (bias ? bias[(size_t)h * d + 8 * c + e] : 0.f) : 0.f;
   }
   const float* w = is_k ? kw : qw;
   if (w) {
@@ -531,7 +543,7 @@ int xi_silu_mul(const void* gate_up, void* out, int dtype, int n_tok, int I, hip
   return 0;
 }
 
-int xi_qk_norm_rope_kv(const void* qkv, int dtype, const float* qw, const float* kw, float eps,
+int xi_qk_norm_rope_kv(const void* qkv, int dtype, const float* bias, const float* qw, const float* kw, float eps,
                        const float* cos_t, const float* sin_t, int rot, int interleaved,
                        const int* positions, const long long* slots, void* q_out, void* k_cache,
                        void* v_cache, int page_size, int n_tok, int nq, int nkv, int d, int v_transposed,
@@ -555,7 +567,7 @@ int xi_qk_norm_rope_kv(const void* qkv, int dtype, const float* qw, const float*
     XI_CHECK(nq + 2 * nkv <= 65535, "qk_norm_rope_kv: too many heads");
     const size_t lds = (size_t)tpw * (d + 2) * sizeof(bf16);
     qk_norm_rope_kvt_bf16_kernel<<<dim3(blocks_x, nq + 2 * nkv), n_waves * 64, lds, stream>>>(
-        (const bf16*)qkv, qw, kw, eps, cos_t, sin_t, rot, interleaved, positions, slots, (bf16*)q_out,
+        (const bf16*)qkv, bias, qw, kw, eps, cos_t, sin_t, rot, interleaved, positions, slots, (bf16*)q_out,
         (bf16*)k_cache, (bf16*)v_cache, page_size, n_tok, nq, nkv, d);
     XI_LAUNCH_CHECK("qk_norm_rope_kv");
     return 0;
@@ -566,7 +578,7 @@ int xi_qk_norm_rope_kv(const void* qkv, int dtype, const float* qw, const float*
   XI_CHECK(blocks < (1ll << 31), "qk_norm_rope_kv: too many tokens");
 #define XI_QK(TT)                                                                               \
   qk_norm_rope_kv_kernel<TT><<<(unsigned)blocks, wpb * kWave, 0, stream>>>(                     \
-      (const TT*)qkv, qw, kw, eps, cos_t, sin_t, rot, interleaved, positions, slots, (TT*)q_out, \
+      (const TT*)qkv, bias, qw, kw, eps, cos_t, sin_t, rot, interleaved, positions, slots, (TT*)q_out, \
       (TT*)k_cache, (TT*)v_cache, page_size, n_tok, nq, nkv, d, v_transposed)
   if (dtype == kF32) XI_QK(float);
   else if (dtype == kBF16) XI_QK(bf16);

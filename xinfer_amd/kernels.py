@@ -147,12 +147,13 @@ def qk_norm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor],
                     positions: torch.Tensor, slots: torch.Tensor, k_cache: torch.Tensor,
                     v_cache: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                     q_out: Optional[torch.Tensor] = None, v_transposed: bool = False,
-                    vector_min_tokens: int = 128) -> torch.Tensor:
+                    vector_min_tokens: int = 128, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Per-head RMSNorm of q and k (if weights are given), rotation by position, q to q_out
     [T, nq, d], k and v into the paged cache [pages, nkv, page_size, d] at `slots`; with
     `v_transposed` the V pool is [pages, nkv, d, page_size].  From `vector_min_tokens` tokens
-    on, bfloat16 with the transposed pool runs the vectorized kernel."""
-    _dev(qkv, q_weight, k_weight, cos, sin, positions, slots, k_cache, v_cache, q_out)
+    on, bfloat16 with the transposed pool runs the vectorized kernel.  `bias` (float32, one
+    value per element of a packed row) is added to the rows first, in float32."""
+    _dev(qkv, q_weight, k_weight, cos, sin, positions, slots, k_cache, v_cache, q_out, bias)
     nq, nkv, d = num_heads, num_kv_heads, head_dim
     T = qkv.shape[0]
     if qkv.dim() != 2 or qkv.shape[1] != (nq + 2 * nkv) * d:
@@ -170,13 +171,17 @@ def qk_norm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor],
             _want(w, torch.float32, "qk_norm_rope_kv: norm weight")
             if w.shape != (d,):
                 raise KernelError("qk_norm_rope_kv: norm weight must be [head_dim]")
+    if bias is not None:
+        _want(bias, torch.float32, "qk_norm_rope_kv: bias")
+        if bias.shape != (qkv.shape[1],):
+            raise KernelError(f"qk_norm_rope_kv: bias {tuple(bias.shape)} is not [{qkv.shape[1]}]")
     _check_cache(k_cache, v_cache, nkv, d, qkv.dtype, v_transposed, "qk_norm_rope_kv")
     if q_out is None:
         q_out = torch.empty((T, nq, d), dtype=qkv.dtype, device=qkv.device)
     elif q_out.shape != (T, nq, d) or q_out.dtype != qkv.dtype:
         raise KernelError("qk_norm_rope_kv: q_out has the wrong shape or dtype")
     _ok(lib().xi_qk_norm_rope_kv(
-        _p(qkv), _code(qkv, "qk_norm_rope_kv"), _p(q_weight), _p(k_weight), ctypes.c_float(eps),
+        _p(qkv), _code(qkv, "qk_norm_rope_kv"), _p(bias), _p(q_weight), _p(k_weight), ctypes.c_float(eps),
         _p(cos), _p(sin), int(rotary_dim), int(bool(interleaved)), _p(positions), _p(slots),
         _p(q_out), _p(k_cache), _p(v_cache), int(k_cache.shape[2]), T, nq, nkv, d,
         int(bool(v_transposed)), int(vector_min_tokens), _stream()))

@@ -1,6 +1,6 @@
 """Paged grouped-query attention as a mixer.
 
-h -> packed q/k/v projection -> per-head RMSNorm of q and k -> rotation by position ->
+h -> packed q/k/v projection (+ bias) -> per-head RMSNorm of q and k -> rotation by position ->
 keys/values into the paged cache -> causal attention over the cache (all keys, or the
 last `window`) -> output projection.  Reference: Attention::forward_with_kv,
 /root/reference/src/models/layers/attention.rs:796-977 (projection 805-828, q/k norm
@@ -38,13 +38,12 @@ class PagedAttention(Mixer):
         self.scale = float(spec.get("scale", self.d ** -0.5))
         if self.nq % self.nkv:
             raise ValueError(f"{self.nq} query heads are not a multiple of {self.nkv} kv heads")
-        if self.bias:
-            raise NotImplementedError("attention projections with bias are not built")
         pos = spec.get("position")
         self.position = position_encoding_class(pos.kind)(pos, dtype) if pos is not None else None
         self.qkv: Optional[Linear] = None
         self.o: Optional[Linear] = None
         self.q_norm_w = self.k_norm_w = None
+        self.qkv_bias = None         # float32 [(nq + 2 nkv) d], added by the kernel after the projection
 
     # ---- weights -----------------------------------------------------------
     @classmethod
@@ -54,6 +53,9 @@ class PagedAttention(Mixer):
                TensorDecl(f"{prefix}.k_proj.weight", (nkv * d, h)),
                TensorDecl(f"{prefix}.v_proj.weight", (nkv * d, h)),
                TensorDecl(f"{prefix}.o_proj.weight", (h, nq * d))]
+        if spec.get("bias", False):    # q, k and v only: the reference's o_proj has none (attention.rs:596-608)
+            out += [TensorDecl(f"{prefix}.q_proj.bias", (nq * d,)), TensorDecl(f"{prefix}.k_proj.bias", (nkv * d,)),
+                    TensorDecl(f"{prefix}.v_proj.bias", (nkv * d,))]
         if spec.get("qk_norm", False):
             out += [TensorDecl(f"{prefix}.q_norm.weight", (d,), "norm"),
                     TensorDecl(f"{prefix}.k_norm.weight", (d,), "norm")]
@@ -67,6 +69,9 @@ class PagedAttention(Mixer):
         common = torch.float32 if any(p.dtype == torch.float32 for p in parts) else parts[0].dtype
         self.qkv = Linear(torch.cat([p.to(common) for p in parts], dim=0))
         self.o = Linear(lin(f"{prefix}.o_proj.weight"))
+        if self.bias:
+            self.qkv_bias = torch.cat([store.get(f"{prefix}.{n}_proj.bias", torch.float32, device)
+                                       for n in ("q", "k", "v")]).contiguous()
         if self.qk_norm:
             self.q_norm_w = store.get(f"{prefix}.q_norm.weight", torch.float32, device).contiguous()
             self.k_norm_w = store.get(f"{prefix}.k_norm.weight", torch.float32, device).contiguous()
@@ -94,6 +99,7 @@ class PagedAttention(Mixer):
             pos.sin if pos is not None else ctx.empty_f32,
             pos.rotary_dim if pos is not None else 0,
             pos.interleaved if pos is not None else False,
-            ctx.positions, slots, cache.k, cache.v, self.nq, self.nkv, self.d, v_transposed=vt)
+            ctx.positions, slots, cache.k, cache.v, self.nq, self.nkv, self.d, v_transposed=vt,
+            bias=self.qkv_bias)
         a = kernels.attention(q, cache.k, cache.v, ctx, cache.group, self.scale, self.window, v_transposed=vt)
         return self.o(a, out_dtype=self.dtype, allow_split=True, sink=sink)     # the next norm adds the parts
