@@ -240,6 +240,68 @@ def test_linear_folded_norm_refuses():
         kernels.linear_fold_in(x[:4].contiguous(), torch.zeros((4, 600), device=DEV), 1e-6, w)
 
 
+@pytest.mark.parametrize("M", [1, 17, 64, 65, 100, 128])
+@pytest.mark.parametrize("N,K", [(128, 64), (200, 256), (130, 1472), (4096, 1408), (640, 4096), (5120, 192)])
+def test_linear_mid(M, N, K):
+    """The tiled product for decode batches of up to 128 rows and narrow outputs: float32 partial
+    sums in slices of K.  Widths that are no multiple of the 128-feature tile or of 4, a last
+    tile of one feature's rows, slices of unequal length (K / 64 tiles dealt over the slices), a
+    slice shorter than the depth of the copy pipeline; a row's values do not depend on the rows
+    beside it, and rows past M leave nothing behind."""
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(11)
+    x = _rand((M, K), torch.bfloat16, g)
+    w = _rand((N, K), torch.bfloat16, g, 0.05)
+    ref = x.double() @ w.double().T
+    xd, wd = x.to(DEV), w.to(DEV)
+    slices = kernels.linear_mid_slices(N, K)
+    assert 1 <= slices <= K // 64
+    y = kernels.linear_mid(xd, wd)
+    assert y.dtype == torch.float32 and tuple(y.shape) == (slices, M, N)
+    got = y.cpu().double().sum(0)
+    err = (got - ref).abs().max() / ref.abs().max()
+    assert err < 1e-5, err
+    # each slice is the product over its own part of K: tiles of 64 dealt out as evenly as they go
+    kt, lo = K // 64, 0
+    for sl in range(slices):
+        n = kt // slices + (1 if sl < kt % slices else 0)
+        part = x[:, 64 * lo:64 * (lo + n)].double() @ w[:, 64 * lo:64 * (lo + n)].double().T
+        assert (y[sl].cpu().double() - part).abs().max() / ref.abs().max() < 1e-5, sl
+        lo += n
+    assert lo == kt
+    # the depth of the copy pipeline changes no bit
+    for depth in (3, 4):
+        assert torch.equal(kernels.linear_mid(xd, wd, depth=depth), y), depth
+    # a row alone, and the first rows alone: the same bits
+    r = M // 2
+    y1 = kernels.linear_mid(xd[r:r + 1].contiguous(), wd)
+    assert torch.equal(y1[:, 0], y[:, r])
+    if M > 70:
+        y70 = kernels.linear_mid(xd[:70].contiguous(), wd)
+        assert torch.equal(y70, y[:, :70])
+
+
+def test_linear_mid_refuses_and_serves_the_norm():
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(12)
+    x = _rand((129, 128), torch.bfloat16, g).to(DEV)
+    w = _rand((256, 128), torch.bfloat16, g).to(DEV)
+    with pytest.raises(kernels.KernelError, match="1..128"):
+        kernels.linear_mid(x, w)
+    assert kernels.linear_mid_slices(256, 96) == 0 and kernels.linear_mid_slices(256, 32) == 0
+    with pytest.raises(kernels.KernelError, match="multiple of 64"):
+        kernels.linear_mid(x[:100, :96].contiguous(), w[:, :96].contiguous())
+    # where a caller takes partial sums, rows 65..128 of a narrow product come from this kernel
+    x, w = _rand((100, 1024), torch.bfloat16, g).to(DEV), _rand((640, 1024), torch.bfloat16, g, 0.05).to(DEV)
+    y = kernels.linear_bf16(x, w, allow_split=True)
+    assert y.dtype == torch.float32 and tuple(y.shape) == (kernels.linear_mid_slices(640, 1024), 100, 640)
+    assert torch.equal(y, kernels.linear_mid(x, w))
+    assert kernels.linear_bf16(x, w).shape == (100, 640)
+    # the slices are chosen from (N, K) alone
+    assert kernels.linear_mid_slices(4096, 12288) == 8 and kernels.linear_mid_slices(5120, 17408) == 6
+    assert kernels.linear_mid_slices(151936, 4096) == 1
+
+
 def test_linear_skinny_plan_fills_the_compute_units():
     """The shapes the streaming product chooses: grids that are multiples of the 256 compute
     units where the width allows (a workgroup may own a number of features that is no multiple

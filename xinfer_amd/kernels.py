@@ -442,6 +442,37 @@ def linear_skinny_plan(M: int, N: int, K: int, gated: bool = False, allow_split:
     return ks, rt, rows, -(-N // rows) * ks
 
 
+MID_ROWS = 128            # most rows of the tiled product for narrow outputs (`linear_mid`)
+MID_FROM = 17             # from this many rows on it is used, where the caller takes partial sums,
+MID_WIDEST = 8192         # for outputs up to this wide (wider ones have tiles enough for the library)
+
+
+def linear_mid_slices(N: int, K: int) -> int:
+    """The slices of K in which `linear_mid` answers for an output of N features; 0 if it does
+    not take the sizes."""
+    return int(lib().xi_linear_mid_slices(int(N), int(K)))
+
+
+def linear_mid(x: torch.Tensor, w: torch.Tensor, depth: int = 0) -> torch.Tensor:
+    """bfloat16 x [M, K] @ w [N, K]^T for up to MID_ROWS rows as float32 partial sums
+    [slices, M, N], to be added in order (the fused add + RMSNorm does): the tiled kernel for
+    decode batches too large for `linear_skinny` and outputs too narrow for the library.
+    `depth`: tiles of loads a thread keeps in flight, 0 = the default; the result does not depend on it."""
+    _dev(x, w)
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError("linear_mid: operands must be bfloat16")
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
+        raise KernelError(f"linear_mid: x {tuple(x.shape)} and w {tuple(w.shape)} do not match")
+    M, K = x.shape
+    N = w.shape[0]
+    slices = linear_mid_slices(N, K)
+    if not (0 < M <= MID_ROWS) or slices < 1:
+        raise KernelError(f"linear_mid: M={M} must be 1..{MID_ROWS} and K={K} a multiple of 64")
+    y = torch.empty((slices, M, N), dtype=torch.float32, device=x.device)
+    _ok(lib().xi_linear_mid(_p(x), _p(w), _p(y), M, N, K, int(depth), _stream()))
+    return y
+
+
 FOLD_ROWS = 16            # most rows of the products that carry a folded norm between them
 FOLD_PARTS = 512          # most parts of a row's sum of squares the product after the norm adds up
 
@@ -517,6 +548,9 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtyp
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError("linear_bf16: operands must be bfloat16")
     out_dtype = out_dtype or torch.bfloat16
+    if allow_split and MID_FROM <= x.shape[0] <= MID_ROWS and linear_mid_slices(w.shape[0], w.shape[1]) > 0 \
+            and w.shape[0] <= MID_WIDEST:
+        return linear_mid(x, w)
     if (allow_split and x.shape[1] % 8 == 0 and x.shape[0] >= SKINNY_SPLIT_FROM
             and int(lib().xi_linear_skinny_slices(w.shape[0], w.shape[1], 0, 1)) > 1):
         skinny_rows = max(skinny_rows, SKINNY_SPLIT_ROWS)
