@@ -240,11 +240,11 @@ def test_linear_folded_norm_refuses():
         kernels.linear_fold_in(x[:4].contiguous(), torch.zeros((4, 600), device=DEV), 1e-6, w)
 
 
-@pytest.mark.parametrize("M", [1, 17, 64, 65, 100, 128])
+@pytest.mark.parametrize("M", [1, 17, 64, 65, 100, 128, 129, 200, 256])
 @pytest.mark.parametrize("N,K", [(128, 64), (200, 256), (130, 1472), (4096, 1408), (640, 4096), (5120, 192)])
 def test_linear_mid(M, N, K):
-    """The tiled product for decode batches of up to 128 rows and narrow outputs: float32 partial
-    sums in slices of K.  Widths that are no multiple of the 128-feature tile or of 4, a last
+    """The tiled product for decode batches of up to 256 rows (blocks of 128) and narrow outputs:
+    float32 partial sums in slices of K.  Widths that are no multiple of the 128-feature tile or of 4, a last
     tile of one feature's rows, slices of unequal length (K / 64 tiles dealt over the slices), a
     slice shorter than the depth of the copy pipeline; a row's values do not depend on the rows
     beside it, and rows past M leave nothing behind."""
@@ -284,9 +284,9 @@ def test_linear_mid(M, N, K):
 def test_linear_mid_refuses_and_serves_the_norm():
     from xinfer_amd import kernels
     g = torch.Generator().manual_seed(12)
-    x = _rand((129, 128), torch.bfloat16, g).to(DEV)
+    x = _rand((257, 128), torch.bfloat16, g).to(DEV)
     w = _rand((256, 128), torch.bfloat16, g).to(DEV)
-    with pytest.raises(kernels.KernelError, match="1..128"):
+    with pytest.raises(kernels.KernelError, match="1..256"):
         kernels.linear_mid(x, w)
     assert kernels.linear_mid_slices(256, 96) == 0 and kernels.linear_mid_slices(256, 32) == 0
     with pytest.raises(kernels.KernelError, match="multiple of 64"):

@@ -44,7 +44,7 @@ constexpr size_t kMidLdsBytes = 2 * 2 * (size_t)kMidTile * sizeof(bf16);
 template <int D, bool HALF>
 __global__ __launch_bounds__(256, 1) void linear_mid_kernel(const bf16* __restrict__ x,
                                                             const bf16* __restrict__ w, float* __restrict__ y,
-                                                            int M, int N, int K, int ks) {
+                                                            int M, int N, int K, int ks, size_t slice_stride) {
   extern __shared__ __align__(16) unsigned char mid_smem[];
   bf16* lds = reinterpret_cast<bf16*>(mid_smem);   // [buffer][w tile | x tile][128][kMidLdsRow]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -144,7 +144,7 @@ __global__ __launch_bounds__(256, 1) void linear_mid_kernel(const bf16* __restri
 #undef XI_MID_ISSUE
 
   // a lane's 4 values of a tile: row 16 tj + r of x, features 4 j .. 4 j + 3
-  float* ys = y + (size_t)slice * M * N;
+  float* ys = y + (size_t)slice * slice_stride;
   const bool vec = (N & 3) == 0;
 #pragma unroll
   for (int tj = 0; tj < 4; ++tj) {
@@ -182,7 +182,7 @@ using namespace xi;
 
 extern "C" {
 
-int xi_linear_mid_max_rows() { return kMidRows; }
+int xi_linear_mid_max_rows() { return 2 * kMidRows; }
 
 // 0 if the sizes are not taken (the caller then uses another product).
 int xi_linear_mid_slices(int N, int K) {
@@ -190,10 +190,12 @@ int xi_linear_mid_slices(int N, int K) {
   return mid_slices(N, K);
 }
 
-// y: float32 [slices, M, N] with slices = xi_linear_mid_slices(N, K).  depth: tiles of loads in
-// flight, 0 = the default (the result does not depend on it).
+// y: float32 [slices, M, N] with slices = xi_linear_mid_slices(N, K).  Up to 256 rows: blocks of
+// 128 rows are launched one after the other (the second pass over w comes in part from the
+// last level cache).  depth: tiles of loads in flight, 0 = the default (the result does not
+// depend on it).
 int xi_linear_mid(const void* x, const void* w, float* y, int M, int N, int K, int depth, hipStream_t stream) {
-  XI_CHECK(M >= 1 && M <= kMidRows, "linear_mid: M=%d must be 1..%d", M, kMidRows);
+  XI_CHECK(M >= 1 && M <= 2 * kMidRows, "linear_mid: M=%d must be 1..%d", M, 2 * kMidRows);
   XI_CHECK(N >= 1 && K >= kMidK && K % kMidK == 0, "linear_mid: N=%d, K=%d (a multiple of %d) are not taken", N, K, kMidK);
   XI_CHECK(((uintptr_t)x | (uintptr_t)w | (uintptr_t)y) % 16 == 0, "linear_mid: operands must be 16-byte aligned");
   const int ks = mid_slices(N, K);
@@ -212,12 +214,16 @@ int xi_linear_mid(const void* x, const void* w, float* y, int M, int N, int K, i
       lds_set = true;                                                                                         \
     }                                                                                                         \
     linear_mid_kernel<D, HALF><<<(unsigned)(tiles * ks), 256, kMidLdsBytes, stream>>>(                        \
-        (const bf16*)x, (const bf16*)w, y, M, N, K, ks);                                                      \
+        (const bf16*)x + (size_t)row0 * K, (const bf16*)w, y + (size_t)row0 * N, rows, N, K, ks,              \
+        (size_t)M * N);                                                                                       \
   } while (0)
-#define XI_MID_D(D)               \
-  do {                            \
-    if (M <= 64) XI_MID(D, true); \
-    else XI_MID(D, false);        \
+#define XI_MID_D(D)                                        \
+  do {                                                     \
+    for (int row0 = 0; row0 < M; row0 += kMidRows) {       \
+      const int rows = M - row0 < kMidRows ? M - row0 : kMidRows; \
+      if (rows <= 64) XI_MID(D, true);                     \
+      else XI_MID(D, false);                               \
+    }                                                      \
   } while (0)
   if (depth == 2) XI_MID_D(2);
   else if (depth == 3) XI_MID_D(3);

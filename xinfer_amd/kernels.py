@@ -442,7 +442,7 @@ def linear_skinny_plan(M: int, N: int, K: int, gated: bool = False, allow_split:
     return ks, rt, rows, -(-N // rows) * ks
 
 
-MID_ROWS = 128            # most rows of the tiled product for narrow outputs (`linear_mid`)
+MID_ROWS = 256            # most rows of the tiled product for narrow outputs (`linear_mid`)
 MID_FROM = 17             # from this many rows on it is used, where the caller takes partial sums,
 MID_WIDEST = 8192         # for outputs up to this wide (wider ones have tiles enough for the library)
 
