@@ -100,6 +100,7 @@ class PagedAttention(Mixer):
             pos.rotary_dim if pos is not None else 0,
             pos.interleaved if pos is not None else False,
             ctx.positions, slots, cache.k, cache.v, self.nq, self.nkv, self.d, v_transposed=vt,
-            bias=self.qkv_bias)
+            # decoded tokens lie in a page each: the form with one wave per head stays ahead longer
+            vector_min_tokens=128 if ctx.max_q_len > 1 else 512, bias=self.qkv_bias)
         a = kernels.attention(q, cache.k, cache.v, ctx, cache.group, self.scale, self.window, v_transposed=vt)
         return self.o(a, out_dtype=self.dtype, allow_split=True, sink=sink)     # the next norm adds the parts
