@@ -302,6 +302,37 @@ def test_linear_mid_refuses_and_serves_the_norm():
     assert kernels.linear_mid_slices(151936, 4096) == 1
 
 
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 32, 33, 64, 65, 128])
+@pytest.mark.parametrize("N,K", [(64, 64), (100, 192), (182, 1024), (4100, 512), (1000, 4096)])
+def test_linear_mid_gated(M, N, K):
+    """The gated form of the tiled product: silu(x gate^T) * (x up^T), one rounding, for every
+    shape of the kernel (up to 16, 32, 64 and 128 rows), widths that are no multiple of the
+    features a workgroup owns, a last workgroup with a single feature; and the folded norm."""
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(13)
+    x = _rand((M, K), torch.bfloat16, g)
+    w = _rand((2 * N, K), torch.bfloat16, g, 0.05)
+    gate, up = x.double() @ w[:N].double().T, x.double() @ w[N:].double().T
+    ref = gate / (1 + torch.exp(-gate)) * up
+    y = kernels.linear_mid_gated(x.to(DEV), w.to(DEV))
+    assert y.dtype == torch.bfloat16 and tuple(y.shape) == (M, N)
+    assert (y.cpu().double() - ref).abs().max() / ref.abs().max() < 2.0 ** -8
+    r = M // 2     # a row alone: the same bits
+    assert torch.equal(kernels.linear_mid_gated(x[r:r + 1].contiguous().to(DEV), w.to(DEV))[0], y[r])
+    if M <= 16:
+        parts = 37
+        ss = torch.rand((M, parts), generator=g) * 3 + 0.1
+        eps = 1e-5
+        inv = torch.rsqrt(ss.double().sum(1) / K + eps)[:, None]
+        gs, us = gate * inv, up * inv
+        want = gs / (1 + torch.exp(-gs)) * us
+        yf = kernels.linear_mid_gated(x.to(DEV), w.to(DEV), ss.to(DEV), eps)
+        assert (yf.cpu().double() - want).abs().max() / want.abs().max() < 2.0 ** -8
+    else:
+        with pytest.raises(kernels.KernelError, match="folded norm"):
+            kernels.linear_mid_gated(x.to(DEV), w.to(DEV), torch.ones((M, 4), device=DEV), 1e-5)
+
+
 def test_linear_skinny_plan_fills_the_compute_units():
     """The shapes the streaming product chooses: grids that are multiples of the 256 compute
     units where the width allows (a workgroup may own a number of features that is no multiple

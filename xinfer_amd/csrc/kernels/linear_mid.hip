@@ -22,6 +22,15 @@
 // L2 holds one slice of x.  An output element's value depends on (N, K) alone (they fix KS):
 // never on M or on what else is in the batch.
 //
+// GATED: w is [2N, K] = [gate; up] (the feed-forward's first product, which is wide: no slices);
+// a workgroup owns R <= 64 features n0 .. n0 + R - 1 (any R, so that the grid is a multiple of
+// the compute units), its tile holds their gate rows in rows 0 .. 63 and their up rows in rows
+// 64 .. 127, a wave multiplies 16-feature tiles of both, and stores silu(gate) * up in bfloat16:
+// one pass over w at any M up to 128, where the streaming kernel's workgroups (16 to 50
+// features) re-read x from L2 more the more rows there are.  FOLD: x is the first half of a
+// folded RMSNorm (see linear_skinny.hip): the rows of the product are multiplied by
+// rsqrt(sum of the row's parts / K + eps) before the activation.
+//
 // Reference call site: candle matmul in /root/reference/src/models/layers/linear.rs:76-124
 // (vendor BLAS).
 #include "common.h"
@@ -32,67 +41,107 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr int kMidRows = 128;          // rows of x a workgroup takes: all of them
-constexpr int kMidFeatures = 128;      // output features of a workgroup
+constexpr int kMidFeatures = 128;      // rows of w in a workgroup's tile
 constexpr int kMidK = 64;              // k per tile
 constexpr int kMidLdsRow = kMidK + 8;  // elements of a row in LDS
 constexpr int kMidDepth = 2;           // tiles whose loads are in flight (the default; measured: more gain nothing)
 constexpr int kMidTile = 128 * kMidLdsRow;   // elements of one operand's tile in LDS
-constexpr size_t kMidLdsBytes = 2 * 2 * (size_t)kMidTile * sizeof(bf16);
+constexpr size_t kMidLdsBytes = 2 * 2 * (size_t)kMidTile * sizeof(bf16) + 16 * sizeof(float);
+constexpr int kMidSsLoads = 32;        // 16 threads x 32 loads: up to 512 parts of a row's sum of squares
 
-// D: tiles whose loads are in flight.  HALF: at most 64 rows of x; the four waves then take a
-// quarter of the features each (32 features by 64 rows) instead of a quarter of the tile.
-template <int D, bool HALF>
+struct MidFold {
+  const float* ss_in;   // [M, parts] parts of each row's sum of squares
+  int parts;
+  float eps;
+  float inv_h;          // 1 / length of the normed rows
+};
+
+// D: tiles whose loads are in flight.  FULL: up to 128 rows of x, the four waves take a quarter
+// of the tile each (64 rows of w by 64 rows of x); else up to 16 * TJ <= 64 rows of x and a wave
+// takes a quarter of the rows of w (32) by all rows of x.  GATED, FOLD: see the head of the file.
+template <int D, int TJ, bool FULL, bool GATED, bool FOLD>
 __global__ __launch_bounds__(256, 1) void linear_mid_kernel(const bf16* __restrict__ x,
-                                                            const bf16* __restrict__ w, float* __restrict__ y,
-                                                            int M, int N, int K, int ks, size_t slice_stride) {
+                                                            const bf16* __restrict__ w, void* __restrict__ yv,
+                                                            int M, int N, int K, int ks, size_t slice_stride,
+                                                            int R, int rotate, MidFold fold) {
+  static_assert(!FULL || TJ == 4, "the full form multiplies 64 rows of x per wave");
+  static_assert(!FOLD || (GATED && !FULL && TJ == 1), "a folded norm: the gated form, up to 16 rows");
   extern __shared__ __align__(16) unsigned char mid_smem[];
   bf16* lds = reinterpret_cast<bf16*>(mid_smem);   // [buffer][w tile | x tile][128][kMidLdsRow]
+  float* inv_s = reinterpret_cast<float*>(mid_smem + 2 * 2 * (size_t)kMidTile * sizeof(bf16));   // [16]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, j = lane >> 4;
-  constexpr int TI = HALF ? 2 : 4;                    // 16-feature tiles of a wave
-  const int wf = HALF ? wave : (wave & 1);            // the wave's features start at 16 * TI * wf,
-  const int wt = HALF ? 0 : (wave >> 1);              // its rows at 64 * wt
+  constexpr int TI = FULL ? 4 : 2;                    // 16-row tiles of w a wave multiplies
+  constexpr int TG = GATED ? TI / 2 : TI;             // of them gate tiles (the others: their up tiles)
+  constexpr int XI = FULL ? 4 : (TJ == 4 ? 2 : 1);    // 32-row groups of x that are copied
+  const int wf = FULL ? (wave & 1) : wave;            // which of the wave's shares of the features,
+  const int wt = FULL ? (wave >> 1) : 0;              // of the rows of x (64 * wt on)
   const int slice = blockIdx.x % ks, tile = blockIdx.x / ks;
-  const int n0 = tile * kMidFeatures;
+  const int n0 = tile * R;
+  const int n_last = (n0 + R < N ? n0 + R : N) - 1;   // the workgroup's last feature
   // the k tiles of this slice: K / 64 tiles dealt out as evenly as they go
   const int kt_total = K / kMidK;
   const int base = kt_total / ks, rem = kt_total % ks;
   const int kt0 = slice * base + (slice < rem ? slice : rem);
   const int nkt = base + (slice < rem ? 1 : 0);
+  // Workgroups start at different tiles of their slice and wrap around, so that they do not all
+  // ask for the same offset of their rows of w at the same time; where a workgroup starts
+  // depends on its features alone, so an output element's sum has one order whatever M is.
+  const int start = (int)(((long long)tile * rotate) % nkt);
+
+  // FOLD: 16 threads per row add up the parts of its sum of squares; the loads start now
+  float ss_mine[FOLD ? kMidSsLoads : 1];
+  if constexpr (FOLD) {
+    const int token = tid >> 4, sub = tid & 15;
+#pragma unroll
+    for (int i = 0; i < kMidSsLoads; ++i) {
+      const int p = sub + 16 * i;
+      ss_mine[i] = (token < M && p < fold.parts) ? fold.ss_in[(size_t)token * fold.parts + p] : 0.f;
+    }
+  }
 
   // ---- copying: a tile is 128 rows of 8 16-byte chunks; thread t moves chunk t % 8 of rows
-  // t / 8 + 32 i.  Rows of w past N read row N - 1 again and rows of x past M row M - 1 (the
-  // same address many times in one instruction costs one access); their results are dropped.
-  // No load is conditional, so the counter of loads in flight is exact and only the tile that
-  // is needed is waited for.
+  // t / 8 + 32 i.  Row q of the w tile is feature n0 + q (GATED: the gate row of feature
+  // n0 + q % 64 for q < 64, its up row for q >= 64); rows past the workgroup's last feature read
+  // that feature's row again and rows of x past M row M - 1 (the same address many times in one
+  // instruction costs one access); their results are dropped.  No load is conditional, so the
+  // counter of loads in flight is exact and only the tile that is needed is waited for.
   const int srow = tid >> 3, skc = tid & 7;
   const bf16* wsrc[4];
-  const bf16* xsrc[4];
+  const bf16* xsrc[XI];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int row = srow + 32 * i;
-    int n = n0 + row;
-    n = n < N ? n : N - 1;
+    int n = n0 + (GATED ? (row & 63) : row);
+    n = n < n_last ? n : n_last;
+    if (GATED && row >= 64) n += N;
     wsrc[i] = w + (size_t)n * K + (size_t)kt0 * kMidK + 8 * skc;
+  }
+#pragma unroll
+  for (int i = 0; i < XI; ++i) {
+    const int row = srow + 32 * i;
     xsrc[i] = x + (size_t)(row < M ? row : M - 1) * K + (size_t)kt0 * kMidK + 8 * skc;
   }
   const int sdst = srow * kMidLdsRow + 8 * skc;
-  bf16x8 wr[D][4], xr[D][4];
+  bf16x8 wr[D][4], xr[D][XI];
 
-  // a wave whose half of the rows lies past M has nothing to multiply
-  const bool active = __builtin_amdgcn_readfirstlane(64 * wt < M ? 1 : 0) != 0;
-  f32x4 acc[TI][4];
+  // a wave whose rows of x lie past M, or whose features past the workgroup's, has nothing to do
+  const int wave_row0 = GATED ? 16 * TG * wf : 16 * TI * wf;     // its first feature within the workgroup
+  const bool active = __builtin_amdgcn_readfirstlane((64 * wt < M && n0 + wave_row0 <= n_last) ? 1 : 0) != 0;
+  f32x4 acc[TI][TJ];
 #pragma unroll
   for (int ti = 0; ti < TI; ++ti)
 #pragma unroll
-    for (int tj = 0; tj < 4; ++tj) acc[ti][tj] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int tj = 0; tj < TJ; ++tj) acc[ti][tj] = f32x4{0.f, 0.f, 0.f, 0.f};
 
 #define XI_MID_ISSUE(slot, t)                                                         \
   do {                                                                                \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                   \
-      wr[slot][i] = *reinterpret_cast<const bf16x8*>(wsrc[i] + (size_t)(t) * kMidK);  \
-      xr[slot][i] = *reinterpret_cast<const bf16x8*>(xsrc[i] + (size_t)(t) * kMidK);  \
-    }                                                                                 \
+    int tt_ = (t) + start;                                                            \
+    tt_ = tt_ >= nkt ? tt_ - nkt : tt_;                                               \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                     \
+      wr[slot][i] = *reinterpret_cast<const bf16x8*>(wsrc[i] + (size_t)tt_ * kMidK);  \
+    _Pragma("unroll") for (int i = 0; i < XI; ++i)                                    \
+      xr[slot][i] = *reinterpret_cast<const bf16x8*>(xsrc[i] + (size_t)tt_ * kMidK);  \
   } while (0)
 
   // Every copy is issued whether or not its tile exists (past the slice's end the last tile is
@@ -102,29 +151,32 @@ __global__ __launch_bounds__(256, 1) void linear_mid_kernel(const bf16* __restri
 #pragma unroll
   for (int s = 0; s < D; ++s) XI_MID_ISSUE(s, s < last ? s : last);
 
-  // One tile: registers of slot s to LDS, the slot loaded again kMidDepth tiles ahead, barrier,
+  // One tile: registers of slot s to LDS, the slot loaded again D tiles ahead, barrier,
   // products.  One barrier a tile is enough: whoever writes this buffer again, two tiles on, has
   // passed the next tile's barrier, which every thread reaches only after these products.
+  // Row of the w tile of the wave's tile ti: its features' rows; GATED: gate tiles first, then
+  // the up tiles of the same features, 64 rows further.
   int buf = 0;
+#define XI_MID_WROW(ti) (GATED ? (((ti) / TG) * 64 + wave_row0 + 16 * ((ti) % TG)) : (wave_row0 + 16 * (ti)))
 #define XI_MID_TILE(s, t)                                                                                 \
   do {                                                                                                    \
     bf16* Ws = lds + buf * (2 * kMidTile);                                                                \
     bf16* Xs = Ws + kMidTile;                                                                             \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                                       \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                         \
       *reinterpret_cast<bf16x8*>(Ws + sdst + 32 * i * kMidLdsRow) = wr[s][i];                             \
+    _Pragma("unroll") for (int i = 0; i < XI; ++i)                                                        \
       *reinterpret_cast<bf16x8*>(Xs + sdst + 32 * i * kMidLdsRow) = xr[s][i];                             \
-    }                                                                                                     \
     XI_MID_ISSUE(s, (t) + D < last ? (t) + D : last);                                                     \
     __syncthreads();                                                                                      \
     if (active) {                                                                                         \
       _Pragma("unroll") for (int kk = 0; kk < kMidK / 32; ++kk) {                                         \
-        bf16x8 a[TI], b[4];                                                                               \
+        bf16x8 a[TI], b[TJ];                                                                              \
         _Pragma("unroll") for (int ti = 0; ti < TI; ++ti) a[ti] = *reinterpret_cast<const bf16x8*>(       \
-            Ws + (16 * TI * wf + 16 * ti + r) * kMidLdsRow + 32 * kk + 8 * j);                            \
-        _Pragma("unroll") for (int tj = 0; tj < 4; ++tj) b[tj] = *reinterpret_cast<const bf16x8*>(        \
+            Ws + (XI_MID_WROW(ti) + r) * kMidLdsRow + 32 * kk + 8 * j);                                   \
+        _Pragma("unroll") for (int tj = 0; tj < TJ; ++tj) b[tj] = *reinterpret_cast<const bf16x8*>(       \
             Xs + (64 * wt + 16 * tj + r) * kMidLdsRow + 32 * kk + 8 * j);                                 \
         _Pragma("unroll") for (int ti = 0; ti < TI; ++ti)                                                 \
-          _Pragma("unroll") for (int tj = 0; tj < 4; ++tj)                                                \
+          _Pragma("unroll") for (int tj = 0; tj < TJ; ++tj)                                               \
             acc[ti][tj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ti], b[tj], acc[ti][tj], 0, 0, 0);    \
       }                                                                                                   \
     }                                                                                                     \
@@ -143,27 +195,60 @@ __global__ __launch_bounds__(256, 1) void linear_mid_kernel(const bf16* __restri
 #undef XI_MID_TILE
 #undef XI_MID_ISSUE
 
-  // a lane's 4 values of a tile: row 16 tj + r of x, features 4 j .. 4 j + 3
-  float* ys = y + (size_t)slice * slice_stride;
-  const bool vec = (N & 3) == 0;
+  if constexpr (FOLD) {
+    float t = 0.f;
 #pragma unroll
-  for (int tj = 0; tj < 4; ++tj) {
-    const int token = 64 * wt + 16 * tj + r;
-    if (token >= M) continue;
+    for (int i = 0; i < kMidSsLoads; ++i) t += ss_mine[i];
 #pragma unroll
-    for (int ti = 0; ti < TI; ++ti) {
-      const int f = n0 + 16 * TI * wf + 16 * ti + 4 * j;
-      float* dst = ys + (size_t)token * N + f;
-      if (vec && f + 3 < N) {
-        *reinterpret_cast<f32x4*>(dst) = acc[ti][tj];
-      } else {
+    for (int o = 8; o; o >>= 1) t += __shfl_xor(t, o, kWave);
+    if ((tid & 15) == 0) inv_s[tid >> 4] = rsqrtf(t * fold.inv_h + fold.eps);
+    __syncthreads();
+  }
+  if (!active) return;
+
+  // a lane's 4 values of a tile: row 16 tj + r of x, features 4 j .. 4 j + 3 of the tile
+  if constexpr (GATED) {
+    bf16* y = reinterpret_cast<bf16*>(yv);
+#pragma unroll
+    for (int tj = 0; tj < TJ; ++tj) {
+      const int token = 64 * wt + 16 * tj + r;
+      if (token >= M) continue;
+      const float inv = FOLD ? inv_s[token] : 1.f;
+#pragma unroll
+      for (int ti = 0; ti < TG; ++ti) {
+        const int f = n0 + wave_row0 + 16 * ti + 4 * j;
+        bf16* dst = y + (size_t)token * N + f;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (f + i < N) dst[i] = acc[ti][tj][i];
+          if (f + i <= n_last) {
+            const float g = acc[ti][tj][i] * inv, u = acc[ti + TG][tj][i] * inv;
+            dst[i] = from_float<bf16>(g / (1.f + __expf(-g)) * u);
+          }
+      }
+    }
+  } else {
+    float* ys = reinterpret_cast<float*>(yv) + (size_t)slice * slice_stride;
+    const bool vec = (N & 3) == 0;
+#pragma unroll
+    for (int tj = 0; tj < TJ; ++tj) {
+      const int token = 64 * wt + 16 * tj + r;
+      if (token >= M) continue;
+#pragma unroll
+      for (int ti = 0; ti < TI; ++ti) {
+        const int f = n0 + wave_row0 + 16 * ti + 4 * j;
+        float* dst = ys + (size_t)token * N + f;
+        if (vec && f + 3 <= n_last) {
+          *reinterpret_cast<f32x4*>(dst) = acc[ti][tj];
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (f + i <= n_last) dst[i] = acc[ti][tj][i];
+        }
       }
     }
   }
 }
+#undef XI_MID_WROW
 
 // Slices of K for an output of N features: tiles x slices fill the 256 compute units once; a
 // slice keeps at least 4 tiles of 64.  It depends on (N, K) alone.
@@ -174,6 +259,26 @@ static int mid_slices(int N, int K) {
   if (ks > 16) ks = 16;
   while (ks > 1 && kt / ks < 4) --ks;
   return ks < 1 ? 1 : ks;
+}
+
+// Features a workgroup of the gated form owns (at most 64): the fewest workgroups that are a
+// multiple of the 256 compute units, or failing that (N < 256 or so) of 64 features each.
+static int mid_gated_features(int N) {
+  for (int waves = 1; waves <= 64; ++waves) {
+    const int wgs = 256 * waves;
+    const int rr = (N + wgs - 1) / wgs;
+    if (rr <= 64) return rr < 16 ? 16 : rr;     // a narrow output: whole 16-feature tiles
+  }
+  return 64;
+}
+
+template <typename Kern>
+static int mid_lds(Kern kern, bool* done) {
+  if (*done) return 0;
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMidLdsBytes);
+  XI_CHECK(e == hipSuccess, "linear_mid: cannot get %zu bytes of LDS: %s", kMidLdsBytes, hipGetErrorString(e));
+  *done = true;
+  return 0;
 }
 
 }  // namespace xi
@@ -190,39 +295,39 @@ int xi_linear_mid_slices(int N, int K) {
   return mid_slices(N, K);
 }
 
+// Features per workgroup of the gated form for an output of N features (w is [2N, K]).
+int xi_linear_mid_gated_features(int N) { return N < 1 ? 0 : mid_gated_features(N); }
+
 // y: float32 [slices, M, N] with slices = xi_linear_mid_slices(N, K).  Up to 256 rows: blocks of
 // 128 rows are launched one after the other (the second pass over w comes in part from the
 // last level cache).  depth: tiles of loads in flight, 0 = the default (the result does not
 // depend on it).
-int xi_linear_mid(const void* x, const void* w, float* y, int M, int N, int K, int depth, hipStream_t stream) {
+int xi_linear_mid(const void* x, const void* w, float* y, int M, int N, int K, int depth, int rotate,
+                  hipStream_t stream) {
   XI_CHECK(M >= 1 && M <= 2 * kMidRows, "linear_mid: M=%d must be 1..%d", M, 2 * kMidRows);
   XI_CHECK(N >= 1 && K >= kMidK && K % kMidK == 0, "linear_mid: N=%d, K=%d (a multiple of %d) are not taken", N, K, kMidK);
   XI_CHECK(((uintptr_t)x | (uintptr_t)w | (uintptr_t)y) % 16 == 0, "linear_mid: operands must be 16-byte aligned");
+  XI_CHECK(rotate >= 0, "linear_mid: rotate=%d", rotate);
   const int ks = mid_slices(N, K);
   const long long tiles = (N + kMidFeatures - 1) / kMidFeatures;
   XI_CHECK(ks >= 1 && ks <= K / kMidK, "linear_mid: %d slices for K=%d", ks, K);
   XI_CHECK(tiles * ks < (1ll << 31), "linear_mid: too many workgroups");
   if (depth == 0) depth = kMidDepth;
-#define XI_MID(D, HALF)                                                                                       \
+  const MidFold none{nullptr, 0, 0.f, 0.f};
+#define XI_MID(D, TJ, FULL)                                                                                   \
   do {                                                                                                        \
     static bool lds_set = false;                                                                              \
-    if (!lds_set) {                                                                                           \
-      hipError_t e = hipFuncSetAttribute((const void*)linear_mid_kernel<D, HALF>,                             \
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMidLdsBytes);      \
-      XI_CHECK(e == hipSuccess, "linear_mid: cannot get %zu bytes of LDS: %s", kMidLdsBytes,                  \
-               hipGetErrorString(e));                                                                         \
-      lds_set = true;                                                                                         \
-    }                                                                                                         \
-    linear_mid_kernel<D, HALF><<<(unsigned)(tiles * ks), 256, kMidLdsBytes, stream>>>(                        \
+    if (mid_lds(linear_mid_kernel<D, TJ, FULL, false, false>, &lds_set)) return 1;                            \
+    linear_mid_kernel<D, TJ, FULL, false, false><<<(unsigned)(tiles * ks), 256, kMidLdsBytes, stream>>>(      \
         (const bf16*)x + (size_t)row0 * K, (const bf16*)w, y + (size_t)row0 * N, rows, N, K, ks,              \
-        (size_t)M * N);                                                                                       \
+        (size_t)M * N, kMidFeatures, rotate, none);                                                           \
   } while (0)
 #define XI_MID_D(D)                                        \
   do {                                                     \
     for (int row0 = 0; row0 < M; row0 += kMidRows) {       \
       const int rows = M - row0 < kMidRows ? M - row0 : kMidRows; \
-      if (rows <= 64) XI_MID(D, true);                     \
-      else XI_MID(D, false);                               \
+      if (rows <= 64) XI_MID(D, 4, false);                 \
+      else XI_MID(D, 4, true);                             \
     }                                                      \
   } while (0)
   if (depth == 2) XI_MID_D(2);
@@ -232,6 +337,39 @@ int xi_linear_mid(const void* x, const void* w, float* y, int M, int N, int K, i
 #undef XI_MID_D
 #undef XI_MID
   XI_LAUNCH_CHECK("linear_mid");
+  return 0;
+}
+
+// y [M, N] bfloat16 = silu(x @ gate^T) * (x @ up^T) with w = [gate; up] [2N, K], M <= 128.
+// ss (or null): x is the first half of a folded RMSNorm, ss [M, parts] float32 the parts of its
+// rows' sums of squares (M <= 16, parts <= 512): rows are scaled by rsqrt(sum / K + eps).
+int xi_linear_mid_gated(const void* x, const void* w, void* y, int M, int N, int K, const float* ss, int parts,
+                        float eps, int rotate, hipStream_t stream) {
+  XI_CHECK(M >= 1 && M <= kMidRows, "linear_mid_gated: M=%d must be 1..%d", M, kMidRows);
+  XI_CHECK(N >= 1 && K >= kMidK && K % kMidK == 0, "linear_mid_gated: N=%d, K=%d (a multiple of %d) are not taken", N,
+           K, kMidK);
+  XI_CHECK(((uintptr_t)x | (uintptr_t)w) % 16 == 0, "linear_mid_gated: operands must be 16-byte aligned");
+  XI_CHECK(rotate >= 0, "linear_mid_gated: rotate=%d", rotate);
+  XI_CHECK(ss == nullptr || (M <= 16 && parts >= 1 && parts <= 16 * kMidSsLoads),
+           "linear_mid_gated: a folded norm takes up to 16 rows and %d parts (M=%d, parts=%d)", 16 * kMidSsLoads, M, parts);
+  const int R = mid_gated_features(N);
+  const long long wgs = (N + R - 1) / R;
+  XI_CHECK(R >= 1 && R <= 64 && wgs < (1ll << 31), "linear_mid_gated: %d features per workgroup", R);
+  const MidFold fold{ss, parts, eps, 1.f / (float)K};
+#define XI_MIDG(TJ, FULL, FOLD)                                                                               \
+  do {                                                                                                        \
+    static bool lds_set = false;                                                                              \
+    if (mid_lds(linear_mid_kernel<kMidDepth, TJ, FULL, true, FOLD>, &lds_set)) return 1;                      \
+    linear_mid_kernel<kMidDepth, TJ, FULL, true, FOLD><<<(unsigned)wgs, 256, kMidLdsBytes, stream>>>(         \
+        (const bf16*)x, (const bf16*)w, y, M, N, K, 1, 0, R, rotate, fold);                                   \
+  } while (0)
+  if (ss != nullptr) XI_MIDG(1, false, true);
+  else if (M <= 16) XI_MIDG(1, false, false);
+  else if (M <= 32) XI_MIDG(2, false, false);
+  else if (M <= 64) XI_MIDG(4, false, false);
+  else XI_MIDG(4, true, false);
+#undef XI_MIDG
+  XI_LAUNCH_CHECK("linear_mid_gated");
   return 0;
 }
 

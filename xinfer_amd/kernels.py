@@ -442,6 +442,9 @@ def linear_skinny_plan(M: int, N: int, K: int, gated: bool = False, allow_split:
     return ks, rt, rows, -(-N // rows) * ks
 
 
+MID_ROTATE = 1            # workgroup tile t of the tiled products starts t * this many k tiles into its slice and
+MID_GATED_ROTATE = 1      # wraps around (0: all start at the slice's first tile, which measured 5% slower in a
+                          # decode step: every workgroup then asks for the same offset of its rows at the same time)
 MID_ROWS = 256            # most rows of the tiled product for narrow outputs (`linear_mid`)
 MID_FROM = 17             # from this many rows on it is used, where the caller takes partial sums,
 MID_WIDEST = 8192         # for outputs up to this wide (wider ones have tiles enough for the library)
@@ -469,7 +472,48 @@ def linear_mid(x: torch.Tensor, w: torch.Tensor, depth: int = 0) -> torch.Tensor
     if not (0 < M <= MID_ROWS) or slices < 1:
         raise KernelError(f"linear_mid: M={M} must be 1..{MID_ROWS} and K={K} a multiple of 64")
     y = torch.empty((slices, M, N), dtype=torch.float32, device=x.device)
-    _ok(lib().xi_linear_mid(_p(x), _p(w), _p(y), M, N, K, int(depth), _stream()))
+    _ok(lib().xi_linear_mid(_p(x), _p(w), _p(y), M, N, K, int(depth), int(MID_ROTATE), _stream()))
+    return y
+
+
+MID_GATED_ROWS = 128      # most rows of the gated form of the tiled product
+MID_GATED_UP_TO = 64      # it is used up to this many rows (more: its reads of x from L2 outweigh the library's
+                          # weakness); measured on MI355X at the gate/up sizes of Qwen3-8B, 14B and 32B, it is
+MID_GATED_FROM = 6        # ahead of the streaming kernel from this many rows on, and from the first row where
+MID_GATED_BIG = 300 << 20  # the weight has this many bytes (the streaming kernel falls behind on large weights)
+
+
+def gated_uses_mid(M: int, w: torch.Tensor) -> bool:
+    """Whether the gated product of M rows with w [2N, K] goes to `linear_mid_gated`."""
+    if w.dtype != torch.bfloat16 or w.shape[1] % 64 or w.shape[1] < 64 or w.shape[0] % 2:
+        return False
+    return (MID_GATED_FROM <= M <= MID_GATED_UP_TO) or (0 < M < MID_GATED_FROM and w.numel() * 2 >= MID_GATED_BIG)
+
+
+def linear_mid_gated(x: torch.Tensor, w: torch.Tensor, ss: Optional[torch.Tensor] = None, eps: float = 0.0) -> torch.Tensor:
+    """silu(x @ gate^T) * (x @ up^T) in bfloat16 for w = [gate; up] [2N, K] and up to MID_GATED_ROWS
+    rows with the tiled kernel: one pass over w whatever the number of rows.  `ss` [M, parts]
+    float32 (up to FOLD_ROWS rows): x is the first half of a folded RMSNorm (`linear_fold_out`)
+    and the rows of the products are multiplied by rsqrt(sum(ss[row]) / K + eps) first."""
+    _dev(x, w, ss)
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError("linear_mid_gated: operands must be bfloat16")
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1] or w.shape[0] % 2:
+        raise KernelError(f"linear_mid_gated: x {tuple(x.shape)} and w {tuple(w.shape)} ([2N, K]) do not match")
+    M, K = x.shape
+    N = w.shape[0] // 2
+    if not (0 < M <= MID_GATED_ROWS) or K % 64 or K < 64:
+        raise KernelError(f"linear_mid_gated: M={M} must be 1..{MID_GATED_ROWS} and K={K} a multiple of 64")
+    parts = 0
+    if ss is not None:
+        _want(ss, torch.float32, "linear_mid_gated: ss")
+        if M > FOLD_ROWS or ss.dim() != 2 or ss.shape[0] != M or not (0 < ss.shape[1] <= FOLD_PARTS):
+            raise KernelError(f"linear_mid_gated: a folded norm takes up to {FOLD_ROWS} rows and ss [M, up to "
+                              f"{FOLD_PARTS} parts], got M={M}, ss {tuple(ss.shape)}")
+        parts = int(ss.shape[1])
+    y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    _ok(lib().xi_linear_mid_gated(_p(x), _p(w), _p(y), M, N, K, _p(ss), parts, ctypes.c_float(eps), int(MID_GATED_ROTATE),
+                                  _stream()))
     return y
 
 

@@ -43,12 +43,16 @@ class Linear:
         w = self.weight
         if isinstance(x, Folded):
             if w.dtype == torch.bfloat16 and x.xg.shape[1] % 8 == 0 and (not gated or out_dtype in (None, torch.bfloat16)):
+                if gated and kernels.gated_uses_mid(x.xg.shape[0], w):
+                    return kernels.linear_mid_gated(x.xg, w, x.ss, x.norm.eps)
                 return kernels.linear_fold_in(x.xg, x.ss, x.norm.eps, w, out_dtype or torch.bfloat16, gated=gated)
             x = x.rows(torch.bfloat16 if w.dtype == torch.bfloat16 else torch.float32)
         if gated:
+            if x.dtype == torch.bfloat16 and x.dim() == 2 and kernels.gated_uses_mid(x.shape[0], w):
+                return kernels.linear_mid_gated(x, w)                 # gate, up and silu*mul in one pass
             if (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
                     and 0 < x.shape[0] <= kernels.SKINNY_GATED_ROWS and x.shape[1] % 8 == 0):
-                return kernels.linear_skinny(x, w, gated=True)        # gate, up and silu*mul in one pass
+                return kernels.linear_skinny(x, w, gated=True)        # the same with the streaming kernel
             return None
         if (sink is not None and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2
                 and 0 < x.shape[0] <= kernels.FOLD_ROWS and x.shape[1] % 8 == 0 and w.shape[0] % 8 == 0
