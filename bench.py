@@ -90,7 +90,7 @@ def serve(workload: str, layers) -> int:
     n = w["requests"]
     pages = n * (-(-w["max_model_len"] // page)) + 8
     eng = LLMEngine(EngineConfig(max_num_seqs=n, max_model_len=w["max_model_len"], num_pages=pages, page_size=page,
-                                 prefill_chunk_size=w["chunk"], max_num_batched_tokens=w["chunk"] + n, seed=1),
+                                 prefill_chunk_size=w["chunk"], seed=1),     # a step's token budget is the chunk
                     model=model)
     g = torch.Generator().manual_seed(4)
     lo, hi = w["prompt"]
