@@ -327,6 +327,14 @@ def test_linear_mid_refuses_and_serves_the_norm():
     # the slices are chosen from (N, K) alone
     assert kernels.linear_mid_slices(4096, 12288) == 8 and kernels.linear_mid_slices(5120, 17408) == 6
     assert kernels.linear_mid_slices(151936, 4096) == 1
+    # a wide output in float32 (the head) comes from the tiled kernel from 4 rows on, whole
+    x, w = _rand((9, 128), torch.bfloat16, g).to(DEV), _rand((40000, 128), torch.bfloat16, g, 0.05).to(DEV)
+    assert kernels.linear_mid_slices(40000, 128) == 1
+    y = kernels.linear_bf16(x, w, torch.float32)
+    assert y.dtype == torch.float32 and tuple(y.shape) == (9, 40000) and torch.equal(y, kernels.linear_mid(x, w)[0])
+    ref = x.cpu().double() @ w.cpu().double().T
+    assert (y.cpu().double() - ref).abs().max() / ref.abs().max() < 1e-5
+    assert torch.equal(kernels.linear_bf16(x[:3].contiguous(), w, torch.float32), kernels.linear_skinny(x[:3].contiguous(), w, torch.float32))
 
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 32, 33, 64, 65, 128])

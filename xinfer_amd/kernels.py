@@ -446,6 +446,8 @@ MID_ROTATE = 1            # workgroup tile t of the tiled products starts t * th
 MID_GATED_ROTATE = 1      # wraps around (0: all start at the slice's first tile, which measured 5% slower in a
                           # decode step: every workgroup then asks for the same offset of its rows at the same time)
 MID_ROWS = 256            # most rows of the tiled product for narrow outputs (`linear_mid`)
+MID_WIDE_FROM = 4         # rows from which it is ahead of the streaming kernel on an output so wide that it needs no
+                          # slices (the head: 215 against 242 us at 8 rows, 238 against 349 at 64, vocabulary 151936)
 MID_FROM = 17             # from this many rows on it is used, where the caller takes partial sums,
 MID_WIDEST = 8192         # for outputs up to this wide (wider ones have tiles enough for the library)
 
@@ -604,6 +606,9 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtyp
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError("linear_bf16: operands must be bfloat16")
     out_dtype = out_dtype or torch.bfloat16
+    if out_dtype == torch.float32 and MID_WIDE_FROM <= x.shape[0] <= MID_GATED_ROWS \
+            and linear_mid_slices(w.shape[0], w.shape[1]) == 1:
+        return linear_mid(x, w)[0]           # a wide output in float32 (the head): one slice is the result
     if allow_split and x.shape[0] <= MID_ROWS and linear_mid_slices(w.shape[0], w.shape[1]) > 0 \
             and w.shape[0] <= MID_WIDEST and (MID_FROM <= x.shape[0] or fold_loses_to_mid(x.shape[0], w)):
         return linear_mid(x, w)
