@@ -226,6 +226,56 @@ def test_linear_folded_norm(M, N, K, N2):
     assert y32.dtype == torch.float32 and (y32.cpu().double() - ref).abs().max() / ref.abs().max() < 2.0 ** -6
 
 
+@pytest.mark.parametrize("M", [1, 5, 16])
+@pytest.mark.parametrize("N,K,N2", [(64, 256, 96), (300, 512, 70), (4096, 1024, 130), (1000, 2304, 64)])
+def test_linear_thin_and_its_folded_norm(M, N, K, N2):
+    """The thin product (few features a workgroup, whole sums, whole lines through LDS) in its
+    three forms: plain, adding into the stream before a norm, scaling its rows after one; widths
+    that are no multiple of the features a workgroup owns, one tile of K and an odd number of
+    them, a row alone."""
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(19)
+    x = _rand((M, K), torch.bfloat16, g)
+    w1 = _rand((N, K), torch.bfloat16, g, 0.05)
+    ref = x.double() @ w1.double().T
+    for dt, tol in ((torch.bfloat16, 2.0 ** -8), (torch.float32, 1e-5)):
+        y = kernels.linear_thin(x.to(DEV), w1.to(DEV), dt)
+        assert y.dtype == dt and (y.cpu().double() - ref).abs().max() / ref.abs().max() < tol
+        r = M // 2
+        assert torch.equal(kernels.linear_thin(x[r:r + 1].contiguous().to(DEV), w1.to(DEV), dt)[0], y[r])
+    resid = _rand((M, N), torch.float32, g, 2.0)
+    gn = 1 + 0.2 * torch.randn(N, generator=g)
+    eps = 1e-6
+    r_dev = resid.to(DEV).clone()
+    xg, ss = kernels.linear_thin_fold_out(x.to(DEV), w1.to(DEV), r_dev, gn.to(DEV))
+    assert tuple(ss.shape) == (M, kernels.linear_thin_parts(N, K))
+    want_r = resid.double() + ref
+    assert (r_dev.cpu().double() - want_r).abs().max() / want_r.abs().max() < 1e-5
+    assert ((ss.cpu().double().sum(1) - (want_r ** 2).sum(1)).abs() / (want_r ** 2).sum(1)).max() < 1e-5
+    assert (xg.cpu().double() - want_r * gn.double()).abs().max() / (want_r * gn.double()).abs().max() < 2.0 ** -8
+    if N % 256 == 0:
+        normed = plain.rms_norm(want_r, gn.double(), eps)
+        w2 = _rand((N2, N), torch.bfloat16, g, 0.05)
+        y2 = kernels.linear_thin_fold_in(xg, ss, eps, w2.to(DEV))
+        ref2 = normed @ w2.double().T
+        assert y2.shape == (M, N2) and (y2.cpu().double() - ref2).abs().max() / ref2.abs().max() < 2.0 ** -6
+        # the folded product of the streaming kernel takes the same operands
+        y3 = kernels.linear_fold_in(xg, ss, eps, w2.to(DEV))
+        assert (y3.cpu().double() - ref2).abs().max() / ref2.abs().max() < 2.0 ** -6
+
+
+def test_linear_thin_refuses():
+    from xinfer_amd import kernels
+    x = torch.zeros((17, 256), dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros((32, 256), dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(kernels.KernelError, match="1..16"):
+        kernels.linear_thin(x, w)
+    with pytest.raises(kernels.KernelError, match="multiple of 256"):
+        kernels.linear_thin(x[:4, :128].contiguous(), w[:, :128].contiguous())
+    assert kernels.linear_thin_parts(4096, 4096) == 256 and kernels.linear_thin_parts(5120, 5120) == 256
+    assert kernels.linear_thin_parts(10240, 5120) == 512 and kernels.linear_thin_parts(64, 100) == 0
+
+
 def test_fold_gives_way_to_the_tiled_product():
     """A product before a norm adds into the stream itself for few rows, but with a long K and
     many of those rows it leaves the norm to its own kernel and answers with partial sums."""

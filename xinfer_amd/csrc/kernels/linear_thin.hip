@@ -1,0 +1,281 @@
+// y[M,N] = x[M,K] @ w[N,K]^T in bfloat16 for up to 16 rows (a decode step of few requests) where
+// every workgroup has to own few output features so that the whole chip works on a narrow
+// output without slices of K: the products around a folded RMSNorm (linear_skinny.hip describes
+// the fold), which need whole sums.  The streaming kernel there loads 16 rows of w by 64 bytes
+// per instruction, and its counters show the texture addresser stalled half of the time; this
+// kernel asks for the same bytes as whole lines.
+//
+// A workgroup of four waves owns R <= 32 features (R from N alone, so that the workgroups are a
+// multiple of the 256 compute units) and all of K.  It walks K in tiles of 256: all 256 threads
+// copy the w tile [32 rows, 512 bytes each: 32 lanes a row] and the x tile [16 rows] from
+// memory into registers, two tiles ahead, and from there into LDS (double buffered, one barrier
+// a tile); wave v multiplies k steps 2v and 2v+1 of the tile's eight (v_mfma_f32_16x16x32_bf16,
+// A = 16 rows of w, B = the 16 rows of x), two tiles of 16 features each.  At the end the four
+// waves' sums are added through LDS in wave order and stored: plain (MODE 0), adding into the
+// float32 residual stream and handing on round(stream * g) and the rows' sums of squares (MODE
+// 1), or scaling the rows by rsqrt(sum of the parts / K + eps) (MODE 2).
+//
+// Workgroup b starts b * rotate tiles into K and wraps around (see linear_mid.hip).  An output
+// element's value depends on (N, K) alone, never on M or on what else is in the batch.
+//
+// Reference call site: candle matmul in /root/reference/src/models/layers/linear.rs:76-124.
+#include "common.h"
+
+namespace xi {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr int kThinRows = 16;            // rows of x
+constexpr int kThinFeatures = 32;        // rows of w in a workgroup's tile
+constexpr int kThinK = 256;              // k per tile
+constexpr int kThinLdsRow = kThinK + 8;  // elements of a row in LDS
+constexpr int kThinDepth = 2;            // tiles whose loads are in flight
+constexpr int kThinSsLoads = 32;         // 16 threads x 32 loads: up to 512 parts of a row's sum of squares
+constexpr int kThinStage = (kThinFeatures + kThinRows) * kThinLdsRow;   // elements of one buffer
+
+struct ThinFold {
+  float* resid;         // MODE 1: [M, N] float32, updated in place
+  const float* g;       // MODE 1: [N] weight of the norm that follows
+  bf16* xg;             // MODE 1: [M, N]
+  float* ss_out;        // MODE 1: [M, gridDim.x]
+  const float* ss_in;   // MODE 2: [M, parts]
+  int parts;            // MODE 2
+  float eps;            // MODE 2
+  float inv_h;          // MODE 2: 1 / length of the normed rows
+};
+
+template <int MODE, typename TO>
+__global__ __launch_bounds__(256) void linear_thin_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
+                                                          TO* __restrict__ y, int M, int N, int K, int R, int rotate,
+                                                          ThinFold fold) {
+  constexpr int D = kThinDepth;
+  __shared__ __align__(16) bf16 lds[2 * kThinStage];          // [buffer][w tile 32 rows | x tile 16 rows][kThinLdsRow]
+  __shared__ __align__(16) float red[4 * 2 * 256];            // [wave][feature tile][lane * 4 + i]
+  __shared__ float side[MODE == 1 ? kThinRows * kThinFeatures : kThinRows];   // squares [row][feature], or 1/rms [row]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, j = lane >> 4;
+  const int n0 = blockIdx.x * R;
+  const int n_last = (n0 + R < N ? n0 + R : N) - 1;
+  const int nkt = K / kThinK;
+  const int start = (int)(((long long)blockIdx.x * rotate) % nkt);
+
+  // MODE 2: 16 threads per row add up the parts of its sum of squares; the loads start now
+  float ss_mine[MODE == 2 ? kThinSsLoads : 1];
+  if constexpr (MODE == 2) {
+    const int token = tid >> 4, sub = tid & 15;
+#pragma unroll
+    for (int i = 0; i < kThinSsLoads; ++i) {
+      const int p = sub + 16 * i;
+      ss_mine[i] = (token < M && p < fold.parts) ? fold.ss_in[(size_t)token * fold.parts + p] : 0.f;
+    }
+  }
+
+  // ---- copying: a row of a tile is 32 16-byte chunks; thread t moves chunk t % 32 of rows
+  // t / 32 + 8 i of w (i < 4) and of x (i < 2).  Rows past the workgroup's last feature read
+  // that feature's row again, rows of x past M row M - 1; no load is conditional.
+  const int srow = tid >> 5, skc = tid & 31;
+  const bf16* wsrc[4];
+  const bf16* xsrc[2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int n = n0 + srow + 8 * i;
+    n = n < n_last ? n : n_last;
+    wsrc[i] = w + (size_t)n * K + 8 * skc;
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = srow + 8 * i;
+    xsrc[i] = x + (size_t)(row < M ? row : M - 1) * K + 8 * skc;
+  }
+  const int sdst = srow * kThinLdsRow + 8 * skc;
+  bf16x8 wr[D][4], xr[D][2];
+  f32x4 acc[2];
+  acc[0] = f32x4{0.f, 0.f, 0.f, 0.f};
+  acc[1] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+#define XI_THIN_ISSUE(slot, t)                                                           \
+  do {                                                                                   \
+    int tt_ = (t) + start;                                                               \
+    tt_ = tt_ >= nkt ? tt_ - nkt : tt_;                                                  \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                        \
+      wr[slot][i] = *reinterpret_cast<const bf16x8*>(wsrc[i] + (size_t)tt_ * kThinK);    \
+    _Pragma("unroll") for (int i = 0; i < 2; ++i)                                        \
+      xr[slot][i] = *reinterpret_cast<const bf16x8*>(xsrc[i] + (size_t)tt_ * kThinK);    \
+  } while (0)
+
+  // every copy is issued whether or not its tile exists (past the end the last tile is read
+  // again and dropped), so that the wait before a tile's use leaves the younger loads in flight
+  const int last = nkt - 1;
+#pragma unroll
+  for (int s = 0; s < D; ++s) XI_THIN_ISSUE(s, s < last ? s : last);
+
+  int buf = 0;
+#define XI_THIN_TILE(s, t)                                                                                \
+  do {                                                                                                    \
+    bf16* Ws = lds + buf * kThinStage;                                                                    \
+    bf16* Xs = Ws + kThinFeatures * kThinLdsRow;                                                          \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                         \
+      *reinterpret_cast<bf16x8*>(Ws + sdst + 8 * i * kThinLdsRow) = wr[s][i];                             \
+    _Pragma("unroll") for (int i = 0; i < 2; ++i)                                                         \
+      *reinterpret_cast<bf16x8*>(Xs + sdst + 8 * i * kThinLdsRow) = xr[s][i];                             \
+    XI_THIN_ISSUE(s, (t) + D < last ? (t) + D : last);                                                    \
+    __syncthreads();                                                                                      \
+    _Pragma("unroll") for (int kk = 0; kk < 2; ++kk) {                                                    \
+      const int col = 32 * (2 * wave + kk) + 8 * j;                                                       \
+      const bf16x8 b = *reinterpret_cast<const bf16x8*>(Xs + r * kThinLdsRow + col);                      \
+      const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(Ws + r * kThinLdsRow + col);                     \
+      const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(Ws + (16 + r) * kThinLdsRow + col);              \
+      acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b, acc[0], 0, 0, 0);                           \
+      acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b, acc[1], 0, 0, 0);                           \
+    }                                                                                                     \
+    buf ^= 1;                                                                                             \
+  } while (0)
+
+  // whole rotations of the slots in a loop without exits inside, then the tiles that are left;
+  // one barrier a tile is enough (see linear_mid.hip)
+  int t0 = 0;
+  for (; t0 + D <= nkt; t0 += D) {
+#pragma unroll
+    for (int s = 0; s < D; ++s) XI_THIN_TILE(s, t0 + s);
+  }
+#pragma unroll
+  for (int s = 0; s < D - 1; ++s)
+    if (t0 + s < nkt) XI_THIN_TILE(s, t0 + s);     // the same for every thread
+#undef XI_THIN_TILE
+#undef XI_THIN_ISSUE
+
+  // ---- the four waves' sums through LDS, added in wave order.  A lane's 4 values of a tile:
+  // row r of x, features 4 j .. 4 j + 3 of the tile.
+  *reinterpret_cast<f32x4*>(&red[(wave * 2 + 0) * 256 + lane * 4]) = acc[0];
+  *reinterpret_cast<f32x4*>(&red[(wave * 2 + 1) * 256 + lane * 4]) = acc[1];
+  if constexpr (MODE == 2) {
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < kThinSsLoads; ++i) t += ss_mine[i];
+#pragma unroll
+    for (int o = 8; o; o >>= 1) t += __shfl_xor(t, o, kWave);
+    if ((tid & 15) == 0) side[tid >> 4] = rsqrtf(t * fold.inv_h + fold.eps);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int e = tid;                       // element of feature tile h
+    const int ln = e >> 2, v = e & 3;
+    const int token = ln & 15, f = 16 * h + 4 * (ln >> 4) + v;      // feature within the workgroup's tile
+    const int n = n0 + f;
+    float a = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < 4; ++wv) a += red[(wv * 2 + h) * 256 + e];
+    const bool mine = n <= n_last && token < M;
+    if constexpr (MODE == 1) {
+      float sq = 0.f;
+      if (mine) {
+        const float rr = fold.resid[(size_t)token * N + n] + a;
+        fold.resid[(size_t)token * N + n] = rr;
+        fold.xg[(size_t)token * N + n] = from_float<bf16>(rr * fold.g[n]);
+        sq = rr * rr;
+      }
+      side[token * kThinFeatures + f] = sq;
+    } else {
+      if constexpr (MODE == 2) a *= side[token];
+      if (mine) y[(size_t)token * N + n] = from_float<TO>(a);
+    }
+  }
+  if constexpr (MODE == 1) {     // a row's squares summed in the order of the features
+    __syncthreads();
+    if (tid < kThinRows && tid < M) {
+      float t = 0.f;
+      for (int i = 0; i < kThinFeatures; ++i) t += side[tid * kThinFeatures + i];
+      fold.ss_out[(size_t)tid * gridDim.x + blockIdx.x] = t;
+    }
+  }
+}
+
+// Features per workgroup: the fewest workgroups that are a multiple of the 256 compute units
+// with at most 32 features each.  From N alone.
+static int thin_features(int N) {
+  for (int waves = 1; waves <= 1024; ++waves) {
+    const int rr = (N + 256 * waves - 1) / (256 * waves);
+    if (rr <= kThinFeatures) return rr < 1 ? 1 : rr;
+  }
+  return kThinFeatures;
+}
+
+}  // namespace xi
+
+using namespace xi;
+
+extern "C" {
+
+// 0 if the sizes are not taken.
+int xi_linear_thin_features(int N, int K) {
+  if (N < 1 || K < kThinK || K % kThinK) return 0;
+  return thin_features(N);
+}
+
+// Workgroups (= parts of a row's sum of squares that xi_linear_thin_fold_out hands on).
+int xi_linear_thin_parts(int N, int K) {
+  const int R = xi_linear_thin_features(N, K);
+  return R ? (N + R - 1) / R : 0;
+}
+
+static int thin_check(const char* what, const void* x, const void* w, int M, int N, int K) {
+  XI_CHECK(M >= 1 && M <= kThinRows, "%s: M=%d must be 1..%d", what, M, kThinRows);
+  XI_CHECK(N >= 1 && K >= kThinK && K % kThinK == 0, "%s: N=%d, K=%d (a multiple of %d) are not taken", what, N, K, kThinK);
+  XI_CHECK(((uintptr_t)x | (uintptr_t)w) % 16 == 0, "%s: operands must be 16-byte aligned", what);
+  XI_CHECK((long long)(N + thin_features(N) - 1) / thin_features(N) < (1ll << 31), "%s: too many workgroups", what);
+  return 0;
+}
+
+// y [M, N] bfloat16 (out_dtype 1) or float32 (0).
+int xi_linear_thin(const void* x, const void* w, void* y, int M, int N, int K, int out_dtype, int rotate,
+                   hipStream_t stream) {
+  if (thin_check("linear_thin", x, w, M, N, K)) return 1;
+  XI_CHECK(rotate >= 0, "linear_thin: rotate=%d", rotate);
+  const int R = thin_features(N);
+  const unsigned wgs = (unsigned)((N + R - 1) / R);
+  const ThinFold none{nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0.f, 0.f};
+  if (out_dtype == kBF16)
+    linear_thin_kernel<0, bf16><<<wgs, 256, 0, stream>>>((const bf16*)x, (const bf16*)w, (bf16*)y, M, N, K, R, rotate, none);
+  else if (out_dtype == kF32)
+    linear_thin_kernel<0, float><<<wgs, 256, 0, stream>>>((const bf16*)x, (const bf16*)w, (float*)y, M, N, K, R, rotate, none);
+  else
+    XI_CHECK(false, "linear_thin: unknown dtype %d", out_dtype);
+  XI_LAUNCH_CHECK("linear_thin");
+  return 0;
+}
+
+// resid [M, N] float32 += x @ w^T; xg [M, N] = round(resid * g); ss [M, xi_linear_thin_parts(N, K)].
+int xi_linear_thin_fold_out(const void* x, const void* w, int M, int N, int K, float* resid, const float* g, void* xg,
+                            float* ss, int rotate, hipStream_t stream) {
+  if (thin_check("linear_thin_fold_out", x, w, M, N, K)) return 1;
+  XI_CHECK(resid && g && xg && ss && rotate >= 0, "linear_thin_fold_out: missing operands");
+  const int R = thin_features(N);
+  const unsigned wgs = (unsigned)((N + R - 1) / R);
+  const ThinFold fold{resid, g, (bf16*)xg, ss, nullptr, 0, 0.f, 0.f};
+  linear_thin_kernel<1, bf16><<<wgs, 256, 0, stream>>>((const bf16*)x, (const bf16*)w, (bf16*)nullptr, M, N, K, R, rotate, fold);
+  XI_LAUNCH_CHECK("linear_thin_fold_out");
+  return 0;
+}
+
+// y [M, N] = (xg @ w^T) with row t scaled by rsqrt(sum(ss[t]) / K + eps); ss [M, parts], parts <= 512.
+int xi_linear_thin_fold_in(const void* xg, const void* w, void* y, int M, int N, int K, int out_dtype, const float* ss,
+                           int parts, float eps, int rotate, hipStream_t stream) {
+  if (thin_check("linear_thin_fold_in", xg, w, M, N, K)) return 1;
+  XI_CHECK(ss && parts >= 1 && parts <= 16 * kThinSsLoads && rotate >= 0, "linear_thin_fold_in: %d parts (1..%d)", parts,
+           16 * kThinSsLoads);
+  const int R = thin_features(N);
+  const unsigned wgs = (unsigned)((N + R - 1) / R);
+  const ThinFold fold{nullptr, nullptr, nullptr, nullptr, ss, parts, eps, 1.f / (float)K};
+  if (out_dtype == kBF16)
+    linear_thin_kernel<2, bf16><<<wgs, 256, 0, stream>>>((const bf16*)xg, (const bf16*)w, (bf16*)y, M, N, K, R, rotate, fold);
+  else if (out_dtype == kF32)
+    linear_thin_kernel<2, float><<<wgs, 256, 0, stream>>>((const bf16*)xg, (const bf16*)w, (float*)y, M, N, K, R, rotate, fold);
+  else
+    XI_CHECK(false, "linear_thin_fold_in: unknown dtype %d", out_dtype);
+  XI_LAUNCH_CHECK("linear_thin_fold_in");
+  return 0;
+}
+
+}  // extern "C"

@@ -595,6 +595,84 @@ def linear_fold_in(xg: torch.Tensor, ss: torch.Tensor, eps: float, w: torch.Tens
     return y
 
 
+THIN_ROTATE = 0           # workgroup b of the thin product starts b * this many k tiles into K (see MID_ROTATE;
+                          # here it measured no gain: 0)
+
+
+THIN_WORK = 96_000        # rows x K from which the thin product is ahead of the streaming kernel where that
+                          # kernel's workgroups own whole tiles of 16 features (N a multiple of 4096); where they
+                          # do not (N = 5120: 20 features, 6144: 24) the thin product is ahead from the first row.
+                          # Measured in decode steps at Qwen3-8B, 14B and 32B sizes (3% of a step at the larger two).
+
+
+def thin_ahead(M: int, w: torch.Tensor) -> bool:
+    """Whether a product of M <= FOLD_ROWS rows with whole sums goes to the thin kernel."""
+    if w.dtype != torch.bfloat16 or not (0 < M <= FOLD_ROWS):
+        return False
+    parts = linear_thin_parts(w.shape[0], w.shape[1])
+    return 0 < parts <= FOLD_PARTS and (w.shape[0] % 4096 != 0 or M * w.shape[1] >= THIN_WORK)
+
+
+def linear_thin_parts(N: int, K: int) -> int:
+    """Workgroups of the thin product for an output of N features (the parts in which
+    `linear_thin_fold_out` hands on a row's sum of squares); 0 if it does not take the sizes."""
+    return int(lib().xi_linear_thin_parts(int(N), int(K)))
+
+
+def _thin_operands(what: str, x: torch.Tensor, w: torch.Tensor):
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError(f"{what}: operands must be bfloat16")
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
+        raise KernelError(f"{what}: x {tuple(x.shape)} and w {tuple(w.shape)} do not match")
+    M, K = x.shape
+    N = w.shape[0]
+    if not (0 < M <= FOLD_ROWS) or linear_thin_parts(N, K) < 1:
+        raise KernelError(f"{what}: M={M} must be 1..{FOLD_ROWS} and K={K} a multiple of 256")
+    return M, N, K
+
+
+def linear_thin(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """bfloat16 x [M, K] @ w [N, K]^T for up to FOLD_ROWS rows, whole sums (no slices of K) with few
+    output features per workgroup, loaded as whole lines through LDS: the shape of the products
+    around a folded norm."""
+    _dev(x, w)
+    M, N, K = _thin_operands("linear_thin", x, w)
+    y = torch.empty((M, N), dtype=out_dtype or torch.bfloat16, device=x.device)
+    _ok(lib().xi_linear_thin(_p(x), _p(w), _p(y), M, N, K, _code(y, "linear_thin"), int(THIN_ROTATE), _stream()))
+    return y
+
+
+def linear_thin_fold_out(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, norm_weight: torch.Tensor):
+    """`linear_fold_out` with the thin kernel: resid [M, N] float32 += x @ w^T in place; returns
+    (xg, ss) with ss [M, linear_thin_parts(N, K)]."""
+    _dev(x, w, resid, norm_weight)
+    M, N, K = _thin_operands("linear_thin_fold_out", x, w)
+    _want(resid, torch.float32, "linear_thin_fold_out: resid")
+    _want(norm_weight, torch.float32, "linear_thin_fold_out: norm weight")
+    if tuple(resid.shape) != (M, N) or tuple(norm_weight.shape) != (N,):
+        raise KernelError(f"linear_thin_fold_out: resid {tuple(resid.shape)} / norm weight {tuple(norm_weight.shape)} "
+                          f"do not match [M={M}, N={N}]")
+    xg = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    ss = torch.empty((M, linear_thin_parts(N, K)), dtype=torch.float32, device=x.device)
+    _ok(lib().xi_linear_thin_fold_out(_p(x), _p(w), M, N, K, _p(resid), _p(norm_weight), _p(xg), _p(ss),
+                                      int(THIN_ROTATE), _stream()))
+    return xg, ss
+
+
+def linear_thin_fold_in(xg: torch.Tensor, ss: torch.Tensor, eps: float, w: torch.Tensor,
+                        out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """`linear_fold_in` (plain form) with the thin kernel."""
+    _dev(xg, ss, w)
+    M, N, K = _thin_operands("linear_thin_fold_in", xg, w)
+    _want(ss, torch.float32, "linear_thin_fold_in: ss")
+    if ss.dim() != 2 or ss.shape[0] != M or not (0 < ss.shape[1] <= FOLD_PARTS):
+        raise KernelError(f"linear_thin_fold_in: ss {tuple(ss.shape)} is not [M={M}, up to {FOLD_PARTS} parts]")
+    y = torch.empty((M, N), dtype=out_dtype or torch.bfloat16, device=xg.device)
+    _ok(lib().xi_linear_thin_fold_in(_p(xg), _p(w), _p(y), M, N, K, _code(y, "linear_thin_fold_in"), _p(ss),
+                                     int(ss.shape[1]), ctypes.c_float(eps), int(THIN_ROTATE), _stream()))
+    return y
+
+
 def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
                 skinny_rows: int = SKINNY_ROWS, allow_split: bool = False) -> torch.Tensor:
     """bfloat16 x @ w.T with float32 accumulation, rounded once to `out_dtype` (bfloat16 or
@@ -617,6 +695,8 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtyp
         skinny_rows = max(skinny_rows, SKINNY_SPLIT_ROWS)
     else:
         allow_split = False
+    if not allow_split and thin_ahead(x.shape[0], w):
+        return linear_thin(x, w, out_dtype)
     if 0 < x.shape[0] <= min(skinny_rows, SKINNY_MAX_ROWS) and x.shape[1] % 8 == 0:
         return linear_skinny(x, w, out_dtype, allow_split=allow_split)
     if out_dtype == torch.float32:

@@ -45,6 +45,8 @@ class Linear:
             if w.dtype == torch.bfloat16 and x.xg.shape[1] % 8 == 0 and (not gated or out_dtype in (None, torch.bfloat16)):
                 if gated and kernels.gated_uses_mid(x.xg.shape[0], w):
                     return kernels.linear_mid_gated(x.xg, w, x.ss, x.norm.eps)
+                if not gated and kernels.thin_ahead(x.xg.shape[0], w):
+                    return kernels.linear_thin_fold_in(x.xg, x.ss, x.norm.eps, w, out_dtype or torch.bfloat16)
                 return kernels.linear_fold_in(x.xg, x.ss, x.norm.eps, w, out_dtype or torch.bfloat16, gated=gated)
             x = x.rows(torch.bfloat16 if w.dtype == torch.bfloat16 else torch.float32)
         if gated:
@@ -60,7 +62,8 @@ class Linear:
                 and sink.norm.foldable and sink.norm.weight.shape[0] == w.shape[0]
                 and sink.resid.dtype == torch.float32 and sink.resid.is_contiguous()
                 and kernels.linear_fold_parts(x.shape[0], w.shape[0], w.shape[1]) <= kernels.FOLD_PARTS):
-            xg, ss = kernels.linear_fold_out(x, w, sink.resid, sink.norm.weight)
+            fold_out = kernels.linear_thin_fold_out if kernels.thin_ahead(x.shape[0], w) else kernels.linear_fold_out
+            xg, ss = fold_out(x, w, sink.resid, sink.norm.weight)
             return Folded(xg, ss, sink.norm)
         out_dtype = out_dtype or x.dtype
         if w.dtype == torch.float32:
