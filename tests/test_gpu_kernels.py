@@ -276,31 +276,34 @@ def test_linear_thin_refuses():
     assert kernels.linear_thin_parts(10240, 5120) == 512 and kernels.linear_thin_parts(64, 100) == 0
 
 
-def test_fold_gives_way_to_the_tiled_product():
-    """A product before a norm adds into the stream itself for few rows, but with a long K and
-    many of those rows it leaves the norm to its own kernel and answers with partial sums."""
+def test_linear_chooses_the_kernel_of_a_folded_product():
+    """A product before a norm adds into the stream itself for up to 16 rows: with the thin kernel
+    where N is no multiple of 4096 or rows x K is large, else with the streaming kernel; more rows
+    come back as partial sums of the tiled kernel for the norm to add."""
     from xinfer_amd import kernels
     from xinfer_amd.config.spec import PartSpec
     from xinfer_amd.parts.base import Folded, NormSink, norm_class
     from xinfer_amd.parts.linear import Linear
     g = torch.Generator().manual_seed(3)
-    N, K = 256, 8192
-    lin = Linear(_rand((N, K), torch.bfloat16, g, 0.02).to(DEV))
-    norm = norm_class("rmsnorm")(PartSpec("rmsnorm", dict(dim=N, eps=1e-6)), torch.bfloat16)
-    norm.weight = torch.ones(N, device=DEV)
-    for M, folded in ((4, True), (12, True), (13, False), (16, False)):
-        x = _rand((M, K), torch.bfloat16, g).to(DEV)
-        resid = torch.zeros((M, N), device=DEV)
-        y = lin(x, allow_split=True, sink=NormSink(resid, norm))
-        ref = x.cpu().double() @ lin.weight.cpu().double().T
-        assert kernels.fold_loses_to_mid(M, lin.weight) == (not folded)
-        if folded:
-            assert isinstance(y, Folded)
-            assert (resid.cpu().double() - ref).abs().max() / ref.abs().max() < 1e-5
-        else:
-            assert y.dtype == torch.float32 and tuple(y.shape) == (kernels.linear_mid_slices(N, K), M, N)
-            assert float(resid.abs().max()) == 0.0
-            assert (y.cpu().double().sum(0) - ref).abs().max() / ref.abs().max() < 1e-5
+    for N, K in ((256, 8192), (4096, 2048)):
+        lin = Linear(_rand((N, K), torch.bfloat16, g, 0.02).to(DEV))
+        norm = norm_class("rmsnorm")(PartSpec("rmsnorm", dict(dim=N, eps=1e-6)), torch.bfloat16)
+        norm.weight = torch.ones(N, device=DEV)
+        for M in (4, 16, 40):
+            x = _rand((M, K), torch.bfloat16, g).to(DEV)
+            resid = torch.zeros((M, N), device=DEV)
+            y = lin(x, allow_split=True, sink=NormSink(resid, norm))
+            ref = x.cpu().double() @ lin.weight.cpu().double().T
+            if M <= kernels.FOLD_ROWS:
+                assert isinstance(y, Folded)
+                thin = kernels.thin_ahead(M, lin.weight)
+                assert thin == (N % 4096 != 0 or M * K >= kernels.THIN_WORK)
+                assert y.ss.shape[1] == (kernels.linear_thin_parts(N, K) if thin else kernels.linear_fold_parts(M, N, K))
+                assert (resid.cpu().double() - ref).abs().max() / ref.abs().max() < 1e-5
+            else:
+                assert y.dtype == torch.float32 and tuple(y.shape) == (kernels.linear_mid_slices(N, K), M, N)
+                assert float(resid.abs().max()) == 0.0
+                assert (y.cpu().double().sum(0) - ref).abs().max() / ref.abs().max() < 1e-5
 
 
 def test_linear_folded_norm_refuses():

@@ -519,18 +519,6 @@ def linear_mid_gated(x: torch.Tensor, w: torch.Tensor, ss: Optional[torch.Tensor
     return y
 
 
-FOLD_UP_TO_WORK = 100_000  # rows x K from which the tiled product plus a norm kernel is ahead of the folded streaming
-                           # product (measured in decode steps at Qwen3-8B, 14B and 32B sizes: 7% of a step at 16 rows
-                           # of the larger two; between 50,000 and 100,000 nothing changes)
-
-
-def fold_loses_to_mid(M: int, w: torch.Tensor) -> bool:
-    """Whether a product of M <= FOLD_ROWS rows before a norm should leave the norm to its own kernel and
-    run as the tiled product: with a long K the streaming kernel's workgroups, 16 features each,
-    re-read so much of x that the saved kernel does not pay."""
-    return M * w.shape[1] >= FOLD_UP_TO_WORK and linear_mid_slices(w.shape[0], w.shape[1]) > 0 and w.shape[0] <= MID_WIDEST
-
-
 FOLD_ROWS = 16            # most rows of the products that carry a folded norm between them
 FOLD_PARTS = 512          # most parts of a row's sum of squares the product after the norm adds up
 
@@ -688,7 +676,7 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtyp
             and linear_mid_slices(w.shape[0], w.shape[1]) == 1:
         return linear_mid(x, w)[0]           # a wide output in float32 (the head): one slice is the result
     if allow_split and x.shape[0] <= MID_ROWS and linear_mid_slices(w.shape[0], w.shape[1]) > 0 \
-            and w.shape[0] <= MID_WIDEST and (MID_FROM <= x.shape[0] or fold_loses_to_mid(x.shape[0], w)):
+            and w.shape[0] <= MID_WIDEST and MID_FROM <= x.shape[0]:
         return linear_mid(x, w)
     if (allow_split and x.shape[1] % 8 == 0 and x.shape[0] >= SKINNY_SPLIT_FROM
             and int(lib().xi_linear_skinny_slices(w.shape[0], w.shape[1], 0, 1)) > 1):

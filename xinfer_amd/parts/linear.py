@@ -58,7 +58,6 @@ class Linear:
             return None
         if (sink is not None and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2
                 and 0 < x.shape[0] <= kernels.FOLD_ROWS and x.shape[1] % 8 == 0 and w.shape[0] % 8 == 0
-                and not (allow_split and kernels.fold_loses_to_mid(x.shape[0], w))
                 and sink.norm.foldable and sink.norm.weight.shape[0] == w.shape[0]
                 and sink.resid.dtype == torch.float32 and sink.resid.is_contiguous()
                 and kernels.linear_fold_parts(x.shape[0], w.shape[0], w.shape[1]) <= kernels.FOLD_PARTS):
