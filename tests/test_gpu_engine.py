@@ -44,6 +44,7 @@ def test_argmax_lowest_index_wins_ties(V):
 @pytest.mark.parametrize("V,T,k,p", [
     (256, 0.8, 0, 1.0), (509, 1.3, 0, 1.0), (300, 0.7, 32, 1.0), (300, 0.7, 0, 0.9),
     (300, 0.7, 32, 0.95), (2000, 1.0, 5, 0.5), (151936, 0.7, 32, 0.95), (151936, 1.0, 0, 0.8),
+    (151936, 0.9, 64, 1.0), (151936, 0.7, 65, 0.95), (5000, 1.1, 1, 0.3), (163841, 0.8, 7, 0.6),
 ])
 def test_sample_matches_plain(V, T, k, p, coarse):
     from xinfer_amd.sampling import Sampler, Strategy

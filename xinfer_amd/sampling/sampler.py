@@ -21,6 +21,7 @@ import torch
 from .. import kernels
 from ..config.engine_config import GenerationConfig, SamplingParams
 
+TOPK_FAST = 64             # largest top-k of the two-stage selection (`sampling_topk.hip`)
 PENALTY_CONTEXT = 128      # last generated tokens that penalties look at (runner.rs:1887-1912)
 _MASK = (1 << 64) - 1
 
@@ -133,6 +134,18 @@ class Sampler:
                                                      kernels._p(fr_d), kernels._p(pr_d), kernels._stream()))
         if all(s.greedy for s in strategies):
             return self.argmax(logits).tolist()
+        chunks = int(self._lib.xi_sample_topk_chunks(V))
+        if chunks > 0 and all(s.greedy or 1 <= s.top_k <= TOPK_FAST for s in strategies):
+            # a small top-k everywhere (the default strategy has 32): the k most probable of a row
+            # are found by many workgroups, the rest is about k numbers
+            par = torch.tensor([[s.temperature for s in strategies], [float(s.top_k) for s in strategies],
+                                [s.top_p for s in strategies], list(uniforms)], dtype=torch.float32).to(dev)
+            cand_v = torch.empty((R, chunks, TOPK_FAST), dtype=torch.float32, device=dev)
+            cand_i = torch.empty((R, chunks, TOPK_FAST), dtype=torch.int32, device=dev)
+            out = torch.empty((R,), dtype=torch.int32, device=dev)
+            kernels._ok(self._lib.xi_sample_topk(kernels._p(logits), R, V, kernels._p(par), kernels._p(cand_v),
+                                                 kernels._p(cand_i), kernels._p(out), kernels._stream()))
+            return out.tolist()
         t = torch.tensor([s.temperature for s in strategies], dtype=torch.float32, device=dev)
         k = torch.tensor([s.top_k for s in strategies], dtype=torch.int32, device=dev)
         p = torch.tensor([s.top_p for s in strategies], dtype=torch.float32, device=dev)
