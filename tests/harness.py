@@ -95,6 +95,17 @@ def trace_mixed(reqs: Dict[str, List[int]], seed: int, max_live: int = 4, tail: 
     return steps
 
 
+def trace_batch_decode(reqs: Dict[str, List[int]], tail: int = 4) -> List[dict]:
+    """All requests live together: their heads as portions of one step, then `tail` steps that
+    bring one token of every request (a wide decode batch), every position wanted."""
+    steps = [{"step": 0, "end": [], "entries": [
+        {"id": rid, "tokens": toks[:len(toks) - tail], "want": list(range(len(toks) - tail))} for rid, toks in reqs.items()]}]
+    for k in range(tail):
+        steps.append({"step": 1 + k, "end": list(reqs) if k == tail - 1 else [], "entries": [
+            {"id": rid, "tokens": [toks[len(toks) - tail + k]], "want": [0]} for rid, toks in reqs.items()]})
+    return steps
+
+
 def tokens_needed(steps: List[dict], page: int) -> int:
     """The most tokens live requests hold at any time, each rounded up to a page."""
     held: Dict[str, int] = {}

@@ -131,3 +131,28 @@ def test_real_layer_sizes(name, real_model_dirs):
             del runner
         del model
         torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("name,live", [("8B", 12), ("8B", 40), ("32B", 16), ("32B", 70)])
+def test_real_layer_sizes_wide_decode_batches(name, live, real_model_dirs):
+    """Decode steps of many requests at real layer sizes, in bfloat16: the kernels that serve 6 to
+    16 rows (thin products with the folded norm, the gated tiled product), 17 to 64 (tiled
+    products with partial sums) and more (the library beside them), inside the model against
+    the plain implementation; the steps are launched one by one and, the third time on, replayed
+    from a graph."""
+    from xinfer_amd.engine import ModelRunner, load_model
+    t = REAL[name]
+    d = real_model_dirs(name)
+    vocab, page = t["config"]["vocab_size"], t["page_size"]
+    rng = random.Random(11)
+    reqs = {f"r{i}": harness.random_prompt(rng, rng.randrange(8, 30), vocab) for i in range(live)}
+    pm = plain.PlainModel(d)
+    ref = {rid: pm.logits(toks) for rid, toks in reqs.items()}
+    del pm
+    model = load_model(d, "bfloat16", "cuda:0")
+    steps = harness.trace_batch_decode(reqs, tail=5)
+    runner = ModelRunner(model, page_size=page, num_pages=live + 2, max_requests=live, graph_after=3, graph_max_batch=64)
+    got = harness.replay(runner, steps)
+    rel = harness.compare(got, ref, harness.TOL["bfloat16"], f"{name}/bfloat16/decode batch of {live}")
+    print(f"{name}/decode batch of {live}: worst error {rel:.2e} of the largest logit")
+    assert (runner.graph_replays > 0) == (live <= 64)
