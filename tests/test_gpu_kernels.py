@@ -755,6 +755,40 @@ def test_attention_prefill_mfma(nq, nkv, d, page, window, seqs):
     assert err < _tol(torch.bfloat16, 2), err
 
 
+@pytest.mark.parametrize("nq,nkv,d,page,window", [(8, 2, 64, 16, 0), (5, 5, 48, 16, 24), (32, 8, 128, 64, 0), (10, 2, 128, 64, 0)])
+def test_attention_of_a_mixed_batch_splits_between_the_kernels(nq, nkv, d, page, window):
+    """A step's attention as the engine asks for it: single tokens of decoding requests at the head of
+    the batch go to the decode kernel, the portions behind them to the prefill kernel, into one
+    result; with fewer than four at the head, or one of them elsewhere, the prefill kernel takes all."""
+    from types import SimpleNamespace
+    from xinfer_amd import kernels
+    if not kernels.mfma_attention_supported(nq, nkv, d, page):
+        pytest.skip("the matrix-core kernels need a page of a power of two of at least 8 tokens")
+    scale = 1.0 / math.sqrt(d)
+    for seqs, split in (([(300, 1), (77, 1), (1, 1), (1030, 1), (64, 1), (90, 40), (200, 200), (17, 1), (33, 2)], True),
+                        ([(300, 1), (77, 1), (90, 40), (64, 1), (31, 1)], False)):
+        g = torch.Generator().manual_seed(33)
+        case = _paged_case(g, torch.bfloat16, nq, nkv, d, page, seqs)
+        ref = _attention_ref(case, seqs, window, scale)
+        q, kc, vt, bt = _mfma_inputs(case)
+        cu, cl = _cu_ctx(seqs)
+        ctx = SimpleNamespace(block_tables=[bt], ctx_lens=cl.to(DEV), cu_q=cu.to(DEV), max_q_len=max(n for _, n in seqs),
+                              max_ctx_len=max(c for c, _ in seqs), num_seqs=len(seqs), cu_q_host=cu.tolist(),
+                              ctx_lens_host=cl.tolist(), scratch={}, similar_lengths=False,
+                              tok_seq=case["tok_seq"].to(DEV), positions=case["positions"].to(DEV))
+        kernels_work = kernels.MIXED_DECODE_WORK
+        kernels.MIXED_DECODE_WORK = 1000          # small sizes here: the rule's threshold is for real ones
+        try:
+            out = kernels.attention(q, kc, vt, ctx, 0, scale, window, v_transposed=True)
+        finally:
+            kernels.MIXED_DECODE_WORK = kernels_work
+        (tiles, small, lead, lead_ctx), = ctx.scratch.values()
+        assert (lead, lead_ctx) == ((5, 1030) if split else (0, 0))
+        assert sorted(set(tiles[:, 0].tolist())) == [b for b in range(len(seqs)) if b >= lead]
+        err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
+        assert err < _tol(torch.bfloat16, 2), (split, err)
+
+
 DECODE_CASES = [
     (4, 2, 32, 16, 0, [(5, 1), (17, 1), (33, 1), (1, 1)]),
     (6, 2, 16, 8, 0, [(200, 1), (130, 1), (513, 1)]),

@@ -306,9 +306,13 @@ def prefill_block(d: int, group: int = 1, small: bool = False) -> int:
 
 
 COMPUTE_UNITS = 256
+MIXED_DECODE_FROM = 4          # single-token sequences at the head of a mixed batch from which they may go to the decode
+MIXED_DECODE_WORK = 40_000     # kernel: where sequences x longest context x reads of a kv head's keys reach this,
+MIXED_DECODE_CONTEXT = 4096    # or the longest context this (measured on MI355X beside a portion of 2,000 tokens:
+                               # 40 query heads on 8 kv heads, 64 sequences at 1,500 keys: 450 -> 155 us a layer)
 
 
-def prefill_tiles(q_lens, ctx_lens, d: int, nq: int, nkv: int, small: Optional[bool] = None):
+def prefill_tiles(q_lens, ctx_lens, d: int, nq: int, nkv: int, small: Optional[bool] = None, first_seq: int = 0):
     """The query blocks of a batch of portions for the prefill kernel: (rows, small).
     rows = [(sequence, first query of the block)] in launch order.  A block's work grows
     with the keys it sees, and the compute units take workgroups in launch order, so the
@@ -321,9 +325,9 @@ def prefill_tiles(q_lens, ctx_lens, d: int, nq: int, nkv: int, small: Optional[b
     heads = nkv * (g // (4 if g % 4 == 0 else 2 if g % 2 == 0 else 1))     # workgroups per query block
     big = prefill_block(d, g, False)
     if small is None:
-        small = sum(-(-n // big) for n in q_lens) * heads < 2 * COMPUTE_UNITS
+        small = sum(-(-n // big) for n in q_lens[first_seq:]) * heads < 2 * COMPUTE_UNITS
     qb = prefill_block(d, g, small)
-    rows = [(b, q0) for b, n in enumerate(q_lens) for q0 in range(0, n, qb)]
+    rows = [(b, q0) for b, n in enumerate(q_lens) if b >= first_seq for q0 in range(0, n, qb)]
     rows.sort(key=lambda t: -(ctx_lens[t[0]] - q_lens[t[0]] + t[1]))
     per_round = max(1, COMPUTE_UNITS // heads)
     out = []
@@ -379,12 +383,33 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx
         cached = ctx.scratch.get(key)
         if cached is None:
             q_lens = [ctx.cu_q_host[b + 1] - ctx.cu_q_host[b] for b in range(ctx.num_seqs)]
-            rows, small = prefill_tiles(q_lens, ctx.ctx_lens_host, d, nq, nkv)
-            cached = (torch.tensor(rows, dtype=torch.int32, device=q.device).reshape(-1, 2), small)
+            # The sequences at the head of the batch that bring one token (the scheduler puts the
+            # decoding requests first) go to the decode kernel, which reads a kv head's keys once
+            # for all its query heads and splits a context over workgroups; the prefill kernel
+            # would give each of them a 16-row tile with one row in use.
+            # The two kernels run one after the other, so it pays only where the prefill kernel
+            # would have much to do for those sequences: keys times the times it reads them (once
+            # per group of query heads it takes together), or a long context for one workgroup to walk.
+            lead = 0
+            while lead < len(q_lens) and q_lens[lead] == 1:
+                lead += 1
+            lead_ctx = max(ctx.ctx_lens_host[:lead]) if lead else 0
+            reads = g // (4 if g % 4 == 0 else 2 if g % 2 == 0 else 1)
+            if (lead < MIXED_DECODE_FROM or not (g <= 16 and (4 * g * d + 8 * g) * 4 <= 64 * 1024)
+                    or not (lead * lead_ctx * reads >= MIXED_DECODE_WORK or lead_ctx >= MIXED_DECODE_CONTEXT)):
+                lead = 0
+            rows, small = prefill_tiles(q_lens, ctx.ctx_lens_host, d, nq, nkv, first_seq=lead)
+            cached = (torch.tensor(rows, dtype=torch.int32, device=q.device).reshape(-1, 2), small, lead,
+                      lead_ctx if lead else 0)
             ctx.scratch[key] = cached
-        tiles, small = cached
+        tiles, small, lead, lead_ctx = cached
+        out = None
+        if lead:
+            out = torch.empty((T, nq * d), dtype=q.dtype, device=q.device)
+            attention_decode_bf16(q[:lead], k_cache, v_cache, bt[:lead], ctx.ctx_lens[:lead], lead_ctx, scale, window,
+                                  out=out[:lead])
         return attention_prefill_bf16(q, k_cache, v_cache, bt, tiles, ctx.cu_q, ctx.ctx_lens, scale, window,
-                                      small=small)
+                                      out=out, small=small)
     return attention_generic(q, k_cache, v_cache, bt, ctx.tok_seq, ctx.positions, scale, window,
                              v_transposed=v_transposed)
 
