@@ -16,6 +16,9 @@ are random values (decode timing does not depend on what the cache holds).
 `--workload serve14b` and `--workload long32b` instead run the two serving workloads of the
 larger configurations through the whole engine (scheduler, chunked prefill, continuous
 batching, greedy sampling) and print their own JSON line: total generated tokens per second.
+`--workload many06b` is the one run the reference publishes a figure for (Qwen3-0.6B, 256
+concurrent requests, 1,024 new tokens each); its line carries the ratio to that figure, which
+was measured on other hardware.
 """
 from __future__ import annotations
 
@@ -37,8 +40,14 @@ QWEN3_14B = dict(QWEN3_8B, hidden_size=5120, intermediate_size=17408, num_hidden
                  num_attention_heads=40, num_key_value_heads=8)
 QWEN3_32B = dict(QWEN3_8B, hidden_size=5120, intermediate_size=25600, num_hidden_layers=64,
                  num_attention_heads=64, num_key_value_heads=8)
-# the serving workloads of the two larger configurations
+QWEN3_0_6B = dict(QWEN3_8B, hidden_size=1024, intermediate_size=3072, num_hidden_layers=28,
+                  num_attention_heads=16, num_key_value_heads=8, tie_word_embeddings=True)
+# the serving workloads of the two larger configurations, and the one the reference publishes a
+# figure for: Qwen3-0.6B, 256 concurrent requests of 16 prompt tokens, 1,024 new tokens each
+# (/root/reference/python/ReadMe.md:2-13: 10,944.62 generated tokens/s on a CUDA GPU)
 WORKLOADS = {
+    "many06b": dict(model=QWEN3_0_6B, name="Qwen3-0.6B layer sizes", requests=256, prompt=(16, 16), new_tokens=1024,
+                    chunk=2048, max_model_len=1088, reference_tok_s=10944.62),
     "serve14b": dict(model=QWEN3_14B, name="Qwen3-14B layer sizes", requests=64, prompt=(128, 2048), new_tokens=256,
                      chunk=2048, max_model_len=2304),
     "long32b": dict(model=QWEN3_32B, name="Qwen3-32B layer sizes", requests=16, prompt=(8192, 8192), new_tokens=512,
@@ -108,6 +117,7 @@ def serve(workload: str, layers) -> int:
     print(json.dumps({
         "metric": f"generated tok/s, {workload} workload, bf16", "value": round(new / dt, 1), "unit": "tokens/s",
         "n_gpus": 1, "seconds": round(dt, 3), "engine_steps": eng.steps - steps0, "higher_is_better": True,
+        "vs_reference_published": round(new / dt / w["reference_tok_s"], 2) if "reference_tok_s" in w else None,
         "dtype": "bf16", "data": "synthetic: seeded random weights, uniform random token ids",
         "config": {"model": w["name"], "layers": cfg.num_hidden_layers, "layers_of_model": full, "requests": n,
                    "prompt_tokens": sum(lens), "new_tokens": new, "prefill_chunk": w["chunk"],

@@ -19,6 +19,7 @@ import torch
 from ..config.engine_config import (EngineConfig, GenerationConfig, GenerationOutput, Message, SamplingParams,
                                     StreamItem)
 from ..sampling import Sampler, Strategy, resolve_strategy, uniform
+from ..sampling.sampler import PENALTY_CONTEXT
 from .loading import load_model, parse_dtype
 from .runner import ModelRunner, StepEntry
 from .scheduler import RequestTooLarge, Scheduler
@@ -161,22 +162,26 @@ class LLMEngine:
         self.steps += 1
         done: List[int] = []
         if sampled:
+            # (a request's generated tokens are tokens[prompt_len:]; no copies of them on this path)
+            strategies = [r.strategy for r in sampled]
+            recent = None
+            if any(s.frequency_penalty or s.presence_penalty for s in strategies):
+                recent = [r.tokens[max(r.prompt_len, len(r.tokens) - PENALTY_CONTEXT):] for r in sampled]
             tokens = self.sampler.sample(
-                logits, [r.strategy for r in sampled],
-                [uniform(r.seed, r.stream, len(r.generated)) for r in sampled],
-                recent=[r.generated for r in sampled])
+                logits, strategies, [uniform(r.seed, r.stream, len(r.tokens) - r.prompt_len) for r in sampled],
+                recent=recent)
             now = _now_ms()
             for r, tok in zip(sampled, tokens):
-                if not r.generated:
+                if len(r.tokens) == r.prompt_len:
                     r.decode_start = now
                 reason = ""
-                if _completes_a_stop(r.stops, r.generated, int(tok)):
+                if r.stops and _completes_a_stop(r.stops, r.generated, int(tok)):
                     reason = "stop"
                 elif tok in self.eos_token_ids and not r.params.ignore_eos:
                     reason = "eos"
                 else:
                     r.tokens.append(int(tok))
-                    if len(r.generated) >= r.max_tokens:
+                    if len(r.tokens) - r.prompt_len >= r.max_tokens:
                         reason = "length"
                     elif len(r.tokens) >= self.max_model_len:
                         reason = "max_model_len"

@@ -112,7 +112,7 @@ class _DecodeGraph:
 
 class ModelRunner:
     def __init__(self, model: CausalLM, page_size: int, num_pages, max_requests: int,
-                 use_graphs: bool = True, graph_max_batch: int = 64, graph_after: Optional[int] = None):
+                 use_graphs: bool = True, graph_max_batch: Optional[int] = None, graph_after: Optional[int] = None):
         """`num_pages`: pages of every group's pool, or a list with one count per group.
         `use_graphs`: record decode steps of up to `graph_max_batch` requests as HIP graphs; a
         (batch size, context bucket) is recorded the `graph_after`-th time it is seen, so that
@@ -121,7 +121,9 @@ class ModelRunner:
         graph's instantiation (12 to 25 ms at 8B to 32B sizes on an MI355X); a replay saves what
         the host's launches of a step take beyond the kernels' own time: everything for a small
         model, 0.1 to 0.2 ms a step for a large one, whose kernels outlast the launches.  Left to
-        the runner, the count is 3 for a model whose step is bound by the host and 12 otherwise."""
+        the runner, the count is 3 for a model whose step is bound by the host and 12 otherwise,
+        and `graph_max_batch` 256 for such a model (its launches cost more than its kernels at
+        any batch size) and 64 otherwise."""
         if not torch.cuda.is_available():
             raise RuntimeError("xinfer_amd runs on an AMD GPU only: no HIP device is visible")
         self.model = model
@@ -155,14 +157,16 @@ class ModelRunner:
         self._empty_f32 = torch.empty((1, 0), dtype=torch.float32, device=self.device)
         self._staging = _Staging(self.device)
         self.use_graphs = bool(use_graphs) and model.graph_safe
-        self.graph_max_batch = int(graph_max_batch)
+        # a step's kernels take about weights / 4 TB/s, its launches about 100 us a layer
+        size = 2 if model.dtype == torch.bfloat16 else 4
+        weights = size * sum(int(np.prod(d.shape)) for d in type(model).declare(model.spec))
+        host_bound = weights / 4e12 < 0.5 * max(1, len(model.spec.layers)) * 100e-6
         if graph_after is None:
-            # a step's kernels take about weights / 4 TB/s, its launches about 100 us a layer
-            size = 2 if model.dtype == torch.bfloat16 else 4
-            weights = size * sum(int(np.prod(d.shape)) for d in type(model).declare(model.spec))
-            layers = max(1, len(model.spec.layers))
-            graph_after = 3 if weights / 4e12 < 0.5 * layers * 100e-6 else 12
+            graph_after = 3 if host_bound else 12
+        if graph_max_batch is None:
+            graph_max_batch = 256 if host_bound else 64
         self.graph_after = max(1, int(graph_after))
+        self.graph_max_batch = int(graph_max_batch)
         self._graphs: Dict[Tuple[int, int, bool], _DecodeGraph] = {}
         self._seen: Dict[Tuple[int, int, bool], int] = {}
         self._graph_pool = None
