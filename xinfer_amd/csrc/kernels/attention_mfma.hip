@@ -221,7 +221,7 @@ __global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
       ll += lds_ml[(wv * g + h) * 2 + 1] * f;
     }
     if (max_splits == 1) {   // the only split of every sequence: the result itself
-      out[((size_t)seq * nq + kvh * g + h) * d + i] = __float2bfloat16(o / ll);
+      out[((size_t)seq * nq + kvh * g + h) * d + i] = __float2bfloat16(o * (1.f / ll));   // as the combine rounds
       continue;
     }
     const size_t pidx = ((size_t)seq * nq + kvh * g + h) * max_splits + split;
