@@ -278,14 +278,14 @@ def test_linear_thin_refuses():
 
 def test_linear_chooses_the_kernel_of_a_folded_product():
     """A product before a norm adds into the stream itself for up to 16 rows: with the thin kernel
-    where N is no multiple of 4096 or rows x K is large, else with the streaming kernel; more rows
-    come back as partial sums of the tiled kernel for the norm to add."""
+    where K is a multiple of 256, else with the streaming kernel; more rows come back as partial
+    sums of the tiled kernel for the norm to add."""
     from xinfer_amd import kernels
     from xinfer_amd.config.spec import PartSpec
     from xinfer_amd.parts.base import Folded, NormSink, norm_class
     from xinfer_amd.parts.linear import Linear
     g = torch.Generator().manual_seed(3)
-    for N, K in ((256, 8192), (4096, 2048)):
+    for N, K in ((256, 8192), (4096, 2048), (512, 1088)):
         lin = Linear(_rand((N, K), torch.bfloat16, g, 0.02).to(DEV))
         norm = norm_class("rmsnorm")(PartSpec("rmsnorm", dict(dim=N, eps=1e-6)), torch.bfloat16)
         norm.weight = torch.ones(N, device=DEV)
@@ -297,7 +297,7 @@ def test_linear_chooses_the_kernel_of_a_folded_product():
             if M <= kernels.FOLD_ROWS:
                 assert isinstance(y, Folded)
                 thin = kernels.thin_ahead(M, lin.weight)
-                assert thin == (N % 4096 != 0 or M * K >= kernels.THIN_WORK)
+                assert thin == (K % 256 == 0)
                 assert y.ss.shape[1] == (kernels.linear_thin_parts(N, K) if thin else kernels.linear_fold_parts(M, N, K))
                 assert (resid.cpu().double() - ref).abs().max() / ref.abs().max() < 1e-5
             else:

@@ -10,7 +10,9 @@
 // copy the w tile [32 rows, 512 bytes each: 32 lanes a row] and the x tile [16 rows] from
 // memory into registers, two tiles ahead, and from there into LDS (double buffered, one barrier
 // a tile); wave v multiplies k steps 2v and 2v+1 of the tile's eight (v_mfma_f32_16x16x32_bf16,
-// A = 16 rows of w, B = the 16 rows of x), two tiles of 16 features each.  At the end the four
+// A = 16 rows of w, B = the 16 rows of x), two tiles of 16 features each.  Workgroups of up to
+// 16 features take tiles of [16 rows, 512 k] instead: the same bytes a tile, no rows that
+// nobody multiplies, half the barriers.  At the end the four
 // waves' sums are added through LDS in wave order and stored: plain (MODE 0), adding into the
 // float32 residual stream and handing on round(stream * g) and the rows' sums of squares (MODE
 // 1), or scaling the rows by rsqrt(sum of the parts / K + eps) (MODE 2).
@@ -27,12 +29,13 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr int kThinRows = 16;            // rows of x
-constexpr int kThinFeatures = 32;        // rows of w in a workgroup's tile
-constexpr int kThinK = 256;              // k per tile
-constexpr int kThinLdsRow = kThinK + 8;  // elements of a row in LDS
+constexpr int kThinFeatures = 32;        // most rows of w in a workgroup's tile
+constexpr int kThinK = 256;              // k per tile of 32 rows of w (a tile of 16 rows takes 512: the same bytes)
 constexpr int kThinDepth = 2;            // tiles whose loads are in flight
 constexpr int kThinSsLoads = 32;         // 16 threads x 32 loads: up to 512 parts of a row's sum of squares
-constexpr int kThinStage = (kThinFeatures + kThinRows) * kThinLdsRow;   // elements of one buffer
+constexpr size_t thin_lds_bytes(int tr) {     // two buffers of a w tile and an x tile, rows padded by 8 elements
+  return 2 * (size_t)(tr + kThinRows) * (8192 / tr + 8) * sizeof(bf16);
+}
 
 struct ThinFold {
   float* resid;         // MODE 1: [M, N] float32, updated in place
@@ -45,19 +48,30 @@ struct ThinFold {
   float inv_h;          // MODE 2: 1 / length of the normed rows
 };
 
-template <int MODE, typename TO>
+// TR: rows of w in a tile, 32 or 16 (for workgroups of up to 16 features: no rows are copied
+// that nobody multiplies); a tile holds 8192 / TR of k.
+template <int MODE, typename TO, int TR>
 __global__ __launch_bounds__(256) void linear_thin_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
                                                           TO* __restrict__ y, int M, int N, int K, int R, int rotate,
                                                           ThinFold fold) {
   constexpr int D = kThinDepth;
-  __shared__ __align__(16) bf16 lds[2 * kThinStage];          // [buffer][w tile 32 rows | x tile 16 rows][kThinLdsRow]
-  __shared__ __align__(16) float red[4 * 2 * 256];            // [wave][feature tile][lane * 4 + i]
-  __shared__ float side[MODE == 1 ? kThinRows * kThinFeatures : kThinRows];   // squares [row][feature], or 1/rms [row]
+  constexpr int BK = 8192 / TR;              // k per tile
+  constexpr int LROW = BK + 8;               // elements of a row in LDS
+  constexpr int CPR = BK / 8;                // 16-byte chunks of a row
+  constexpr int RPP = 256 / CPR;             // rows the 256 threads copy at once
+  constexpr int WP = TR / RPP, XP = kThinRows / RPP;     // copies of a thread per tile of w, of x
+  constexpr int RT = TR / 16;                // 16-feature tiles
+  constexpr int SPW = BK / 32 / 4;           // 32-wide k steps of a tile that a wave multiplies
+  constexpr int STAGE = (TR + kThinRows) * LROW;         // elements of one buffer
+  extern __shared__ __align__(16) unsigned char thin_smem[];
+  bf16* lds = reinterpret_cast<bf16*>(thin_smem);        // [buffer][w tile TR rows | x tile 16 rows][LROW]
+  __shared__ __align__(16) float red[4 * RT * 256];      // [wave][feature tile][lane * 4 + i]
+  __shared__ float side[MODE == 1 ? kThinRows * TR : kThinRows];   // squares [row][feature], or 1/rms [row]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, j = lane >> 4;
   const int n0 = blockIdx.x * R;
   const int n_last = (n0 + R < N ? n0 + R : N) - 1;
-  const int nkt = K / kThinK;
+  const int nkt = K / BK;
   const int start = (int)(((long long)blockIdx.x * rotate) % nkt);
 
   // MODE 2: 16 threads per row add up the parts of its sum of squares; the loads start now
@@ -71,37 +85,37 @@ __global__ __launch_bounds__(256) void linear_thin_kernel(const bf16* __restrict
     }
   }
 
-  // ---- copying: a row of a tile is 32 16-byte chunks; thread t moves chunk t % 32 of rows
-  // t / 32 + 8 i of w (i < 4) and of x (i < 2).  Rows past the workgroup's last feature read
-  // that feature's row again, rows of x past M row M - 1; no load is conditional.
-  const int srow = tid >> 5, skc = tid & 31;
-  const bf16* wsrc[4];
-  const bf16* xsrc[2];
+  // ---- copying: a row of a tile is CPR 16-byte chunks; thread t moves chunk t % CPR of rows
+  // t / CPR + RPP i of w (i < WP) and of x (i < XP).  Rows past the workgroup's last feature
+  // read that feature's row again, rows of x past M row M - 1; no load is conditional.
+  const int srow = tid / CPR, skc = tid % CPR;
+  const bf16* wsrc[WP];
+  const bf16* xsrc[XP];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    int n = n0 + srow + 8 * i;
+  for (int i = 0; i < WP; ++i) {
+    int n = n0 + srow + RPP * i;
     n = n < n_last ? n : n_last;
     wsrc[i] = w + (size_t)n * K + 8 * skc;
   }
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int row = srow + 8 * i;
+  for (int i = 0; i < XP; ++i) {
+    const int row = srow + RPP * i;
     xsrc[i] = x + (size_t)(row < M ? row : M - 1) * K + 8 * skc;
   }
-  const int sdst = srow * kThinLdsRow + 8 * skc;
-  bf16x8 wr[D][4], xr[D][2];
-  f32x4 acc[2];
-  acc[0] = f32x4{0.f, 0.f, 0.f, 0.f};
-  acc[1] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int sdst = srow * LROW + 8 * skc;
+  bf16x8 wr[D][WP], xr[D][XP];
+  f32x4 acc[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
 #define XI_THIN_ISSUE(slot, t)                                                           \
   do {                                                                                   \
     int tt_ = (t) + start;                                                               \
     tt_ = tt_ >= nkt ? tt_ - nkt : tt_;                                                  \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                        \
-      wr[slot][i] = *reinterpret_cast<const bf16x8*>(wsrc[i] + (size_t)tt_ * kThinK);    \
-    _Pragma("unroll") for (int i = 0; i < 2; ++i)                                        \
-      xr[slot][i] = *reinterpret_cast<const bf16x8*>(xsrc[i] + (size_t)tt_ * kThinK);    \
+    _Pragma("unroll") for (int i = 0; i < WP; ++i)                                       \
+      wr[slot][i] = *reinterpret_cast<const bf16x8*>(wsrc[i] + (size_t)tt_ * BK);        \
+    _Pragma("unroll") for (int i = 0; i < XP; ++i)                                       \
+      xr[slot][i] = *reinterpret_cast<const bf16x8*>(xsrc[i] + (size_t)tt_ * BK);        \
   } while (0)
 
   // every copy is issued whether or not its tile exists (past the end the last tile is read
@@ -113,21 +127,21 @@ __global__ __launch_bounds__(256) void linear_thin_kernel(const bf16* __restrict
   int buf = 0;
 #define XI_THIN_TILE(s, t)                                                                                \
   do {                                                                                                    \
-    bf16* Ws = lds + buf * kThinStage;                                                                    \
-    bf16* Xs = Ws + kThinFeatures * kThinLdsRow;                                                          \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                         \
-      *reinterpret_cast<bf16x8*>(Ws + sdst + 8 * i * kThinLdsRow) = wr[s][i];                             \
-    _Pragma("unroll") for (int i = 0; i < 2; ++i)                                                         \
-      *reinterpret_cast<bf16x8*>(Xs + sdst + 8 * i * kThinLdsRow) = xr[s][i];                             \
+    bf16* Ws = lds + buf * STAGE;                                                                         \
+    bf16* Xs = Ws + TR * LROW;                                                                            \
+    _Pragma("unroll") for (int i = 0; i < WP; ++i)                                                        \
+      *reinterpret_cast<bf16x8*>(Ws + sdst + RPP * i * LROW) = wr[s][i];                                  \
+    _Pragma("unroll") for (int i = 0; i < XP; ++i)                                                        \
+      *reinterpret_cast<bf16x8*>(Xs + sdst + RPP * i * LROW) = xr[s][i];                                  \
     XI_THIN_ISSUE(s, (t) + D < last ? (t) + D : last);                                                    \
     __syncthreads();                                                                                      \
-    _Pragma("unroll") for (int kk = 0; kk < 2; ++kk) {                                                    \
-      const int col = 32 * (2 * wave + kk) + 8 * j;                                                       \
-      const bf16x8 b = *reinterpret_cast<const bf16x8*>(Xs + r * kThinLdsRow + col);                      \
-      const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(Ws + r * kThinLdsRow + col);                     \
-      const bf16x8 a1 = *reinterpret_cast<const bf16x8*>(Ws + (16 + r) * kThinLdsRow + col);              \
-      acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b, acc[0], 0, 0, 0);                           \
-      acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b, acc[1], 0, 0, 0);                           \
+    _Pragma("unroll") for (int kk = 0; kk < SPW; ++kk) {                                                  \
+      const int col = 32 * (SPW * wave + kk) + 8 * j;                                                     \
+      const bf16x8 b = *reinterpret_cast<const bf16x8*>(Xs + r * LROW + col);                             \
+      _Pragma("unroll") for (int t_ = 0; t_ < RT; ++t_) {                                                 \
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(Ws + (16 * t_ + r) * LROW + col);               \
+        acc[t_] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t_], 0, 0, 0);                        \
+      }                                                                                                   \
     }                                                                                                     \
     buf ^= 1;                                                                                             \
   } while (0)
@@ -147,8 +161,8 @@ __global__ __launch_bounds__(256) void linear_thin_kernel(const bf16* __restrict
 
   // ---- the four waves' sums through LDS, added in wave order.  A lane's 4 values of a tile:
   // row r of x, features 4 j .. 4 j + 3 of the tile.
-  *reinterpret_cast<f32x4*>(&red[(wave * 2 + 0) * 256 + lane * 4]) = acc[0];
-  *reinterpret_cast<f32x4*>(&red[(wave * 2 + 1) * 256 + lane * 4]) = acc[1];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) *reinterpret_cast<f32x4*>(&red[(wave * RT + t) * 256 + lane * 4]) = acc[t];
   if constexpr (MODE == 2) {
     float t = 0.f;
 #pragma unroll
@@ -159,14 +173,14 @@ __global__ __launch_bounds__(256) void linear_thin_kernel(const bf16* __restrict
   }
   __syncthreads();
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
+  for (int h = 0; h < RT; ++h) {
     const int e = tid;                       // element of feature tile h
     const int ln = e >> 2, v = e & 3;
     const int token = ln & 15, f = 16 * h + 4 * (ln >> 4) + v;      // feature within the workgroup's tile
     const int n = n0 + f;
     float a = 0.f;
 #pragma unroll
-    for (int wv = 0; wv < 4; ++wv) a += red[(wv * 2 + h) * 256 + e];
+    for (int wv = 0; wv < 4; ++wv) a += red[(wv * RT + h) * 256 + e];
     const bool mine = n <= n_last && token < M;
     if constexpr (MODE == 1) {
       float sq = 0.f;
@@ -176,7 +190,7 @@ __global__ __launch_bounds__(256) void linear_thin_kernel(const bf16* __restrict
         fold.xg[(size_t)token * N + n] = from_float<bf16>(rr * fold.g[n]);
         sq = rr * rr;
       }
-      side[token * kThinFeatures + f] = sq;
+      side[token * TR + f] = sq;
     } else {
       if constexpr (MODE == 2) a *= side[token];
       if (mine) y[(size_t)token * N + n] = from_float<TO>(a);
@@ -186,7 +200,7 @@ __global__ __launch_bounds__(256) void linear_thin_kernel(const bf16* __restrict
     __syncthreads();
     if (tid < kThinRows && tid < M) {
       float t = 0.f;
-      for (int i = 0; i < kThinFeatures; ++i) t += side[tid * kThinFeatures + i];
+      for (int i = 0; i < TR; ++i) t += side[tid * TR + i];
       fold.ss_out[(size_t)tid * gridDim.x + blockIdx.x] = t;
     }
   }
@@ -228,6 +242,28 @@ static int thin_check(const char* what, const void* x, const void* w, int M, int
   return 0;
 }
 
+// A tile of 16 rows of w where the workgroups own at most 16 features and K is a multiple of 512.
+static int thin_tile_rows(int R, int K) { return (R <= 16 && K % 512 == 0) ? 16 : 32; }
+
+#define XI_THIN_LAUNCH(MODE, TO, TR, yptr)                                                                      \
+  do {                                                                                                          \
+    static bool lds_set = false;                                                                                \
+    if (!lds_set) {                                                                                             \
+      hipError_t e = hipFuncSetAttribute((const void*)linear_thin_kernel<MODE, TO, TR>,                         \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)thin_lds_bytes(TR));  \
+      XI_CHECK(e == hipSuccess, "linear_thin: cannot get %zu bytes of LDS: %s", thin_lds_bytes(TR),             \
+               hipGetErrorString(e));                                                                           \
+      lds_set = true;                                                                                           \
+    }                                                                                                           \
+    linear_thin_kernel<MODE, TO, TR><<<wgs, 256, thin_lds_bytes(TR), stream>>>((const bf16*)x, (const bf16*)w,   \
+                                                                               (TO*)(yptr), M, N, K, R, rotate, fold); \
+  } while (0)
+#define XI_THIN_TILE_ROWS(MODE, TO, yptr)                   \
+  do {                                                      \
+    if (thin_tile_rows(R, K) == 16) XI_THIN_LAUNCH(MODE, TO, 16, yptr); \
+    else XI_THIN_LAUNCH(MODE, TO, 32, yptr);                \
+  } while (0)
+
 // y [M, N] bfloat16 (out_dtype 1) or float32 (0).
 int xi_linear_thin(const void* x, const void* w, void* y, int M, int N, int K, int out_dtype, int rotate,
                    hipStream_t stream) {
@@ -235,13 +271,10 @@ int xi_linear_thin(const void* x, const void* w, void* y, int M, int N, int K, i
   XI_CHECK(rotate >= 0, "linear_thin: rotate=%d", rotate);
   const int R = thin_features(N);
   const unsigned wgs = (unsigned)((N + R - 1) / R);
-  const ThinFold none{nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0.f, 0.f};
-  if (out_dtype == kBF16)
-    linear_thin_kernel<0, bf16><<<wgs, 256, 0, stream>>>((const bf16*)x, (const bf16*)w, (bf16*)y, M, N, K, R, rotate, none);
-  else if (out_dtype == kF32)
-    linear_thin_kernel<0, float><<<wgs, 256, 0, stream>>>((const bf16*)x, (const bf16*)w, (float*)y, M, N, K, R, rotate, none);
-  else
-    XI_CHECK(false, "linear_thin: unknown dtype %d", out_dtype);
+  const ThinFold fold{nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0.f, 0.f};
+  if (out_dtype == kBF16) XI_THIN_TILE_ROWS(0, bf16, y);
+  else if (out_dtype == kF32) XI_THIN_TILE_ROWS(0, float, y);
+  else XI_CHECK(false, "linear_thin: unknown dtype %d", out_dtype);
   XI_LAUNCH_CHECK("linear_thin");
   return 0;
 }
@@ -254,28 +287,27 @@ int xi_linear_thin_fold_out(const void* x, const void* w, int M, int N, int K, f
   const int R = thin_features(N);
   const unsigned wgs = (unsigned)((N + R - 1) / R);
   const ThinFold fold{resid, g, (bf16*)xg, ss, nullptr, 0, 0.f, 0.f};
-  linear_thin_kernel<1, bf16><<<wgs, 256, 0, stream>>>((const bf16*)x, (const bf16*)w, (bf16*)nullptr, M, N, K, R, rotate, fold);
+  XI_THIN_TILE_ROWS(1, bf16, nullptr);
   XI_LAUNCH_CHECK("linear_thin_fold_out");
   return 0;
 }
 
 // y [M, N] = (xg @ w^T) with row t scaled by rsqrt(sum(ss[t]) / K + eps); ss [M, parts], parts <= 512.
-int xi_linear_thin_fold_in(const void* xg, const void* w, void* y, int M, int N, int K, int out_dtype, const float* ss,
+int xi_linear_thin_fold_in(const void* x, const void* w, void* y, int M, int N, int K, int out_dtype, const float* ss,
                            int parts, float eps, int rotate, hipStream_t stream) {
-  if (thin_check("linear_thin_fold_in", xg, w, M, N, K)) return 1;
+  if (thin_check("linear_thin_fold_in", x, w, M, N, K)) return 1;
   XI_CHECK(ss && parts >= 1 && parts <= 16 * kThinSsLoads && rotate >= 0, "linear_thin_fold_in: %d parts (1..%d)", parts,
            16 * kThinSsLoads);
   const int R = thin_features(N);
   const unsigned wgs = (unsigned)((N + R - 1) / R);
   const ThinFold fold{nullptr, nullptr, nullptr, nullptr, ss, parts, eps, 1.f / (float)K};
-  if (out_dtype == kBF16)
-    linear_thin_kernel<2, bf16><<<wgs, 256, 0, stream>>>((const bf16*)xg, (const bf16*)w, (bf16*)y, M, N, K, R, rotate, fold);
-  else if (out_dtype == kF32)
-    linear_thin_kernel<2, float><<<wgs, 256, 0, stream>>>((const bf16*)xg, (const bf16*)w, (float*)y, M, N, K, R, rotate, fold);
-  else
-    XI_CHECK(false, "linear_thin_fold_in: unknown dtype %d", out_dtype);
+  if (out_dtype == kBF16) XI_THIN_TILE_ROWS(2, bf16, y);
+  else if (out_dtype == kF32) XI_THIN_TILE_ROWS(2, float, y);
+  else XI_CHECK(false, "linear_thin_fold_in: unknown dtype %d", out_dtype);
   XI_LAUNCH_CHECK("linear_thin_fold_in");
   return 0;
 }
+#undef XI_THIN_TILE_ROWS
+#undef XI_THIN_LAUNCH
 
 }  // extern "C"

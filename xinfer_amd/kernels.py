@@ -619,18 +619,13 @@ THIN_ROTATE = 0           # workgroup b of the thin product starts b * this many
                           # here it measured no gain: 0)
 
 
-THIN_WORK = 96_000        # rows x K from which the thin product is ahead of the streaming kernel where that
-                          # kernel's workgroups own whole tiles of 16 features (N a multiple of 4096); where they
-                          # do not (N = 5120: 20 features, 6144: 24) the thin product is ahead from the first row.
-                          # Measured in decode steps at Qwen3-8B, 14B and 32B sizes (3% of a step at the larger two).
-
-
 def thin_ahead(M: int, w: torch.Tensor) -> bool:
-    """Whether a product of M <= FOLD_ROWS rows with whole sums goes to the thin kernel."""
+    """Whether a product of M <= FOLD_ROWS rows with whole sums goes to the thin kernel: wherever it
+    takes the sizes (K a multiple of 256).  Measured in decode steps at Qwen3-8B, 14B and 32B sizes
+    against the streaming kernel: level at one row, 1 to 3% of a step ahead from two rows on."""
     if w.dtype != torch.bfloat16 or not (0 < M <= FOLD_ROWS):
         return False
-    parts = linear_thin_parts(w.shape[0], w.shape[1])
-    return 0 < parts <= FOLD_PARTS and (w.shape[0] % 4096 != 0 or M * w.shape[1] >= THIN_WORK)
+    return 0 < linear_thin_parts(w.shape[0], w.shape[1]) <= FOLD_PARTS
 
 
 def linear_thin_parts(N: int, K: int) -> int:
