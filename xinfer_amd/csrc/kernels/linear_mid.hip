@@ -344,7 +344,7 @@ int xi_linear_mid(const void* x, const void* w, float* y, int M, int N, int K, i
 // ss (or null): x is the first half of a folded RMSNorm, ss [M, parts] float32 the parts of its
 // rows' sums of squares (M <= 16, parts <= 512): rows are scaled by rsqrt(sum / K + eps).
 int xi_linear_mid_gated(const void* x, const void* w, void* y, int M, int N, int K, const float* ss, int parts,
-                        float eps, int rotate, hipStream_t stream) {
+                        float eps, int rotate, int features, hipStream_t stream) {
   XI_CHECK(M >= 1 && M <= kMidRows, "linear_mid_gated: M=%d must be 1..%d", M, kMidRows);
   XI_CHECK(N >= 1 && K >= kMidK && K % kMidK == 0, "linear_mid_gated: N=%d, K=%d (a multiple of %d) are not taken", N,
            K, kMidK);
@@ -352,7 +352,7 @@ int xi_linear_mid_gated(const void* x, const void* w, void* y, int M, int N, int
   XI_CHECK(rotate >= 0, "linear_mid_gated: rotate=%d", rotate);
   XI_CHECK(ss == nullptr || (M <= 16 && parts >= 1 && parts <= 16 * kMidSsLoads),
            "linear_mid_gated: a folded norm takes up to 16 rows and %d parts (M=%d, parts=%d)", 16 * kMidSsLoads, M, parts);
-  const int R = mid_gated_features(N);
+  const int R = features > 0 ? features : mid_gated_features(N);     // features: an override, for measurements
   const long long wgs = (N + R - 1) / R;
   XI_CHECK(R >= 1 && R <= 64 && wgs < (1ll << 31), "linear_mid_gated: %d features per workgroup", R);
   const MidFold fold{ss, parts, eps, 1.f / (float)K};

@@ -511,9 +511,10 @@ def linear_mid(x: torch.Tensor, w: torch.Tensor, depth: int = 0) -> torch.Tensor
 
 
 MID_GATED_ROWS = 128      # most rows of the gated form of the tiled product
+MID_GATED_FEATURES = 0    # features a workgroup of it owns; 0: chosen from N (the fewest workgroups that are a multiple of 256)
 MID_GATED_UP_TO = 64      # it is used up to this many rows (more: its reads of x from L2 outweigh the library's
                           # weakness); measured on MI355X at the gate/up sizes of Qwen3-8B, 14B and 32B, it is
-MID_GATED_FROM = 6        # ahead of the streaming kernel from this many rows on, and from the first row where
+MID_GATED_FROM = 2        # ahead of the streaming kernel from this many rows on, and from the first row where
 MID_GATED_BIG = 300 << 20  # the weight has this many bytes (the streaming kernel falls behind on large weights)
 
 
@@ -547,7 +548,7 @@ def linear_mid_gated(x: torch.Tensor, w: torch.Tensor, ss: Optional[torch.Tensor
         parts = int(ss.shape[1])
     y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
     _ok(lib().xi_linear_mid_gated(_p(x), _p(w), _p(y), M, N, K, _p(ss), parts, ctypes.c_float(eps), int(MID_GATED_ROTATE),
-                                  _stream()))
+                                  int(MID_GATED_FEATURES), _stream()))
     return y
 
 
