@@ -164,3 +164,45 @@ def test_real_layer_sizes_wide_decode_batches(name, live, real_model_dirs):
         harness.compare(again, ref, harness.TOL["bfloat16"], f"{name}/bfloat16/decode batch of {live}, launched")
         scale = max(float(r.abs().max()) for r in ref.values())
         assert max(float((got[k] - again[k]).abs().max()) for k in got) < 2e-3 * scale
+
+
+def test_mixed_step_with_long_contexts_both_attention_paths(real_model_dirs):
+    """A step that brings single tokens of six requests with contexts of some thousand tokens and a
+    portion of a seventh, at Qwen3-8B layer sizes: the decode kernel takes the six (their contexts
+    are long), the prefill kernel the portion; with the rule switched off the prefill kernel takes
+    all.  The two agree to rounding, and a request alone gives the same logits as in the batch."""
+    from xinfer_amd import kernels
+    from xinfer_amd.engine import ModelRunner, StepEntry, load_model
+    t = REAL["8B"]
+    vocab, page = t["config"]["vocab_size"], t["page_size"]
+    model = load_model(real_model_dirs("8B"), "bfloat16", "cuda:0")
+    rng = random.Random(21)
+    lens = [900, 1000, 700, 1003, 960, 1010]         # the model's 1,024 positions bound the contexts
+    prompts = [harness.random_prompt(rng, n, vocab) for n in lens]
+    portion = harness.random_prompt(rng, 300, vocab)
+    nxt = [rng.randrange(vocab) for _ in lens]
+
+    def run(switch_off):
+        old = kernels.MIXED_DECODE_CONTEXT, kernels.MIXED_DECODE_WORK
+        runner = ModelRunner(model, page_size=page, num_pages=8 * 16 + 8, max_requests=8, use_graphs=False)
+        try:
+            kernels.MIXED_DECODE_CONTEXT, kernels.MIXED_DECODE_WORK = (1 << 30, 1 << 60) if switch_off else (512, 1 << 60)
+            for i, p in enumerate(prompts):
+                runner.add_request(i)
+                runner.step([StepEntry(i, p, [])])
+            runner.add_request(7)
+            entries = [StepEntry(i, [tok], [0]) for i, tok in enumerate(nxt)] + [StepEntry(7, portion, [0, 299])]
+            return runner.step(entries).float().cpu()
+        finally:
+            kernels.MIXED_DECODE_CONTEXT, kernels.MIXED_DECODE_WORK = old
+
+    split, together = run(False), run(True)
+    scale = float(together.abs().max())
+    assert float((split - together).abs().max()) < harness.TOL["bfloat16"] * scale
+    assert not torch.equal(split[:6], together[:6])          # another kernel did run
+    # the first request alone, decoded by the decode kernel as a batch of one
+    runner = ModelRunner(model, page_size=page, num_pages=24, max_requests=2, use_graphs=False)
+    runner.add_request(0)
+    runner.step([StepEntry(0, prompts[0], [])])
+    alone = runner.step([StepEntry(0, [nxt[0]], [0])]).float().cpu()
+    assert float((alone[0] - split[0]).abs().max()) < harness.TOL["bfloat16"] * scale
