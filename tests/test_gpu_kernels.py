@@ -226,7 +226,7 @@ def test_linear_folded_norm(M, N, K, N2):
     assert y32.dtype == torch.float32 and (y32.cpu().double() - ref).abs().max() / ref.abs().max() < 2.0 ** -6
 
 
-@pytest.mark.parametrize("M", [1, 5, 16])
+@pytest.mark.parametrize("M", [1, 3, 4, 5, 8, 9, 16])
 @pytest.mark.parametrize("N,K,N2", [(64, 256, 96), (300, 512, 70), (4096, 1024, 130), (1000, 2304, 64)])
 def test_linear_thin_and_its_folded_norm(M, N, K, N2):
     """The thin product (few features a workgroup, whole sums, whole lines through LDS) in its

@@ -7,7 +7,7 @@
 //
 // A workgroup of four waves owns R <= 32 features (R from N alone, so that the workgroups are a
 // multiple of the 256 compute units) and all of K.  It walks K in tiles of 256: all 256 threads
-// copy the w tile [32 rows, 512 bytes each: 32 lanes a row] and the x tile [16 rows] from
+// copy the w tile [32 rows, 512 bytes each: 32 lanes a row] and the x tile [4, 8 or 16 rows] from
 // memory into registers, two tiles ahead, and from there into LDS (double buffered, one barrier
 // a tile); wave v multiplies k steps 2v and 2v+1 of the tile's eight (v_mfma_f32_16x16x32_bf16,
 // A = 16 rows of w, B = the 16 rows of x), two tiles of 16 features each.  Workgroups of up to
@@ -49,8 +49,11 @@ struct ThinFold {
 };
 
 // TR: rows of w in a tile, 32 or 16 (for workgroups of up to 16 features: no rows are copied
-// that nobody multiplies); a tile holds 8192 / TR of k.
-template <int MODE, typename TO, int TR>
+// that nobody multiplies); a tile holds 8192 / TR of k.  XR: rows of x in a tile, the power of
+// two from M up that the copying takes (a workgroup reads all of x, as many bytes per row as of
+// a row of w, so rows that are not there cost as much as features); the product's rows past XR
+// repeat earlier ones and are dropped.
+template <int MODE, typename TO, int TR, int XR>
 __global__ __launch_bounds__(256) void linear_thin_kernel(const bf16* __restrict__ x, const bf16* __restrict__ w,
                                                           TO* __restrict__ y, int M, int N, int K, int R, int rotate,
                                                           ThinFold fold) {
@@ -59,10 +62,11 @@ __global__ __launch_bounds__(256) void linear_thin_kernel(const bf16* __restrict
   constexpr int LROW = BK + 8;               // elements of a row in LDS
   constexpr int CPR = BK / 8;                // 16-byte chunks of a row
   constexpr int RPP = 256 / CPR;             // rows the 256 threads copy at once
-  constexpr int WP = TR / RPP, XP = kThinRows / RPP;     // copies of a thread per tile of w, of x
+  constexpr int WP = TR / RPP, XP = XR / RPP;
+  static_assert(XR % RPP == 0 && XP >= 1, "rows of x in a tile");     // copies of a thread per tile of w, of x
   constexpr int RT = TR / 16;                // 16-feature tiles
   constexpr int SPW = BK / 32 / 4;           // 32-wide k steps of a tile that a wave multiplies
-  constexpr int STAGE = (TR + kThinRows) * LROW;         // elements of one buffer
+  constexpr int STAGE = (TR + XR) * LROW;         // elements of one buffer
   extern __shared__ __align__(16) unsigned char thin_smem[];
   bf16* lds = reinterpret_cast<bf16*>(thin_smem);        // [buffer][w tile TR rows | x tile 16 rows][LROW]
   __shared__ __align__(16) float red[4 * RT * 256];      // [wave][feature tile][lane * 4 + i]
@@ -137,7 +141,7 @@ __global__ __launch_bounds__(256) void linear_thin_kernel(const bf16* __restrict
     __syncthreads();                                                                                      \
     _Pragma("unroll") for (int kk = 0; kk < SPW; ++kk) {                                                  \
       const int col = 32 * (SPW * wave + kk) + 8 * j;                                                     \
-      const bf16x8 b = *reinterpret_cast<const bf16x8*>(Xs + r * LROW + col);                             \
+      const bf16x8 b = *reinterpret_cast<const bf16x8*>(Xs + (r & (XR - 1)) * LROW + col);                             \
       _Pragma("unroll") for (int t_ = 0; t_ < RT; ++t_) {                                                 \
         const bf16x8 a = *reinterpret_cast<const bf16x8*>(Ws + (16 * t_ + r) * LROW + col);               \
         acc[t_] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[t_], 0, 0, 0);                        \
@@ -245,18 +249,25 @@ static int thin_check(const char* what, const void* x, const void* w, int M, int
 // A tile of 16 rows of w where the workgroups own at most 16 features and K is a multiple of 512.
 static int thin_tile_rows(int R, int K) { return (R <= 16 && K % 512 == 0) ? 16 : 32; }
 
-#define XI_THIN_LAUNCH(MODE, TO, TR, yptr)                                                                      \
+#define XI_THIN_LAUNCH_(MODE, TO, TR, XR, yptr)                                                                      \
   do {                                                                                                          \
     static bool lds_set = false;                                                                                \
     if (!lds_set) {                                                                                             \
-      hipError_t e = hipFuncSetAttribute((const void*)linear_thin_kernel<MODE, TO, TR>,                         \
+      hipError_t e = hipFuncSetAttribute((const void*)linear_thin_kernel<MODE, TO, TR, XR>,                         \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)thin_lds_bytes(TR));  \
       XI_CHECK(e == hipSuccess, "linear_thin: cannot get %zu bytes of LDS: %s", thin_lds_bytes(TR),             \
                hipGetErrorString(e));                                                                           \
       lds_set = true;                                                                                           \
     }                                                                                                           \
-    linear_thin_kernel<MODE, TO, TR><<<wgs, 256, thin_lds_bytes(TR), stream>>>((const bf16*)x, (const bf16*)w,   \
-                                                                               (TO*)(yptr), M, N, K, R, rotate, fold); \
+    linear_thin_kernel<MODE, TO, TR, XR><<<wgs, 256, thin_lds_bytes(TR), stream>>>(                             \
+        (const bf16*)x, (const bf16*)w, (TO*)(yptr), M, N, K, R, rotate, fold);                                 \
+  } while (0)
+// rows of x in a tile: 4 (tiles of 16 rows of w only: their copying takes 4 rows at once), 8 or 16
+#define XI_THIN_LAUNCH(MODE, TO, TR, yptr)                                    \
+  do {                                                                        \
+    if (M <= 4 && TR == 16) XI_THIN_LAUNCH_(MODE, TO, 16, 4, yptr);           \
+    else if (M <= 8) XI_THIN_LAUNCH_(MODE, TO, TR, 8, yptr);                  \
+    else XI_THIN_LAUNCH_(MODE, TO, TR, 16, yptr);                             \
   } while (0)
 #define XI_THIN_TILE_ROWS(MODE, TO, yptr)                   \
   do {                                                      \
@@ -309,5 +320,6 @@ int xi_linear_thin_fold_in(const void* x, const void* w, void* y, int M, int N, 
 }
 #undef XI_THIN_TILE_ROWS
 #undef XI_THIN_LAUNCH
+#undef XI_THIN_LAUNCH_
 
 }  // extern "C"
