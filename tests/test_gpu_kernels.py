@@ -814,6 +814,50 @@ def test_attention_decode_mfma(nq, nkv, d, page, window, seqs):
     assert err < _tol(torch.bfloat16, 2), err
 
 
+@pytest.mark.parametrize("nq,nkv,d,page,window,seqs,kpw", [
+    (8, 2, 128, 64, 0, [(7000, 1), (300, 1), (3201, 1)], 256),          # 28 splits, 2 and 13
+    (4, 4, 48, 16, 0, [(3300, 1)], 128),                                # 26 splits, a head size of 48
+    (2, 1, 256, 16, 0, [(6000, 1), (1, 1)], 128),                       # 47 splits and one
+    (6, 2, 64, 32, 4000, [(7000, 1), (3999, 1)], 128),                  # a window over 32 splits
+])
+def test_attention_decode_many_splits(nq, nkv, d, page, window, seqs, kpw):
+    """More than 24 splits go to the sixteen-wave combine kernel: against the plain attention, and
+    with one far key made to win the softmax, whose value row must come back."""
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(29)
+    case = _paged_case(g, torch.bfloat16, nq, nkv, d, page, seqs)
+    scale = 1.0 / math.sqrt(d)
+    q, kc, vt, bt = _mfma_inputs(case)
+    _, ctx = _cu_ctx(seqs)
+    longest = int(ctx.max())
+    assert (min(longest, window + 31) if window else longest) // kpw + 1 > 24
+    ref = _attention_ref(case, seqs, window, scale)
+    out = kernels.attention_decode_bf16(q, kc, vt, bt, ctx.to(DEV), longest, scale, window, keys_per_workgroup=kpw)
+    err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
+    assert err < _tol(torch.bfloat16, 2), err
+    far = longest - 1 - (window // 2 if window else longest // 3)       # a key in the middle of the splits
+    qv = case["qs"][0]
+    gsz = nq // nkv
+    for kvh in range(nkv):
+        kfar = (qv[0, kvh * gsz].float() / qv[0, kvh * gsz].float().norm() * 80).to(torch.bfloat16)
+        case["ks"][0][far, kvh] = kfar
+        case["kc"][int(case["bt"][0, far // page]), kvh, far % page] = kfar
+    ref = _attention_ref(case, seqs, window, scale)
+    assert (ref[0, :d] - case["vs"][0][far, 0].double()).abs().max() < 0.05
+    q, kc, vt, bt = _mfma_inputs(case)
+    out = kernels.attention_decode_bf16(q, kc, vt, bt, ctx.to(DEV), longest, scale, window, keys_per_workgroup=kpw)
+    assert (out.cpu().double() - ref).abs().max() / ref.abs().max() < _tol(torch.bfloat16, 2)
+
+
+def test_decode_keys_per_workgroup_grow_with_the_work():
+    from xinfer_amd import kernels
+    assert kernels.decode_keys_per_workgroup(64, 4096) == 256
+    assert kernels.decode_keys_per_workgroup(8, 131072) == 512
+    assert kernels.decode_keys_per_workgroup(32, 65536) == 1024
+    assert kernels.decode_keys_per_workgroup(128, 32768) == 2048
+    assert kernels.decode_keys_per_workgroup(1024, 1 << 20) == 2048
+
+
 @pytest.mark.parametrize("window", [0, 100])
 def test_attention_decode_one_split_per_sequence(window):
     """Many sequences of about the same length: a workgroup takes a whole sequence and writes the

@@ -294,6 +294,78 @@ __global__ __launch_bounds__(64) void attn_decode_combine_kernel(
   }
 }
 
+// The same for many splits (a long context of few sequences: 513 splits at 131,072 keys), where
+// one wave's walk over the splits takes longer than the attention itself: sixteen waves per
+// (head, sequence).  All threads share out the splits for the common maximum and the weights;
+// wave w then sums splits [w c, (w + 1) c), c = ceil(splits / 16), in split order, four splits
+// of loads in flight, and the sixteen sums are added in wave order.  The order depends on the
+// number of splits alone.
+constexpr int kWideWaves = 16;
+constexpr int kCombineWideFrom = 24;           // launches with more splits than this take the wide kernel
+__global__ __launch_bounds__(64 * kWideWaves) void attn_decode_combine_wide_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, const int* __restrict__ ctx_lens,
+    bf16* __restrict__ out, int max_splits, int window, int nq, int d, int keys_per_wg) {
+  extern __shared__ float f_s[];                 // [max_splits] weights | [16][d] sums of the waves | [16] | [16]
+  float* o_w = f_s + max_splits;
+  float* red_m = o_w + kWideWaves * d;
+  float* red_l = red_m + kWideWaves;
+  const int head = blockIdx.x, seq = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const size_t base = ((size_t)seq * nq + head) * max_splits;
+  const float* po = part_o + base * d;
+  const int pos = ctx_lens[seq] - 1;
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int n_splits = (pos - (lo & ~31)) / keys_per_wg + 1;
+  float mm = -INFINITY;
+  for (int s = tid; s < n_splits; s += 64 * kWideWaves) mm = fmaxf(mm, part_ml[(base + s) * 2]);
+  mm = wave_max(mm);
+  if (lane == 0) red_m[wave] = mm;
+  __syncthreads();
+  mm = red_m[0];
+#pragma unroll
+  for (int w = 1; w < kWideWaves; ++w) mm = fmaxf(mm, red_m[w]);
+  float ll = 0.f;
+  for (int s = tid; s < n_splits; s += 64 * kWideWaves) {
+    const float2 ml = *reinterpret_cast<const float2*>(part_ml + (base + s) * 2);
+    const float f = __builtin_amdgcn_exp2f(ml.x - mm);
+    f_s[s] = f;
+    ll += ml.y * f;
+  }
+  ll = wave_sum(ll);
+  if (lane == 0) red_l[wave] = ll;
+  __syncthreads();
+  ll = 0.f;
+#pragma unroll
+  for (int w = 0; w < kWideWaves; ++w) ll += red_l[w];
+  const int chunk = (n_splits + kWideWaves - 1) / kWideWaves;
+  const int s0 = wave * chunk, s1 = min(s0 + chunk, n_splits);
+  float o[4] = {0.f, 0.f, 0.f, 0.f};             // output dims lane + 64 c (head sizes up to 256)
+  for (int s = s0; s < s1; s += 4) {
+    float a[4][4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        a[u][c] = (s + u < s1 && lane + 64 * c < d) ? po[(size_t)(s + u) * d + lane + 64 * c] : 0.f;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float f = s + u < s1 ? f_s[s + u] : 0.f;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) o[c] += a[u][c] * f;
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c)
+    if (lane + 64 * c < d) o_w[wave * d + lane + 64 * c] = o[c];
+  __syncthreads();
+  const float inv = 1.f / ll;
+  for (int i = tid; i < d; i += 64 * kWideWaves) {
+    float t = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWideWaves; ++w) t += o_w[w * d + i];
+    out[((size_t)seq * nq + head) * d + i] = __float2bfloat16(t * inv);
+  }
+}
+
 }  // namespace xi
 
 using namespace xi;
@@ -332,8 +404,15 @@ int xi_attention_decode_bf16(const void* q, const void* k_cache, const void* vt_
 #undef XI_DC
   XI_LAUNCH_CHECK("attention_decode_split");
   if (max_splits == 1) return 0;   // the split kernel has written the result
-  attn_decode_combine_kernel<<<dim3(nq, n_seq), 64, max_splits * sizeof(float), stream>>>(part_o, part_ml, ctx_lens, (bf16*)out,
-                                                                  max_splits, window, nq, d, keys_per_wg);
+  if (max_splits > kCombineWideFrom) {
+    const size_t wide_lds = (size_t)(max_splits + kWideWaves * d + 2 * kWideWaves) * sizeof(float);
+    XI_CHECK(wide_lds <= 64 * 1024, "attention_decode: %d splits of head_dim %d are too many", max_splits, d);
+    attn_decode_combine_wide_kernel<<<dim3(nq, n_seq), 64 * kWideWaves, wide_lds, stream>>>(
+        part_o, part_ml, ctx_lens, (bf16*)out, max_splits, window, nq, d, keys_per_wg);
+  } else {
+    attn_decode_combine_kernel<<<dim3(nq, n_seq), 64, max_splits * sizeof(float), stream>>>(
+        part_o, part_ml, ctx_lens, (bf16*)out, max_splits, window, nq, d, keys_per_wg);
+  }
   XI_LAUNCH_CHECK("attention_decode_combine");
   return 0;
 }
