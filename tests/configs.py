@@ -38,7 +38,7 @@ TINY["O"] = dict(
     seed=5, linear_std=0.04, norm_std=0.15, page_size=8)
 
 
-# Real layer sizes (Qwen3-0.6B, 4B, 8B and 32B) with few layers and a small vocabulary: the
+# Real layer sizes (Qwen3-0.6B, 4B, 8B, 14B and 32B) with few layers and a small vocabulary: the
 # kernels run at the head size, group, widths and K lengths they serve in production.
 REAL = {
     "8B": dict(
@@ -56,6 +56,11 @@ REAL = {
                     head_dim=128, intermediate_size=9728, vocab_size=1601, rope_theta=1e6,
                     rms_norm_eps=1e-6, tie_word_embeddings=True, max_position_embeddings=1024),
         seed=7, linear_std=0.02, norm_std=0.1, page_size=64),
+    "14B": dict(
+        config=_cfg(num_hidden_layers=1, hidden_size=5120, num_attention_heads=40, num_key_value_heads=8,
+                    head_dim=128, intermediate_size=17408, vocab_size=1409, rope_theta=1e6,
+                    rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=1024),
+        seed=8, linear_std=0.02, norm_std=0.1, page_size=64),
     "32B": dict(
         config=_cfg(num_hidden_layers=1, hidden_size=5120, num_attention_heads=64, num_key_value_heads=8,
                     head_dim=128, intermediate_size=25600, vocab_size=1501, rope_theta=1e6,

@@ -107,7 +107,7 @@ def test_float32_does_not_depend_on_cutting(name, model_dirs):
 # ---- real layer sizes ---------------------------------------------------------------------------
 @pytest.mark.parametrize("name", list(REAL))
 def test_real_layer_sizes(name, real_model_dirs):
-    """Qwen3-0.6B, 4B, 8B and 32B layer sizes (few layers, small vocabulary): whole requests, a
+    """Qwen3-0.6B, 4B, 8B, 14B and 32B layer sizes (few layers, small vocabulary): whole requests, a
     mixed trace with pages used again and a tail decoded one by one, in float32 and in
     bfloat16, against the plain implementation."""
     from xinfer_amd.engine import ModelRunner, load_model
@@ -133,7 +133,7 @@ def test_real_layer_sizes(name, real_model_dirs):
         torch.cuda.empty_cache()
 
 
-@pytest.mark.parametrize("name,live", [("8B", 12), ("8B", 40), ("32B", 16), ("32B", 70), ("0.6B", 9), ("0.6B", 33),
+@pytest.mark.parametrize("name,live", [("8B", 12), ("8B", 40), ("14B", 8), ("14B", 48), ("32B", 16), ("32B", 70), ("0.6B", 9), ("0.6B", 33),
                                        ("4B", 16), ("4B", 64)])
 def test_real_layer_sizes_wide_decode_batches(name, live, real_model_dirs):
     """Decode steps of many requests at real layer sizes, in bfloat16: the kernels that serve 6 to
