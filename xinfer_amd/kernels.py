@@ -260,15 +260,16 @@ def gemm_tn(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] =
 
 
 DECODE_KEYS_PER_WORKGROUP = 256
-DECODE_KEYS_PER_WORKGROUP_MOST = 2048
+DECODE_KEYS_PER_WORKGROUP_MOST = 512
 DECODE_WORKGROUPS_MOST = 3000
 
 
 def decode_keys_per_workgroup(pairs: int, span: int, similar: bool = False) -> int:
     """Keys per workgroup of the split-K decode kernel for `pairs` (sequence, kv head) pairs of
     up to `span` keys: 256 (each of the four waves takes two steps) unless that makes thousands
-    of workgroups, where 512, 1024 or 2048 make fewer partial results to write and combine (4
-    sequences of 65,536 keys: 207 us at 256, 181 at 2048).  `similar`: the
+    of workgroups, where 512 halves the partial results to write and combine (more keys gain
+    another 4 to 6% where all sequences are long and equally so, and lose 20 to 50% in batches of
+    mixed lengths, measured at 16 to 128 sequences of 128 to 16,384 keys).  `similar`: the
     sequences are about equally long; then, if the pairs alone fill the compute units evenly, a
     workgroup takes a whole sequence: long loops, no partial results, no second kernel (measured
     on an MI355X: 8 to 11% less time at 256 to 1024 pairs, but a quarter more where the pairs
