@@ -44,7 +44,7 @@ __device__ __forceinline__ bf16x8 zero8() {
 }
 
 // =====================================================================================
-// Decode: every sequence has one query token.  Workgroup (split, kv head, sequence): the
+// Decode: every sequence has one query token.  Workgroup (kv head, sequence, split): the
 // query heads of the kv group are the columns of one tile; the workgroup's four waves take
 // alternate 32-key steps of its chunk of `keys_per_wg` keys and merge through LDS.  A wave keeps loads in flight all the time: the K operands of the next
 // step are asked for as soon as the scores of this one are computed, the V operands as soon
@@ -62,7 +62,11 @@ __global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
   extern __shared__ float lds[];  // [4 waves][g][d] + [4][g][2] + page numbers of the chunk
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, j = lane >> 4;
-  const int split = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
+  // the kv head runs fastest: workgroups go to the chip's eight dies in turn, and with eight kv
+  // heads a die then has one head of every sequence and split, the same work as every other die
+  // (with the split fastest and an even number of splits, one half of the dies got the full
+  // chunks and the other half the sequences' short last ones)
+  const int kvh = blockIdx.x, seq = blockIdx.y, split = blockIdx.z;
   const int g = nq / nkv;
   const int ctx = ctx_lens[seq];
   const int pos = ctx - 1;
@@ -392,7 +396,7 @@ int xi_attention_decode_bf16(const void* q, const void* k_cache, const void* vt_
   const size_t lds = (size_t)(4 * g * d + 4 * g * 2) * sizeof(float) + (size_t)(keys_per_wg / page + 2) * sizeof(int);
   XI_CHECK(lds <= 64 * 1024, "attention_decode: group %d x head_dim %d needs too much LDS", g, d);
   if (n_seq == 0) return 0;
-  dim3 grid(max_splits, nkv, n_seq);
+  dim3 grid(nkv, n_seq, max_splits);
   const float sl = scale * kLog2e;
 #define XI_DC(KC, DT)                                                                              \
   attn_decode_split_kernel<KC, DT><<<grid, 256, lds, stream>>>(                                    \
