@@ -850,10 +850,16 @@ def test_attention_decode_many_splits(nq, nkv, d, page, window, seqs, kpw):
 
 
 def test_decode_keys_per_workgroup_grow_with_the_work():
+    """About 512 workgroups a launch: chunks of 128 keys for one short sequence, of 2,048 for long ones;
+    at most 512 where the lengths are mixed."""
     from xinfer_amd import kernels
-    assert kernels.decode_keys_per_workgroup(64, 4096) == 256
-    assert kernels.decode_keys_per_workgroup(8, 131072) == 512
-    assert kernels.decode_keys_per_workgroup(1024, 1 << 20) == 512
+    assert kernels.decode_keys_per_workgroup(8, 4096, similar=True) == 128
+    assert kernels.decode_keys_per_workgroup(64, 4096, similar=True) == 512
+    assert kernels.decode_keys_per_workgroup(8, 131072, similar=True) == 2048
+    assert kernels.decode_keys_per_workgroup(1024, 1 << 20, similar=True) > 1 << 20      # one split
+    assert kernels.decode_keys_per_workgroup(1100, 1 << 20, similar=True) == 2048
+    assert kernels.decode_keys_per_workgroup(512, 2304, similar=False) == 512
+    assert kernels.decode_keys_per_workgroup(64, 1 << 20, similar=False) == 512
 
 
 @pytest.mark.parametrize("window", [0, 100])
@@ -865,8 +871,8 @@ def test_attention_decode_one_split_per_sequence(window):
     g = torch.Generator().manual_seed(23)
     seqs = [(290 + (7 * b) % 30, 1) for b in range(32)]
     assert kernels.decode_keys_per_workgroup(32 * nkv, 320, similar=True) > 320
-    assert kernels.decode_keys_per_workgroup(32 * nkv, 320, similar=False) == 256
-    assert kernels.decode_keys_per_workgroup(48 * nkv, 320, similar=True) == 256     # 384 pairs leave units idle
+    assert kernels.decode_keys_per_workgroup(32 * nkv, 320, similar=False) == 128
+    assert kernels.decode_keys_per_workgroup(48 * nkv, 320, similar=True) == 128     # 384 pairs leave units idle
     case = _paged_case(g, torch.bfloat16, nq, nkv, d, page, seqs)
     scale = 1.0 / math.sqrt(d)
     ref = _attention_ref(case, seqs, window, scale)

@@ -66,7 +66,9 @@ __global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
   // heads a die then has one head of every sequence and split, the same work as every other die
   // (with the split fastest and an even number of splits, one half of the dies got the full
   // chunks and the other half the sequences' short last ones)
-  const int kvh = blockIdx.x, seq = blockIdx.y, split = blockIdx.z;
+  // The last splits are launched first: only the longest sequences have them, and launched last
+  // they would run alone at the end.
+  const int kvh = blockIdx.x, seq = blockIdx.y, split = gridDim.z - 1 - blockIdx.z;
   const int g = nq / nkv;
   const int ctx = ctx_lens[seq];
   const int pos = ctx - 1;

@@ -296,7 +296,7 @@ class ModelRunner:
                                  ex.kind, f"the step could not be prepared ({ex.kind})")) from None
         bucket = 1024
         while bucket < longest:
-            bucket *= 4
+            bucket *= 2
         g = self._graphs.get((B, bucket, similar))
         if g is None:
             return None
@@ -359,7 +359,7 @@ class ModelRunner:
         longest = int(a.ctx_lens.max())
         bucket = 1024
         while bucket < longest:
-            bucket *= 4
+            bucket *= 2
         key = (B, bucket, _similar(a.ctx_lens))     # what kernels choose their shapes from
         all_rows = np.zeros(B, dtype=np.int32)
         all_rows[:rows32.size] = rows32

@@ -259,27 +259,31 @@ def gemm_tn(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] =
     return out
 
 
-DECODE_KEYS_PER_WORKGROUP = 256
-DECODE_KEYS_PER_WORKGROUP_MOST = 512
-DECODE_WORKGROUPS_MOST = 3000
+DECODE_WORKGROUPS = 512             # workgroups of the split-K decode kernel a launch aims at: two a compute unit
+DECODE_KEYS_LEAST = 128             # keys of a workgroup: from one 32-key step a wave
+DECODE_KEYS_MOST = 2048             # to sixteen, where the sequences are about equally long,
+DECODE_KEYS_MOST_MIXED = 512        # and four where they are not
 
 
 def decode_keys_per_workgroup(pairs: int, span: int, similar: bool = False) -> int:
     """Keys per workgroup of the split-K decode kernel for `pairs` (sequence, kv head) pairs of
-    up to `span` keys: 256 (each of the four waves takes two steps) unless that makes thousands
-    of workgroups, where 512 halves the partial results to write and combine (more keys gain
-    another 4 to 6% where all sequences are long and equally so, and lose 20 to 50% in batches of
-    mixed lengths, measured at 16 to 128 sequences of 128 to 16,384 keys).  `similar`: the
-    sequences are about equally long; then, if the pairs alone fill the compute units evenly, a
-    workgroup takes a whole sequence: long loops, no partial results, no second kernel (measured
-    on an MI355X: 8 to 11% less time at 256 to 1024 pairs, but a quarter more where the pairs
-    leave compute units idle at the end, and no gain where one sequence is much longer)."""
+    up to `span` keys: the power of two (times 128) that makes about DECODE_WORKGROUPS
+    workgroups.  Launching a workgroup costs the chip about 5 ns whatever it does, so thousands of
+    small ones lose to a few hundred larger ones (8 sequences of 4,096 keys on 8 kv heads: 33.9 us
+    at 256 keys, 30.9 at 512; one sequence of 4,096: 11.2 us at 128, 13.0 at 256, 16.3 at 512; 16
+    of 32,768: 435 us at 256, 376 at 2,048), while chunks much longer than a batch's shorter
+    sequences leave workgroups of very different lengths (64 sequences of 256 to 2,304 keys: 75
+    us at 512, 81 at 1,024).  `similar`: the sequences are about equally long; then, if the
+    pairs alone fill the compute units evenly, a workgroup takes a whole sequence: long loops, no
+    partial results, no second kernel (8 to 11% less time at 256 to 1024 pairs, but a quarter more
+    where the pairs leave compute units idle at the end)."""
     if similar and pairs >= COMPUTE_UNITS:
         rounds = pairs / COMPUTE_UNITS
         if math.ceil(rounds) / rounds <= 1.1:
             return (span + 128) // 128 * 128          # more than span: one split
-    kpw = DECODE_KEYS_PER_WORKGROUP
-    while kpw < DECODE_KEYS_PER_WORKGROUP_MOST and pairs * (span // kpw + 1) > DECODE_WORKGROUPS_MOST:
+    most = DECODE_KEYS_MOST if similar else DECODE_KEYS_MOST_MIXED
+    kpw = DECODE_KEYS_LEAST
+    while kpw < most and pairs * span >= 2 * kpw * DECODE_WORKGROUPS:
         kpw *= 2
     return kpw
 
