@@ -268,8 +268,8 @@ DECODE_KEYS_MOST_MIXED = 512        # and four where they are not
 def decode_keys_per_workgroup(pairs: int, span: int, similar: bool = False) -> int:
     """Keys per workgroup of the split-K decode kernel for `pairs` (sequence, kv head) pairs of
     up to `span` keys: the power of two (times 128) that makes about DECODE_WORKGROUPS
-    workgroups.  Launching a workgroup costs the chip about 5 ns whatever it does, so thousands of
-    small ones lose to a few hundred larger ones (8 sequences of 4,096 keys on 8 kv heads: 33.9 us
+    workgroups.  A workgroup costs the chip about 5 ns beyond its keys (launch, page numbers, merge,
+    partial results), so thousands of small ones lose to a few hundred larger ones (8 sequences of 4,096 keys on 8 kv heads: 33.9 us
     at 256 keys, 30.9 at 512; one sequence of 4,096: 11.2 us at 128, 13.0 at 256, 16.3 at 512; 16
     of 32,768: 435 us at 256, 376 at 2,048), while chunks much longer than a batch's shorter
     sequences leave workgroups of very different lengths (64 sequences of 256 to 2,304 keys: 75
