@@ -609,6 +609,45 @@ def test_qk_norm_rope_kv_bias(dtype, T, nq, nkv, d, rot, interleaved):
                                 bias=bias[:-1].contiguous().to(DEV))
 
 
+@pytest.mark.parametrize("T,nq,nkv,d,rot,interleaved,slices,with_bias", [
+    (20, 4, 2, 128, 128, False, 5, False), (33, 6, 3, 48, 32, True, 3, True), (1, 2, 1, 256, 256, False, 1, False),
+    (300, 4, 4, 64, 64, False, 8, True)])
+def test_qk_norm_rope_kv_of_partial_sums(T, nq, nkv, d, rot, interleaved, slices, with_bias):
+    """The packed rows as float32 partial sums of a product cut along K (what the tiled split-K
+    product hands on): the kernel adds the slices, then does as with rows; against the plain
+    formulas on the sum, and with one wave per head whatever the number of tokens."""
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(31)
+    page, pages, eps = 16, 24, 1e-6
+    positions = torch.randint(0, 300, (T,), generator=g).to(torch.int32)
+    cos, sin = plain.rope_tables(1e6, rot, 300)
+    width = (nq + 2 * nkv) * d
+    parts = torch.randn((slices, T, width), generator=g)
+    bias = torch.randn(width, generator=g) * 0.5 if with_bias else None
+    qw, kw = 1 + 0.3 * torch.randn(d, generator=g), 1 + 0.3 * torch.randn(d, generator=g)
+    slots = torch.randperm(pages * page, generator=g)[:T].to(torch.int64)
+    kc = torch.zeros((pages, nkv, page, d), dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros((pages, nkv, d, page), dtype=torch.bfloat16, device=DEV)
+    q_out = kernels.qk_norm_rope_kv(parts.to(DEV), qw.to(DEV), kw.to(DEV), eps, cos.to(DEV), sin.to(DEV), rot, interleaved,
+                                    positions.to(DEV), slots.to(DEV), kc, vc, nq, nkv, d, v_transposed=True,
+                                    bias=None if bias is None else bias.to(DEV))
+    assert q_out.dtype == torch.bfloat16 and tuple(q_out.shape) == (T, nq, d)
+    total = parts.double().sum(0) + (0 if bias is None else bias.double())
+    x = total.reshape(T, nq + 2 * nkv, d)
+    q = _rope_ref(plain.rms_norm(x[:, :nq], qw.double(), eps), positions.long(), cos, sin, rot, interleaved)
+    k = _rope_ref(plain.rms_norm(x[:, nq:nq + nkv], kw.double(), eps), positions.long(), cos, sin, rot, interleaved)
+    v = x[:, nq + nkv:]
+    tol = _tol(torch.bfloat16)
+    assert (q_out.cpu().double() - q).abs().max() / q.abs().max() < tol
+    got_k = kc.cpu().double().permute(0, 2, 1, 3).reshape(pages * page, nkv, d)
+    got_v = vc.cpu().double().permute(0, 3, 1, 2).reshape(pages * page, nkv, d)
+    assert (got_k[slots] - k).abs().max() / k.abs().max() < tol
+    assert (got_v[slots] - v).abs().max() / v.abs().max() < tol
+    with pytest.raises(kernels.KernelError, match="partial sums"):
+        kernels.qk_norm_rope_kv(parts.to(DEV).to(torch.bfloat16), qw.to(DEV), kw.to(DEV), eps, cos.to(DEV), sin.to(DEV), rot,
+                                interleaved, positions.to(DEV), slots.to(DEV), kc, vc, nq, nkv, d, v_transposed=True)
+
+
 def _paged_case(g, dtype, nq, nkv, d, page, seqs, extra_pages=3):
     """Random K/V of several sequences laid into a paged cache under a shuffled page map.
     `seqs` = list of (context length, number of query tokens at its end)."""

@@ -216,8 +216,11 @@ __global__ void silu_mul_vec8_kernel(const bf16* __restrict__ gu, bf16* __restri
 //   bias: it is added here, in float32, to the product the row holds (q, k and v alike;
 //   reference attention.rs:819-828 adds it in the linear layer).
 // ---------------------------------------------------------------------------------
-template <typename T>
-__global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, const float* __restrict__ bias,
+// PARTS: the packed rows come as `slices` float32 partial sums [slices, T, heads * d] (a product
+// cut along K, `slice_stride` elements apart), added here in slice order.
+template <typename T, bool PARTS>
+__global__ void qk_norm_rope_kv_kernel(const void* __restrict__ qkv_v, int slices, size_t slice_stride,
+                                       const float* __restrict__ bias,
                                        const float* __restrict__ qw,
                                        const float* __restrict__ kw, float eps,
                                        const float* __restrict__ cos_t,
@@ -232,8 +235,20 @@ __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, const float* _
   if (wid >= (long long)n_tok * heads) return;
   const int t = (int)(wid / heads);
   const int h = (int)(wid - (long long)t * heads);
-  const T* src = qkv + (size_t)t * heads * d + (size_t)h * d;
+  const size_t row0 = (size_t)t * heads * d + (size_t)h * d;
   const float* bs = bias ? bias + (size_t)h * d : nullptr;
+  // element i of this head's row, without the bias
+  auto ld = [&](int i) -> float {
+    if constexpr (PARTS) {
+      const float* p = reinterpret_cast<const float*>(qkv_v) + row0 + i;
+      float a = 0.f;
+#pragma unroll 4
+      for (int sl = 0; sl < slices; ++sl) a += p[(size_t)sl * slice_stride];
+      return a;
+    } else {
+      return to_float(reinterpret_cast<const T*>(qkv_v)[row0 + i]);
+    }
+  };
 
   T* dst;
   const float* w = nullptr;
@@ -251,7 +266,7 @@ __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, const float* _
     if (!is_k && v_transposed) {  // V kept as [page, kv_head, d, offset]
       T* vt = v_cache + ((size_t)page * nkv + kvh) * d * page_size + off;
       for (int i = lane; i < d; i += kWave)
-        vt[(size_t)i * page_size] = bs ? from_float<T>(to_float(src[i]) + bs[i]) : src[i];
+        vt[(size_t)i * page_size] = from_float<T>(bs ? ld(i) + bs[i] : ld(i));
       return;
     }
     T* cache = is_k ? k_cache : v_cache;
@@ -260,7 +275,7 @@ __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, const float* _
     rotate = is_k;
   }
   if (!rotate) {  // v: plain copy
-    for (int i = lane; i < d; i += kWave) dst[i] = bs ? from_float<T>(to_float(src[i]) + bs[i]) : src[i];
+    for (int i = lane; i < d; i += kWave) dst[i] = from_float<T>(bs ? ld(i) + bs[i] : ld(i));
     return;
   }
   // The kernel lives on latency: everything that can be asked for at once is.  A lane holds
@@ -276,8 +291,8 @@ __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, const float* _
     const bool ok = i < half;
     const int ia = interleaved ? 2 * i : i;
     const int ib = interleaved ? 2 * i + 1 : i + half;
-    xa[p] = ok ? to_float(src[ia]) + (bs ? bs[ia] : 0.f) : 0.f;
-    xb[p] = ok ? to_float(src[ib]) + (bs ? bs[ib] : 0.f) : 0.f;
+    xa[p] = ok ? ld(ia) + (bs ? bs[ia] : 0.f) : 0.f;
+    xb[p] = ok ? ld(ib) + (bs ? bs[ib] : 0.f) : 0.f;
     wa[p] = (ok && w) ? w[ia] : 1.f;
     wb[p] = (ok && w) ? w[ib] : 1.f;
   }
@@ -285,7 +300,7 @@ __global__ void qk_norm_rope_kv_kernel(const T* __restrict__ qkv, const float* _
   for (int p = 0; p < 4; ++p) {
     const int i = rot + lane + kWave * p;
     const bool ok = i < d;
-    xt[p] = ok ? to_float(src[i]) + (bs ? bs[i] : 0.f) : 0.f;
+    xt[p] = ok ? ld(i) + (bs ? bs[i] : 0.f) : 0.f;
     wt[p] = (ok && w) ? w[i] : 1.f;
   }
   const float* c = cos_t + (size_t)pos * half;
@@ -552,7 +567,9 @@ int xi_silu_mul(const void* gate_up, void* out, int dtype, int n_tok, int I, hip
   return 0;
 }
 
-int xi_qk_norm_rope_kv(const void* qkv, int dtype, const float* bias, const float* qw, const float* kw, float eps,
+// qkv: [T, heads * d] in `dtype`, or, with slices > 0, float32 partial sums [slices, T, heads * d]
+// of it (then `dtype` is that of q_out and the cache, and the form of one wave per head runs).
+int xi_qk_norm_rope_kv(const void* qkv, int dtype, int slices, const float* bias, const float* qw, const float* kw, float eps,
                        const float* cos_t, const float* sin_t, int rot, int interleaved,
                        const int* positions, const long long* slots, void* q_out, void* k_cache,
                        void* v_cache, int page_size, int n_tok, int nq, int nkv, int d, int v_transposed,
@@ -565,7 +582,8 @@ int xi_qk_norm_rope_kv(const void* qkv, int dtype, const float* bias, const floa
   if (n_tok == 0) return 0;
   // Many tokens (prompt portions): the vectorized form.  Few (decode steps): one wave per
   // (token, head) below, whose shorter chain of dependent loads finishes sooner.
-  if (n_tok >= vector_min_tokens && dtype == kBF16 && v_transposed && d % 8 == 0 && d <= 256 &&
+  XI_CHECK(slices >= 0 && slices <= 64, "qk_norm_rope_kv: %d slices", slices);
+  if (slices == 0 && n_tok >= vector_min_tokens && dtype == kBF16 && v_transposed && d % 8 == 0 && d <= 256 &&
       (interleaved || rot % 16 == 0) &&
       ((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)cos_t | (uintptr_t)sin_t) % 16 == 0) {
     const int lph = d / 8, hpw = 64 / lph;
@@ -585,12 +603,15 @@ int xi_qk_norm_rope_kv(const void* qkv, int dtype, const float* bias, const floa
   const int wpb = 4;
   const long long blocks = (waves + wpb - 1) / wpb;
   XI_CHECK(blocks < (1ll << 31), "qk_norm_rope_kv: too many tokens");
-#define XI_QK(TT)                                                                               \
-  qk_norm_rope_kv_kernel<TT><<<(unsigned)blocks, wpb * kWave, 0, stream>>>(                     \
-      (const TT*)qkv, bias, qw, kw, eps, cos_t, sin_t, rot, interleaved, positions, slots, (TT*)q_out, \
+  const size_t slice_stride = (size_t)n_tok * (nq + 2 * nkv) * d;
+#define XI_QK(TT, PARTS)                                                                        \
+  qk_norm_rope_kv_kernel<TT, PARTS><<<(unsigned)blocks, wpb * kWave, 0, stream>>>(              \
+      qkv, slices, slice_stride, bias, qw, kw, eps, cos_t, sin_t, rot, interleaved, positions, slots, (TT*)q_out, \
       (TT*)k_cache, (TT*)v_cache, page_size, n_tok, nq, nkv, d, v_transposed)
-  if (dtype == kF32) XI_QK(float);
-  else if (dtype == kBF16) XI_QK(bf16);
+  if (dtype == kF32 && slices == 0) XI_QK(float, false);
+  else if (dtype == kF32) XI_QK(float, true);
+  else if (dtype == kBF16 && slices == 0) XI_QK(bf16, false);
+  else if (dtype == kBF16) XI_QK(bf16, true);
   else XI_CHECK(false, "qk_norm_rope_kv: unknown dtype %d", dtype);
 #undef XI_QK
   XI_LAUNCH_CHECK("qk_norm_rope_kv");

@@ -159,11 +159,19 @@ def qk_norm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor],
     [T, nq, d], k and v into the paged cache [pages, nkv, page_size, d] at `slots`; with
     `v_transposed` the V pool is [pages, nkv, d, page_size].  From `vector_min_tokens` tokens
     on, bfloat16 with the transposed pool runs the vectorized kernel.  `bias` (float32, one
-    value per element of a packed row) is added to the rows first, in float32."""
+    value per element of a packed row) is added to the rows first, in float32.  `qkv` may be a
+    stack [slices, T, width] of float32 partial sums (`linear_mid`), added here in slice order;
+    q and the cache then have the cache's dtype and the form of one wave per head runs."""
     _dev(qkv, q_weight, k_weight, cos, sin, positions, slots, k_cache, v_cache, q_out, bias)
     nq, nkv, d = num_heads, num_kv_heads, head_dim
-    T = qkv.shape[0]
-    if qkv.dim() != 2 or qkv.shape[1] != (nq + 2 * nkv) * d:
+    slices, dtype = 0, qkv.dtype
+    if qkv.dim() == 3:            # float32 partial sums [slices, T, width] of a product cut along K
+        _want(qkv, torch.float32, "qk_norm_rope_kv: partial sums")
+        slices, dtype = int(qkv.shape[0]), k_cache.dtype
+        if not (0 < slices <= 64) or not qkv.is_contiguous():
+            raise KernelError(f"qk_norm_rope_kv: partial sums {tuple(qkv.shape)} must be contiguous [1..64, T, width]")
+    T = qkv.shape[-2]
+    if qkv.dim() not in (2, 3) or qkv.shape[-1] != (nq + 2 * nkv) * d:
         raise KernelError(f"qk_norm_rope_kv: qkv {tuple(qkv.shape)} is not [T, {(nq + 2 * nkv) * d}]")
     _want(positions, torch.int32, "qk_norm_rope_kv: positions")
     _want(slots, torch.int64, "qk_norm_rope_kv: slots")
@@ -180,15 +188,15 @@ def qk_norm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor],
                 raise KernelError("qk_norm_rope_kv: norm weight must be [head_dim]")
     if bias is not None:
         _want(bias, torch.float32, "qk_norm_rope_kv: bias")
-        if bias.shape != (qkv.shape[1],):
-            raise KernelError(f"qk_norm_rope_kv: bias {tuple(bias.shape)} is not [{qkv.shape[1]}]")
-    _check_cache(k_cache, v_cache, nkv, d, qkv.dtype, v_transposed, "qk_norm_rope_kv")
+        if bias.shape != (qkv.shape[-1],):
+            raise KernelError(f"qk_norm_rope_kv: bias {tuple(bias.shape)} is not [{qkv.shape[-1]}]")
+    _check_cache(k_cache, v_cache, nkv, d, dtype, v_transposed, "qk_norm_rope_kv")
     if q_out is None:
-        q_out = torch.empty((T, nq, d), dtype=qkv.dtype, device=qkv.device)
-    elif q_out.shape != (T, nq, d) or q_out.dtype != qkv.dtype:
+        q_out = torch.empty((T, nq, d), dtype=dtype, device=qkv.device)
+    elif q_out.shape != (T, nq, d) or q_out.dtype != dtype:
         raise KernelError("qk_norm_rope_kv: q_out has the wrong shape or dtype")
     _ok(lib().xi_qk_norm_rope_kv(
-        _p(qkv), _code(qkv, "qk_norm_rope_kv"), _p(bias), _p(q_weight), _p(k_weight), ctypes.c_float(eps),
+        _p(qkv), _code(q_out, "qk_norm_rope_kv"), slices, _p(bias), _p(q_weight), _p(k_weight), ctypes.c_float(eps),
         _p(cos), _p(sin), int(rotary_dim), int(bool(interleaved)), _p(positions), _p(slots),
         _p(q_out), _p(k_cache), _p(v_cache), int(k_cache.shape[2]), T, nq, nkv, d,
         int(bool(v_transposed)), int(vector_min_tokens), _stream()))

@@ -16,13 +16,14 @@ import torch
 from .. import kernels
 from ..config.spec import PartSpec
 from ..weights.store import TensorDecl, WeightStore
-from .base import (KVNeed, LayerCache, Mixer, StepContext, position_encoding_class,
+from .base import (Folded, KVNeed, LayerCache, Mixer, StepContext, position_encoding_class,
                    register_mixer)
 from .linear import Linear
 
 
 @register_mixer("attention")
 class PagedAttention(Mixer):
+    VECTOR_MIN_DECODE = 512      # decoded tokens lie in a page each: the form with one wave per head stays ahead up to here
     graph_safe = True
 
     def __init__(self, spec: PartSpec, dtype: torch.dtype):
@@ -89,7 +90,12 @@ class PagedAttention(Mixer):
 
     def forward(self, x, ctx: StepContext, cache: LayerCache, sink=None):
         """`x`: rows or a `Folded`; `sink`: see `Part.takes_sink`."""
-        qkv = self.qkv(x, out_dtype=self.dtype)
+        # a decode step of 17 to 256 rows: the tiled split-K product is ahead of the library, and the
+        # kernel below adds its partial sums (which the form for prompt portions does not take)
+        rows = None if isinstance(x, Folded) else x.shape[0]
+        parts = (rows is not None and self.dtype == torch.bfloat16 and ctx.max_q_len == 1
+                 and kernels.MID_FROM <= rows <= min(kernels.MID_ROWS, self.VECTOR_MIN_DECODE - 1))
+        qkv = self.qkv(x, out_dtype=self.dtype, allow_split=parts)
         pos = self.position
         slots = ctx.slots[cache.group] if cache.write else ctx.no_slots
         vt = self.dtype == torch.bfloat16
@@ -100,7 +106,6 @@ class PagedAttention(Mixer):
             pos.rotary_dim if pos is not None else 0,
             pos.interleaved if pos is not None else False,
             ctx.positions, slots, cache.k, cache.v, self.nq, self.nkv, self.d, v_transposed=vt,
-            # decoded tokens lie in a page each: the form with one wave per head stays ahead longer
-            vector_min_tokens=128 if ctx.max_q_len > 1 else 512, bias=self.qkv_bias)
+            vector_min_tokens=128 if ctx.max_q_len > 1 else self.VECTOR_MIN_DECODE, bias=self.qkv_bias)
         a = kernels.attention(q, cache.k, cache.v, ctx, cache.group, self.scale, self.window, v_transposed=vt)
         return self.o(a, out_dtype=self.dtype, allow_split=True, sink=sink)     # the next norm adds the parts
