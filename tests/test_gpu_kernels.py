@@ -889,16 +889,15 @@ def test_attention_decode_many_splits(nq, nkv, d, page, window, seqs, kpw):
 
 
 def test_decode_keys_per_workgroup_grow_with_the_work():
-    """About 512 workgroups a launch: chunks of 128 keys for one short sequence, of 2,048 for long ones;
-    at most 512 where the lengths are mixed."""
+    """About 512 workgroups a launch: chunks of 128 keys for one short sequence, of 512 at most."""
     from xinfer_amd import kernels
     assert kernels.decode_keys_per_workgroup(8, 4096, similar=True) == 128
+    assert kernels.decode_keys_per_workgroup(32, 4096, similar=True) == 256
     assert kernels.decode_keys_per_workgroup(64, 4096, similar=True) == 512
-    assert kernels.decode_keys_per_workgroup(8, 131072, similar=True) == 2048
+    assert kernels.decode_keys_per_workgroup(8, 131072, similar=True) == 512
     assert kernels.decode_keys_per_workgroup(1024, 1 << 20, similar=True) > 1 << 20      # one split
-    assert kernels.decode_keys_per_workgroup(1100, 1 << 20, similar=True) == 2048
+    assert kernels.decode_keys_per_workgroup(1100, 1 << 20, similar=True) == 512
     assert kernels.decode_keys_per_workgroup(512, 2304, similar=False) == 512
-    assert kernels.decode_keys_per_workgroup(64, 1 << 20, similar=False) == 512
 
 
 @pytest.mark.parametrize("window", [0, 100])

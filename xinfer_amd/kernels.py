@@ -269,29 +269,30 @@ def gemm_tn(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] =
 
 DECODE_WORKGROUPS = 512             # workgroups of the split-K decode kernel a launch aims at: two a compute unit
 DECODE_KEYS_LEAST = 128             # keys of a workgroup: from one 32-key step a wave
-DECODE_KEYS_MOST = 2048             # to sixteen, where the sequences are about equally long,
-DECODE_KEYS_MOST_MIXED = 512        # and four where they are not
+DECODE_KEYS_MOST = 512              # to four
 
 
 def decode_keys_per_workgroup(pairs: int, span: int, similar: bool = False) -> int:
     """Keys per workgroup of the split-K decode kernel for `pairs` (sequence, kv head) pairs of
-    up to `span` keys: the power of two (times 128) that makes about DECODE_WORKGROUPS
-    workgroups.  A workgroup costs the chip about 5 ns beyond its keys (launch, page numbers, merge,
-    partial results), so thousands of small ones lose to a few hundred larger ones (8 sequences of 4,096 keys on 8 kv heads: 33.9 us
-    at 256 keys, 30.9 at 512; one sequence of 4,096: 11.2 us at 128, 13.0 at 256, 16.3 at 512; 16
-    of 32,768: 435 us at 256, 376 at 2,048), while chunks much longer than a batch's shorter
-    sequences leave workgroups of very different lengths (64 sequences of 256 to 2,304 keys: 75
-    us at 512, 81 at 1,024).  `similar`: the sequences are about equally long; then, if the
-    pairs alone fill the compute units evenly, a workgroup takes a whole sequence: long loops, no
-    partial results, no second kernel (8 to 11% less time at 256 to 1024 pairs, but a quarter more
-    where the pairs leave compute units idle at the end)."""
+    up to `span` keys: 128, 256 or 512, whichever makes about DECODE_WORKGROUPS workgroups.  A
+    workgroup costs the chip about 5 ns beyond its keys (launch, page numbers, merge, partial
+    results), so thousands of small ones lose to a few hundred larger ones (8 sequences of 4,096
+    keys on 8 kv heads: 33.9 us at 256 keys, 30.9 at 512; one sequence of 4,096: 11.2 us at 128,
+    13.0 at 256, 16.3 at 512).  Chunks of 1,024 or 2,048 keys gain another 4 to 8% on long
+    sequences of one length, but where they leave two or three workgroups a compute unit the time
+    depends on where the workgroups land (16 sequences of 8,400 keys in chunks of 2,048: 91 us
+    with a grid laid out for 10,240 keys, 115 for 16,384), and in batches of mixed lengths they
+    lose (64 sequences of 256 to 2,304 keys: 75 us at 512, 81 at 1,024): not used.  `similar`: the
+    sequences are about equally long; then, if the pairs alone fill the compute units evenly, a
+    workgroup takes a whole sequence: long loops, no partial results, no second kernel (8 to 11%
+    less time at 256 to 1024 pairs, but a quarter more where the pairs leave compute units idle
+    at the end)."""
     if similar and pairs >= COMPUTE_UNITS:
         rounds = pairs / COMPUTE_UNITS
         if math.ceil(rounds) / rounds <= 1.1:
             return (span + 128) // 128 * 128          # more than span: one split
-    most = DECODE_KEYS_MOST if similar else DECODE_KEYS_MOST_MIXED
     kpw = DECODE_KEYS_LEAST
-    while kpw < most and pairs * span >= 2 * kpw * DECODE_WORKGROUPS:
+    while kpw < DECODE_KEYS_MOST and pairs * span >= 2 * kpw * DECODE_WORKGROUPS:
         kpw *= 2
     return kpw
 
@@ -499,7 +500,10 @@ MID_ROWS = 256            # most rows of the tiled product for narrow outputs (`
 MID_WIDE_FROM = 4         # rows from which it is ahead of the streaming kernel on an output so wide that it needs no
                           # slices (the head: 215 against 242 us at 8 rows, 238 against 349 at 64, vocabulary 151936)
 MID_FROM = 17             # from this many rows on it is used, where the caller takes partial sums,
-MID_WIDEST = 8192         # for outputs up to this wide (wider ones have tiles enough for the library)
+MID_WIDEST = 12288        # for outputs up to this wide (N = 10240, K = 5120: 21 / 23 / 30 us at 17 / 64 / 128 rows against
+                          # 24 / 31 / 39 in the library), and above 128 rows (two passes over w) for weights from
+MID_BLOCK = 128           # (rows of one pass)
+MID_TWO_BLOCKS = 32 << 20  # this many bytes on (below, the library is ahead: 8 MB at 256 rows, 16 against 9 us)
 
 
 def linear_mid_slices(N: int, K: int) -> int:
@@ -721,8 +725,8 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtyp
     if out_dtype == torch.float32 and MID_WIDE_FROM <= x.shape[0] <= MID_GATED_ROWS \
             and linear_mid_slices(w.shape[0], w.shape[1]) == 1:
         return linear_mid(x, w)[0]           # a wide output in float32 (the head): one slice is the result
-    if allow_split and x.shape[0] <= MID_ROWS and linear_mid_slices(w.shape[0], w.shape[1]) > 0 \
-            and w.shape[0] <= MID_WIDEST and MID_FROM <= x.shape[0]:
+    if allow_split and MID_FROM <= x.shape[0] <= MID_ROWS and linear_mid_slices(w.shape[0], w.shape[1]) > 0 \
+            and w.shape[0] <= MID_WIDEST and (x.shape[0] <= MID_BLOCK or w.numel() * 2 >= MID_TWO_BLOCKS):
         return linear_mid(x, w)
     if (allow_split and x.shape[1] % 8 == 0 and x.shape[0] >= SKINNY_SPLIT_FROM
             and int(lib().xi_linear_skinny_slices(w.shape[0], w.shape[1], 0, 1)) > 1):
