@@ -168,8 +168,9 @@ class LLMEngine:
             if any(s.frequency_penalty or s.presence_penalty for s in strategies):
                 recent = [r.tokens[max(r.prompt_len, len(r.tokens) - PENALTY_CONTEXT):] for r in sampled]
             tokens = self.sampler.sample(
-                logits, strategies, [uniform(r.seed, r.stream, len(r.tokens) - r.prompt_len) for r in sampled],
-                recent=recent)
+                logits, strategies,
+                [0.0 if r.strategy.greedy else uniform(r.seed, r.stream, len(r.tokens) - r.prompt_len) for r in sampled],
+                recent=recent)         # (a greedy row draws nothing)
             now = _now_ms()
             for r, tok in zip(sampled, tokens):
                 if len(r.tokens) == r.prompt_len:
