@@ -29,7 +29,7 @@ HOST_DIR = os.path.join(_HERE, "host")
 
 HIP_FLAGS = [
     "-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950",
-    # packed-FP32 instructions are kept out of the generated code on this hardware pool
+    # no packed-FP32 instructions in the generated code: some of their forms have given wrong results on gfx950
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
@@ -135,10 +135,17 @@ def build_kernels(force: bool = False) -> str:
     _say(f"compiling {len(srcs)} HIP sources for gfx950 into {lib}")
     t0 = time.time()
 
+    headers = _sources(KERNEL_DIR, (".h",))
+
     def one(src: str) -> str:
+        # an object is kept while its source, the headers and the flags are what it was made from
         obj = os.path.join(obj_dir, os.path.basename(src) + ".o")
+        own = _digest([src] + headers, HIP_FLAGS)
+        if not force and _current(obj, own):
+            return obj
         t = time.time()
         _run([hipcc, *HIP_FLAGS, "-I", KERNEL_DIR, "-c", src, "-o", obj], f"hipcc {os.path.basename(src)}")
+        _stamp(obj, own)
         _say(f"  {os.path.basename(src)} done in {time.time() - t:.0f}s")
         return obj
 
