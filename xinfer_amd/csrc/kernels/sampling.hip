@@ -12,6 +12,17 @@
 // bfloat16).  v is found without sorting, by a search over float bit patterns.  The draw
 // takes a uniform number from the caller and walks the kept tokens in index order.
 #include "common.h"
+#include "no_alloc.h"
+
+#include <mutex>
+
+// Scratch of `xi_argmax_static`: per row and chunk the winner's value (float) and index (int).
+// In host code this name is a stand-in, not a device address: host code uses the per-device
+// pointer that hipGetSymbolAddress gives (`static_scratch` below), never the name itself.
+constexpr int kStaticArgmaxRows = 256;
+constexpr int kStaticArgmaxChunks = 32;
+constexpr size_t kStaticArgmaxBytes = (size_t)kStaticArgmaxRows * kStaticArgmaxChunks * (sizeof(float) + sizeof(int));
+static __device__ __align__(256) unsigned char scratch[kStaticArgmaxBytes];
 
 namespace xi {
 
@@ -423,6 +434,59 @@ int xi_argmax(const float* logits, int rows, int V, int* out, float* pval, int* 
   XI_LAUNCH_CHECK("argmax_partial");
   argmax_merge_kernel<<<rows, 64, 0, stream>>>(pval, pidx, n_chunks, out);
   XI_LAUNCH_CHECK("argmax_merge");
+  return 0;
+}
+
+// ---- the entry point that allocates nothing (no_alloc.h) ----------------------------------
+// Each GPU holds its own copy of `scratch` at its own address; the address is asked for once
+// per device, with that device current, and kept.
+constexpr int kStaticMaxDevices = 64;
+static void* g_static_scratch[kStaticMaxDevices];
+static std::mutex g_static_mutex;
+
+static int static_scratch(unsigned char** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  XI_CHECK(e == hipSuccess, "argmax_static: hipGetDevice failed: %s", hipGetErrorString(e));
+  XI_CHECK(dev >= 0 && dev < kStaticMaxDevices, "argmax_static: device %d is beyond the %d this library keeps", dev,
+           kStaticMaxDevices);
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  if (g_static_scratch[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    XI_CHECK(e == hipSuccess && p != nullptr, "argmax_static: hipGetSymbolAddress failed on device %d: %s", dev,
+             hipGetErrorString(e));
+    g_static_scratch[dev] = p;
+  }
+  *ptr = static_cast<unsigned char*>(g_static_scratch[dev]);
+  return 0;
+}
+
+int xi_argmax_static_max_rows() { return kStaticArgmaxRows; }
+
+int xi_argmax_static(const float* logits, int rows, int V, int* out, hipStream_t stream) {
+  XI_CHECK(rows >= 0 && V > 0, "argmax_static: bad sizes rows=%d V=%d", rows, V);
+  XI_CHECK(rows <= kStaticArgmaxRows, "argmax_static: %d rows are more than the %d the fixed scratch holds", rows,
+           kStaticArgmaxRows);
+  if (rows == 0) return 0;
+  XI_CHECK(logits != nullptr && out != nullptr, "argmax_static: logits or out is null");
+  const int n_chunks = xi_argmax_chunks(V);
+  XI_CHECK(n_chunks <= kStaticArgmaxChunks, "argmax_static: %d chunks are more than the %d the fixed scratch holds",
+           n_chunks, kStaticArgmaxChunks);
+  if (n_chunks == 1) {
+    argmax_kernel<<<rows, kSampleThreads, 0, stream>>>(logits, V, out);
+    XI_LAUNCH_CHECK("argmax_static");
+    return 0;
+  }
+  unsigned char* base = nullptr;
+  if (int rc = static_scratch(&base)) return rc;
+  float* pval = reinterpret_cast<float*>(base);
+  int* pidx = reinterpret_cast<int*>(base + (size_t)kStaticArgmaxRows * kStaticArgmaxChunks * sizeof(float));
+  // stage one writes all rows * n_chunks slots that stage two reads: the last call's contents never show
+  argmax_partial_kernel<<<dim3(n_chunks, rows), 256, 0, stream>>>(logits, V, n_chunks, pval, pidx);
+  XI_LAUNCH_CHECK("argmax_static_partial");
+  argmax_merge_kernel<<<rows, 64, 0, stream>>>(pval, pidx, n_chunks, out);
+  XI_LAUNCH_CHECK("argmax_static_merge");
   return 0;
 }
 
