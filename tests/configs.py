@@ -67,3 +67,16 @@ REAL = {
                     rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=1024),
         seed=4, linear_std=0.02, norm_std=0.1, page_size=64),
 }
+
+
+# Long contexts: Qwen3-0.6B widths, two layers, 8,192 positions.  `sharpen` multiplies every
+# q_norm weight: scores then have a standard deviation of about 1.5 instead of 1, so that some
+# hundred of some thousand keys carry a row's softmax.  More would make a dropped or misplaced key
+# show more, but bfloat16's rounding of q and k grows with the scores too (measured on 3,000 tokens:
+# worst error 1.1% of the largest logit at 1, 1.4% at 1.5, 2.0% at 2, 2.8% at 3); float32 shows a
+# single dropped key at any sharpness.
+LONG = dict(
+    config=_cfg(num_hidden_layers=2, hidden_size=1024, num_attention_heads=16, num_key_value_heads=8,
+                head_dim=128, intermediate_size=3072, vocab_size=1201, rope_theta=1e6,
+                rms_norm_eps=1e-6, tie_word_embeddings=True, max_position_embeddings=8192),
+    seed=9, linear_std=0.03, norm_std=0.1, page_size=64, sharpen=1.5)
