@@ -182,3 +182,113 @@ def test_bias_is_one_more_input_column(tmp_path):
     no_bias = plain.attention_block(x1, W1, p, dict(c, attention_bias=False), positions, cos, sin, None)
     assert torch.allclose(with_bias, no_bias, atol=1e-12)
     assert f"{p}.o_proj.bias" not in W
+
+
+# ---- q/k norm and the embedding's scale -----------------------------------------------------------
+def _attention_inputs(tmp_path, T=7, eps=None):
+    """Tiny A's layer 0 in float64 (4 query heads in 2 groups, head size 32) with q_norm and k_norm
+    weights that differ within every rotation pair (i, i + d/2)."""
+    pm = _tiny_weights("A", tmp_path)
+    c = dict(pm.config)
+    if eps is not None:
+        c["rms_norm_eps"] = eps
+    p = "model.layers.0.self_attn"
+    W = {k: v.double().clone() for k, v in pm.weights.items() if k.startswith(p)}
+    d = c["head_dim"]
+    g = torch.Generator().manual_seed(12)
+    W[f"{p}.q_norm.weight"] = 0.5 + torch.rand(d, generator=g, dtype=torch.float64) * 2.0
+    W[f"{p}.k_norm.weight"] = 0.5 + torch.rand(d, generator=g, dtype=torch.float64) * 2.0
+    x = torch.randn(T, c["hidden_size"], generator=g, dtype=torch.float64)
+    positions = torch.arange(5, 5 + T)
+    cos, sin = plain.rope_tables(c["rope_theta"], d, 64)
+    return c, W, p, x, positions, cos.double(), sin.double()
+
+
+def test_qk_norm_is_per_head_with_one_weight_for_all_heads(tmp_path):
+    """The norm runs on [T * heads, d] with one weight vector of d values
+    (/root/reference/src/models/layers/attention.rs:732-741): (1) permuting the query heads together
+    with their kv heads, and the columns of o_proj with them, leaves the block's output unchanged (a
+    weight per head would not); (2) with eps = 0, multiplying one head's rows of q_proj, or one kv
+    head's rows of k_proj, by a constant changes nothing (a norm over all heads together, the full-width
+    form of attention.rs:723-731, would let it through to the other heads)."""
+    c, W, p, x, positions, cos, sin = _attention_inputs(tmp_path, eps=0.0)
+    nq, nkv, d = c["num_attention_heads"], c["num_key_value_heads"], c["head_dim"]
+    base = plain.attention_block(x, W, p, c, positions, cos, sin, None)
+
+    def heads(w, n, order):                    # rows of a projection, head blocks reordered
+        return w.reshape(n, d, -1)[order].reshape(n * d, -1)
+    q_order, kv_order = [2, 3, 0, 1], [1, 0]   # the two groups change places
+    W2 = dict(W)
+    W2[f"{p}.q_proj.weight"] = heads(W[f"{p}.q_proj.weight"], nq, q_order)
+    W2[f"{p}.k_proj.weight"] = heads(W[f"{p}.k_proj.weight"], nkv, kv_order)
+    W2[f"{p}.v_proj.weight"] = heads(W[f"{p}.v_proj.weight"], nkv, kv_order)
+    W2[f"{p}.o_proj.weight"] = heads(W[f"{p}.o_proj.weight"].T.contiguous(), nq, q_order).T
+    assert torch.allclose(plain.attention_block(x, W2, p, c, positions, cos, sin, None), base, atol=1e-12)
+    # within a group the query heads may change places too, the kv heads staying
+    W3 = dict(W)
+    W3[f"{p}.q_proj.weight"] = heads(W[f"{p}.q_proj.weight"], nq, [1, 0, 2, 3])
+    W3[f"{p}.o_proj.weight"] = heads(W[f"{p}.o_proj.weight"].T.contiguous(), nq, [1, 0, 2, 3]).T
+    assert torch.allclose(plain.attention_block(x, W3, p, c, positions, cos, sin, None), base, atol=1e-12)
+
+    W4 = dict(W)
+    wq = W[f"{p}.q_proj.weight"].clone()
+    wq[d:2 * d] *= 7.0                          # query head 1 alone
+    wk = W[f"{p}.k_proj.weight"].clone()
+    wk[:d] *= 0.2                               # kv head 0 alone
+    W4[f"{p}.q_proj.weight"], W4[f"{p}.k_proj.weight"] = wq, wk
+    assert torch.allclose(plain.attention_block(x, W4, p, c, positions, cos, sin, None), base, atol=1e-10)
+    # ... while the same constant on v does change the output: the norm is on q and k alone
+    W5 = dict(W)
+    W5[f"{p}.v_proj.weight"] = W[f"{p}.v_proj.weight"] * 2.0
+    assert not torch.allclose(plain.attention_block(x, W5, p, c, positions, cos, sin, None), base, atol=1e-3)
+
+
+def test_qk_norm_runs_before_the_rotation_and_adds_no_one(tmp_path):
+    """The block must equal its parts put together in the reference's order: projections, per-head
+    norm with the plain weight (no 1 + w: qk_norm_add_one is false for Qwen3, attention.rs:491),
+    rotation (attention.rs:868-879, after prepare_qk_for_rope), attention, o_proj.  With weights that
+    differ within a rotation pair the other order (rotate, then norm) gives another result, and
+    so does 1 + w."""
+    c, W, p, x, positions, cos, sin = _attention_inputs(tmp_path)
+    T, nq, nkv, d, eps = x.shape[0], c["num_attention_heads"], c["num_key_value_heads"], c["head_dim"], c["rms_norm_eps"]
+    q = (x @ W[f"{p}.q_proj.weight"].T).reshape(T, nq, d)
+    k = (x @ W[f"{p}.k_proj.weight"].T).reshape(T, nkv, d)
+    v = (x @ W[f"{p}.v_proj.weight"].T).reshape(T, nkv, d)
+    wq, wk = W[f"{p}.q_norm.weight"], W[f"{p}.k_norm.weight"]
+    rope = lambda t: plain.apply_rope(t, positions, cos, sin)
+    out = lambda qq, kk: plain.attention(qq, kk, v).reshape(T, nq * d) @ W[f"{p}.o_proj.weight"].T
+    norm_then_rotate = out(rope(plain.rms_norm(q, wq, eps)), rope(plain.rms_norm(k, wk, eps)))
+    rotate_then_norm = out(plain.rms_norm(rope(q), wq, eps), plain.rms_norm(rope(k), wk, eps))
+    plus_one = out(rope(plain.rms_norm(q, 1.0 + wq, eps)), rope(plain.rms_norm(k, 1.0 + wk, eps)))
+    no_norm = out(rope(q), rope(k))
+    got = plain.attention_block(x, W, p, c, positions, cos, sin, None)
+    assert torch.allclose(got, norm_then_rotate, atol=1e-13)
+    scale = float(got.abs().max())
+    for other in (rotate_then_norm, plus_one, no_norm):
+        assert float((got - other).abs().max()) > 1e-2 * scale
+    # the sum of squares of a row survives the rotation, so with a constant weight the two orders agree:
+    # only the place of the weight tells them apart
+    ones = torch.ones(d, dtype=torch.float64)
+    assert torch.allclose(rope(plain.rms_norm(q, ones, eps)), plain.rms_norm(rope(q), ones, eps), atol=1e-12)
+
+
+def test_embedding_is_not_scaled(tmp_path):
+    """x = E[ids] goes into the stream as it is (/root/reference/src/models/qwen3.rs:302-309): a
+    one-layer model's logits equal the parts put together on the bare table rows, and a table
+    multiplied by a constant (what a hidden sqrt(hidden_size) would amount to) gives other logits:
+    the first norm removes the scale from the branches, but not from the residual path."""
+    pm = _tiny_weights("B", tmp_path)                          # untied head
+    c = dict(pm.config, num_hidden_layers=1)
+    W = pm.weights
+    ids = [4, 99, 310, 7, 250]
+    cos, sin = plain.rope_tables(float(c["rope_theta"]), c["head_dim"], c["max_position_embeddings"])
+    x = W["model.embed_tokens.weight"][torch.tensor(ids)]
+    y = plain.decoder_layer(x, W, 0, c, torch.arange(len(ids)), cos.double(), sin.double())
+    want = plain.rms_norm(y, W["model.norm.weight"], c["rms_norm_eps"]) @ W["lm_head.weight"].T
+    got = plain.model_logits(c, W, ids)
+    assert torch.allclose(got.double(), want, atol=1e-5)
+    for factor in (math.sqrt(c["hidden_size"]), 1.0 / math.sqrt(c["hidden_size"])):
+        W2 = dict(W)
+        W2["model.embed_tokens.weight"] = W["model.embed_tokens.weight"] * factor
+        other = plain.model_logits(c, W2, ids)
+        assert float((other - got).abs().max()) > 1e-2 * float(got.abs().max())
