@@ -144,17 +144,60 @@ def test_one_error_lists_everything_wrong(tmp_path):
         assert needle in text
 
 
-def test_tied_model_must_not_carry_a_head(tmp_path):
+def test_tensors_nobody_asks_for_are_ignored(tmp_path, capfd):
+    """The reference reads by name and never looks at the rest: a tied checkpoint that also stores
+    lm_head.weight, or an old export's rotary_emb.inv_freq, loads, and the head is the embedding
+    table (/root/reference/src/models/qwen3.rs:267-287).  `check` returns the ignored names and the
+    loader says so once."""
+    from xinfer_amd.engine.loading import build_model
     d = write_random_model(str(tmp_path / "m"), TINY["A"]["config"], seed=0)
     st = SafetensorsStore(d)
     assert "lm_head.weight" not in st.names()
     tensors = {n: st.get(n) for n in st.names()}
-    tensors["lm_head.weight"] = tensors["model.embed_tokens.weight"].clone()
+    tensors["lm_head.weight"] = torch.full_like(tensors["model.embed_tokens.weight"], 3.0)    # not the table's values
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(16)
+    extra = tmp_path / "extra"
+    extra.mkdir()
+    write_safetensors(str(extra / "model.safetensors"), tensors.items())
+    store = SafetensorsStore(str(extra))
+    assert store.check(_decls("A")) == ["lm_head.weight", "model.layers.0.self_attn.rotary_emb.inv_freq"]
+    _, cfg = config_from_dict(TINY["A"]["config"])
+    model = build_model(cfg, store, "f32", device="cpu")
+    assert model.ignored_tensors == ["lm_head.weight", "model.layers.0.self_attn.rotary_emb.inv_freq"]
+    assert model.head.tied and model.head.proj.weight.data_ptr() == model.embedding.table.data_ptr()
+    assert "2 tensors the model does not use are ignored" in capfd.readouterr().err
+    # a missing tensor is still the one error, and it lists the ignored ones beside it
+    del tensors["model.norm.weight"]
     bad = tmp_path / "bad"
     bad.mkdir()
     write_safetensors(str(bad / "model.safetensors"), tensors.items())
-    with pytest.raises(WeightError, match="unexpected"):
+    with pytest.raises(WeightError) as e:
         SafetensorsStore(str(bad)).check(_decls("A"))
+    assert e.value.missing == ["model.norm.weight"] and "lm_head.weight" in e.value.unexpected
+
+
+def test_checkpoint_without_the_model_prefix_is_tied(tmp_path):
+    """A checkpoint that holds embed_tokens.weight without the `model.` prefix: every tensor is read
+    without the prefix and the head is the table, whatever config.json says about tying
+    (/root/reference/src/models/qwen3.rs:200-209)."""
+    from xinfer_amd.engine.loading import build_model
+    raw = dict(TINY["B"]["config"])
+    assert raw["tie_word_embeddings"] is False
+    d = write_random_model(str(tmp_path / "m"), raw, seed=1)
+    st = SafetensorsStore(d)
+    tensors = {n[len("model."):]: st.get(n) for n in st.names() if n.startswith("model.")}
+    bare = tmp_path / "bare"
+    bare.mkdir()
+    write_safetensors(str(bare / "model.safetensors"), tensors.items())
+    _, cfg = config_from_dict(raw)
+    store = SafetensorsStore(str(bare))
+    model = build_model(cfg, store, "f32", device="cpu")
+    assert model.spec.layers[0].prefix == "layers.0" and model.head.tied and model.ignored_tensors == []
+    assert torch.equal(model.embedding.table, tensors["embed_tokens.weight"].float())
+    assert model.head.proj.weight.data_ptr() == model.embedding.table.data_ptr()
+    assert torch.equal(model.final_norm.weight, tensors["norm.weight"].float())
+    # with the prefix the same config is untied
+    assert not build_model(cfg, st, "f32", device="cpu").head.tied
 
 
 def test_storage_policy(tmp_path):

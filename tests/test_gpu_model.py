@@ -206,3 +206,48 @@ def test_mixed_step_with_long_contexts_both_attention_paths(real_model_dirs):
     runner.step([StepEntry(0, prompts[0], [])])
     alone = runner.step([StepEntry(0, [nxt[0]], [0])]).float().cpu()
     assert float((alone[0] - split[0]).abs().max()) < harness.TOL["bfloat16"] * scale
+
+
+def test_extra_tensors_and_a_checkpoint_without_prefix_give_the_same_logits(model_dirs, tmp_path):
+    """A tied checkpoint that also stores an lm_head.weight (of other values) and a stray buffer
+    gives the logits of the checkpoint without them: the head is the table.  A checkpoint whose
+    names lack the `model.` prefix is read without it and tied (qwen3.rs:200-209): it gives the
+    logits of the same tensors under the usual names with tie_word_embeddings set."""
+    import json
+    import shutil
+    from xinfer_amd.engine import ModelRunner, StepEntry, load_model
+    from xinfer_amd.weights import SafetensorsStore, write_safetensors
+    toks = harness.random_prompt(random.Random(3), 40, 256)
+
+    def logits(folder, page):
+        runner = ModelRunner(load_model(folder, "float32", "cuda:0"), page_size=page, num_pages=8, max_requests=1)
+        runner.add_request(0)
+        return runner.step([StepEntry(0, toks, list(range(len(toks))))]).cpu()
+
+    st = SafetensorsStore(model_dirs["A"])
+    tensors = {n: st.get(n) for n in st.names()}
+    tensors["lm_head.weight"] = torch.full_like(tensors["model.embed_tokens.weight"], 0.5)
+    tensors["model.layers.1.self_attn.rotary_emb.inv_freq"] = torch.ones(16)
+    extra = tmp_path / "extra"
+    extra.mkdir()
+    shutil.copy(model_dirs["A"] + "/config.json", extra / "config.json")
+    write_safetensors(str(extra / "model.safetensors"), tensors.items())
+    base = logits(model_dirs["A"], 16)
+    assert torch.equal(logits(str(extra), 16), base)
+    ref = plain.PlainModel(model_dirs["A"]).logits(toks)
+    assert float((base - ref).abs().max()) < harness.TOL["float32"] * float(ref.abs().max())
+
+    st = SafetensorsStore(model_dirs["B"])
+    named = {n: st.get(n) for n in st.names() if n.startswith("model.")}
+    with open(model_dirs["B"] + "/config.json") as f:
+        raw = json.load(f)
+    bare, tied = tmp_path / "bare", tmp_path / "tied"
+    for folder, tens, cfg in ((bare, {n[len("model."):]: t for n, t in named.items()}, raw),
+                              (tied, named, dict(raw, tie_word_embeddings=True))):
+        folder.mkdir()
+        (folder / "config.json").write_text(json.dumps(cfg))
+        write_safetensors(str(folder / "model.safetensors"), tens.items())
+    toks = [t % 509 for t in toks]
+    assert torch.equal(logits(str(bare), 8), logits(str(tied), 8))
+    ref = plain.PlainModel(str(tied)).logits(toks)
+    assert float((logits(str(bare), 8) - ref).abs().max()) < harness.TOL["float32"] * float(ref.abs().max())

@@ -37,6 +37,6 @@ def load_model(model_dir: str, dtype, device="cuda:0") -> CausalLM:
 
 def build_model(config, store: WeightStore, dtype, device="cuda:0") -> CausalLM:
     fam = family_of(config.architecture)
-    model = CausalLM(fam.build_spec(config), parse_dtype(dtype))
+    model = CausalLM(fam.spec(config, store.names()), parse_dtype(dtype))
     model.config = config
     return model.load(store, device)

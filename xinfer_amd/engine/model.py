@@ -8,6 +8,7 @@ rows may be asked for.
 """
 from __future__ import annotations
 
+import sys
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Tuple
 
@@ -64,7 +65,12 @@ class CausalLM:
         return out
 
     def load(self, store: WeightStore, device) -> "CausalLM":
-        store.check(self.declare(self.spec))
+        # tensors of the source that no part asked for are left alone, as the reference leaves them
+        self.ignored_tensors = store.check(self.declare(self.spec))
+        if self.ignored_tensors:
+            shown = ", ".join(self.ignored_tensors[:4]) + (", ..." if len(self.ignored_tensors) > 4 else "")
+            print(f"[xinfer_amd] {store.where}: {len(self.ignored_tensors)} tensors the model does not use "
+                  f"are ignored ({shown})", file=sys.stderr, flush=True)
         self.device = torch.device(device)
         self.embedding.load(store, "", device)
         for b in self.blocks:

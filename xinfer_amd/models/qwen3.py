@@ -11,13 +11,24 @@ from ..config.spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
 from .registry import ModelFamily, register_architecture
 
 
-def qwen3_spec(cfg: Qwen3Config) -> ModelSpec:
+def qwen3_spec_for(cfg: Qwen3Config, tensor_names) -> ModelSpec:
+    """A checkpoint that holds `embed_tokens.weight` without the `model.` prefix has no prefix
+    anywhere and no head of its own: the reference then reads every tensor without the prefix
+    and ties the head to the table (embedding checkpoints, qwen3.rs:200-209)."""
+    names = set(tensor_names)
+    if "embed_tokens.weight" in names and "model.embed_tokens.weight" not in names:
+        return qwen3_spec(cfg, prefix="", tied=True)
+    return qwen3_spec(cfg)
+
+
+def qwen3_spec(cfg: Qwen3Config, prefix: str = "model.", tied=None) -> ModelSpec:
+    tied = cfg.tie_word_embeddings if tied is None else bool(tied)
     rope = PartSpec("rope", dict(
         head_dim=cfg.head_dim, rotary_dim=cfg.head_dim, theta=cfg.rope_theta,
         max_positions=cfg.max_position_embeddings, interleaved=False))
     layers = []
     for i in range(cfg.num_hidden_layers):
-        prefix = f"model.layers.{i}"
+        layer_prefix = f"{prefix}layers.{i}"
         mixer = PartSpec("attention", dict(
             hidden_size=cfg.hidden_size, num_heads=cfg.num_attention_heads,
             num_kv_heads=cfg.num_key_value_heads, head_dim=cfg.head_dim,
@@ -29,7 +40,7 @@ def qwen3_spec(cfg: Qwen3Config) -> ModelSpec:
             activation=cfg.hidden_act))
         norm = PartSpec("rmsnorm", dict(dim=cfg.hidden_size, eps=cfg.rms_norm_eps))
         layers.append(LayerSpec(
-            prefix=prefix, block="prenorm", mixer=mixer, feed_forward=ffn,
+            prefix=layer_prefix, block="prenorm", mixer=mixer, feed_forward=ffn,
             norms={"input_layernorm": norm, "post_attention_layernorm": norm}))
     return ModelSpec(
         architecture=cfg.architecture,
@@ -37,19 +48,19 @@ def qwen3_spec(cfg: Qwen3Config) -> ModelSpec:
         hidden_size=cfg.hidden_size,
         max_positions=cfg.max_position_embeddings,
         embedding=PartSpec("embedding", dict(
-            name="model.embed_tokens.weight", vocab_size=cfg.vocab_size, dim=cfg.hidden_size)),
+            name=f"{prefix}embed_tokens.weight", vocab_size=cfg.vocab_size, dim=cfg.hidden_size)),
         layers=tuple(layers),
         schedule=tuple(ScheduleEntry(i) for i in range(cfg.num_hidden_layers)),
         final_norm=PartSpec("rmsnorm", dict(
-            dim=cfg.hidden_size, eps=cfg.rms_norm_eps, name="model.norm.weight")),
+            dim=cfg.hidden_size, eps=cfg.rms_norm_eps, name=f"{prefix}norm.weight")),
         head=PartSpec("lm_head", dict(
-            name="model.embed_tokens.weight" if cfg.tie_word_embeddings else "lm_head.weight",
-            tied=cfg.tie_word_embeddings, vocab_size=cfg.vocab_size, dim=cfg.hidden_size)),
+            name=f"{prefix}embed_tokens.weight" if tied else "lm_head.weight",
+            tied=tied, vocab_size=cfg.vocab_size, dim=cfg.hidden_size)),
         eos_token_ids=tuple(cfg.eos_token_id or ()),
     )
 
 
-QWEN3 = ModelFamily("qwen3", Qwen3Config, qwen3_spec)
+QWEN3 = ModelFamily("qwen3", Qwen3Config, qwen3_spec, qwen3_spec_for)
 # The reference maps all of these names to ModelType::Qwen3 (utils/mod.rs:2357-2365);
 # only the Qwen3 name is registered here because Qwen2 differs (bias, no q/k norm).
 register_architecture("Qwen3ForCausalLM", QWEN3)

@@ -9,7 +9,7 @@ everything after that is architecture-neutral.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Callable, Dict
+from typing import Any, Callable, Dict, Optional, Sequence
 
 from ..config.model_config import ConfigError, architecture_name, read_config_json
 from ..config.spec import ModelSpec
@@ -20,6 +20,14 @@ class ModelFamily:
     name: str
     config_class: Any                       # has from_dict(raw, where) and to_dict()
     build_spec: Callable[[Any], ModelSpec]  # typed config -> ModelSpec
+    # (typed config, names of the tensors a checkpoint holds) -> ModelSpec, for a family whose
+    # checkpoints come in more than one naming; None: `build_spec` whatever the names
+    build_spec_for: Optional[Callable[[Any, Sequence[str]], ModelSpec]] = None
+
+    def spec(self, config, tensor_names: Optional[Sequence[str]] = None) -> ModelSpec:
+        if tensor_names is not None and self.build_spec_for is not None:
+            return self.build_spec_for(config, tensor_names)
+        return self.build_spec(config)
 
 
 _FAMILIES: Dict[str, ModelFamily] = {}

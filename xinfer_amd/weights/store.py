@@ -4,9 +4,14 @@ A `WeightStore` answers `get(name)` for every tensor of a model.  Two sources ex
 the safetensors files of a model folder, and seeded random values.  Parts declare the
 tensors they need (`TensorDecl`), the model collects the declarations, and `check`
 compares them with what the source holds before anything is loaded, so that a broken
-checkpoint produces one error that lists every missing, unexpected and mis-shaped
-tensor (the reference surfaces these one at a time as candle errors,
-/root/reference/src/models/layers/mod.rs:170-194).
+checkpoint produces one error that lists every missing and mis-shaped tensor, and beside
+them the tensors the model did not ask for (a misnamed tensor shows up as one of each);
+the reference surfaces these one at a time as candle errors
+(/root/reference/src/models/layers/mod.rs:170-194).  Tensors the model does not ask for
+are no error by themselves: the reference reads by name and never looks at the rest (a
+tied checkpoint that also stores lm_head.weight, an old export's rotary_emb.inv_freq;
+/root/reference/src/models/qwen3.rs:267-287), so `check` returns their names and the
+loader says once that it leaves them alone.
 
 Storage policy: floating tensors are kept in bfloat16, except that a tensor stored in
 32 bits stays in 32 bits; integer tensors become int32.  Parts ask for the compute
@@ -27,7 +32,8 @@ from .safetensors_io import SafetensorsFile
 
 
 class WeightError(RuntimeError):
-    """One error for everything that is wrong with a checkpoint."""
+    """One error for everything that is wrong with a checkpoint: missing tensors and wrong
+    shapes; the tensors nobody asked for are listed with them."""
 
     def __init__(self, where: str, missing: Sequence[str], unexpected: Sequence[str],
                  wrong_shape: Sequence[Tuple[str, Tuple[int, ...], Tuple[int, ...]]]):
@@ -39,7 +45,7 @@ class WeightError(RuntimeError):
             lines.append(f"  missing tensors ({len(self.missing)}):")
             lines += [f"    {n}" for n in self.missing]
         if self.unexpected:
-            lines.append(f"  unexpected tensors ({len(self.unexpected)}):")
+            lines.append(f"  unexpected tensors, which the model does not use ({len(self.unexpected)}):")
             lines += [f"    {n}" for n in self.unexpected]
         if self.wrong_shape:
             lines.append(f"  wrong shapes ({len(self.wrong_shape)}):")
@@ -90,7 +96,9 @@ class WeightStore:
         want = dtype if dtype is not None else _storage_dtype(t.dtype)
         return t.to(device=device, dtype=want)
 
-    def check(self, decls: Iterable[TensorDecl]) -> None:
+    def check(self, decls: Iterable[TensorDecl]) -> List[str]:
+        """Raises one `WeightError` if a declared tensor is missing or has another shape.
+        Returns the names of the tensors that no declaration asks for."""
         decls = list(decls)
         have = set(self.names())
         want: Dict[str, Tuple[int, ...]] = {}
@@ -100,8 +108,9 @@ class WeightStore:
         unexpected = sorted(n for n in have if n not in want)
         wrong = sorted((n, self.shape(n), s) for n, s in want.items()
                        if n in have and tuple(self.shape(n)) != tuple(s))
-        if missing or unexpected or wrong:
+        if missing or wrong:
             raise WeightError(self.where, missing, unexpected, wrong)
+        return unexpected
 
 
 class SafetensorsStore(WeightStore):
