@@ -189,6 +189,35 @@ def test_eos_and_limits(model_dirs):
         eng.generate([[1] * 40], SamplingParams(max_tokens=2))
 
 
+def test_eos_ids_of_config_and_generation_config_both_stop(model_dirs, tmp_path):
+    """config.json names one end-of-sequence id and generation_config.json a list with another:
+    the engine stops on either (Config::apply_generation_cfg, /root/reference/src/utils/config.rs:360-375)."""
+    import json
+    import shutil
+    from xinfer_amd import SamplingParams
+    prompts = [[1, 2, 3, 4, 5], [9, 8, 7]]
+    free = _engine(model_dirs["A"], "A", "f32", max_num_seqs=2, num_pages=16).generate(
+        prompts, SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))
+    a, b = free[0].token_ids[5], free[1].token_ids[3]
+    assert a not in free[1].token_ids[:4] and b not in free[0].token_ids[:6] and a != b
+    d = tmp_path / "with_eos"
+    shutil.copytree(model_dirs["A"], d)
+    with open(d / "config.json") as f:
+        raw = json.load(f)
+    raw["eos_token_id"] = a
+    (d / "config.json").write_text(json.dumps(raw))
+    (d / "generation_config.json").write_text(json.dumps({"eos_token_id": [b, 255], "temperature": 0.6, "top_k": 20}))
+    eng = _engine(str(d), "A", "f32", max_num_seqs=2, num_pages=16)
+    assert eng.eos_token_ids == {a, b, 255}
+    assert (eng.generation_cfg.temperature, eng.generation_cfg.top_k) == (0.6, 20)
+    out = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12))
+    assert out[0].token_ids == free[0].token_ids[:free[0].token_ids.index(a)] and out[0].finish_reason == "eos"
+    assert out[1].token_ids == free[1].token_ids[:free[1].token_ids.index(b)] and out[1].finish_reason == "eos"
+    # one id instead of a list
+    (d / "generation_config.json").write_text(json.dumps({"eos_token_id": b}))
+    assert _engine(str(d), "A", "f32", max_num_seqs=2, num_pages=16).eos_token_ids == {a, b}
+
+
 # ---- streaming -----------------------------------------------------------------------------------
 def test_streams_interleave_and_cancel(model_dirs):
     """Two streams read in turn give the tokens `generate` gives; a cancelled stream gives its
@@ -415,6 +444,90 @@ def test_a_batch_size_is_recorded_the_third_time_it_is_seen(model_dirs):
     runner.release(1)
     runner.step([StepEntry(0, [9], [0])])                      # another batch size: first sighting
     assert (len(runner._graphs), runner.graph_replays) == (1, 3)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_graphs_across_a_bucket_edge(dtype, tmp_path):
+    """A request grows from 1,021 to 1,030 keys: the steps up to 1,024 replay the graph of the
+    1,024 bucket, the later ones that of 2,048 (whose attention grid is laid out for 2,048 keys).
+    Every replayed step against the same step launched kernel by kernel, bit for bit, stopping at
+    the first difference, and against the plain model."""
+    from xinfer_amd.engine import ModelRunner, StepEntry, load_model
+    from xinfer_amd.weights import write_random_model
+    t = TINY["B"]
+    cfg = dict(t["config"], max_position_embeddings=2048)
+    d = write_random_model(str(tmp_path / "b2048"), cfg, t["seed"], t["linear_std"], t["norm_std"])
+    vocab, page = cfg["vocab_size"], t["page_size"]
+    model = load_model(d, dtype, DEV)
+    rng = random.Random(5)
+    long = harness.random_prompt(rng, 1030, vocab)
+    short = harness.random_prompt(rng, 40, vocab)
+
+    def run(use_graphs):
+        runner = ModelRunner(model, page, 2048 // page + 8, 2, use_graphs=use_graphs, graph_after=1)
+        runner.add_request(0)
+        runner.add_request(1)
+        runner.step([StepEntry(0, long[:1020], []), StepEntry(1, short[:30], [])])
+        out = [runner.step([StepEntry(0, [long[1020 + k]], [0]), StepEntry(1, [short[30 + k]], [0])]).cpu() for k in range(10)]
+        return out, runner
+
+    want, _ = run(False)
+    got, runner = run(True)
+    assert sorted(runner._graphs) == [(2, 1024, False), (2, 2048, False)] and runner.graph_replays == 10
+    for k, (a, b) in enumerate(zip(want, got)):
+        assert torch.equal(a, b), f"the step that makes {1021 + k} keys differs between graph and launches"
+    ref = plain.PlainModel(d).logits(long)
+    scale = float(ref.abs().max())
+    for k, a in enumerate(got):
+        assert float((a[0] - ref[1020 + k]).abs().max()) < harness.TOL[dtype] * scale, 1021 + k
+
+
+def test_recorded_graphs_are_bounded(model_dirs):
+    """With room for two graphs the least recently used one goes when a third is recorded; its
+    batch size is recorded again when it comes back, and the logits stay those of launched steps."""
+    from xinfer_amd.engine import ModelRunner, StepEntry, load_model
+    model = load_model(model_dirs["A"], "bfloat16", DEV)
+
+    def run(**kw):
+        runner = ModelRunner(model, 16, 12, 3, graph_after=1, **kw)
+        out = []
+        for i in range(3):
+            runner.add_request(i)
+        for step, live in enumerate([[0], [0], [0, 1], [0], [0, 1, 2], [0, 1, 2], [0, 1], [0, 1]]):
+            out.append(runner.step([StepEntry(i, [step + 3 * i], [0]) for i in live]).cpu())
+        return out, runner
+
+    want, _ = run(use_graphs=False)
+    got, runner = run(graphs_most=2)
+    assert all(torch.equal(a, b) for a, b in zip(want, got))
+    # sizes 1, 2 recorded; 1 used again; 3 recorded: 2 goes; 2 recorded again: 1 goes
+    assert [k[0] for k in runner._graphs] == [3, 2] and runner.graphs_dropped == 2 and runner.graph_replays == 8
+    got, runner = run(graph_bytes_most=1)          # no room beyond the graph in use
+    assert all(torch.equal(a, b) for a, b in zip(want, got))
+    assert len(runner._graphs) == 1 and runner.graphs_dropped == 4
+
+
+def test_sizes_the_decode_kernel_does_not_take_are_not_recorded(tmp_path):
+    """32 query heads on one kv head: the split-K decode kernel takes up to 16 per kv head, so the
+    prefill kernel serves single tokens too, and it reads the step's lengths on the host: the model
+    says so and its steps are launched one by one, many times over."""
+    from xinfer_amd.engine import ModelRunner, StepEntry, load_model
+    from xinfer_amd.weights import write_random_model
+    cfg = dict(TINY["B"]["config"], num_attention_heads=32, num_key_value_heads=1, head_dim=16, hidden_size=64,
+               num_hidden_layers=1)
+    d = write_random_model(str(tmp_path / "g32"), cfg, 3, 0.05, 0.1)
+    model = load_model(d, "bfloat16", DEV)
+    assert not model.graph_safe and load_model(d, "float32", DEV).graph_safe
+    runner = ModelRunner(model, 8, 16, 2, graph_after=2)
+    assert not runner.use_graphs
+    toks = harness.random_prompt(random.Random(1), 30, cfg["vocab_size"])
+    runner.add_request(0)
+    got = [runner.step([StepEntry(0, toks[:20], [19])]).cpu()[0]]
+    got += [runner.step([StepEntry(0, [toks[20 + k]], [0])]).cpu()[0] for k in range(10)]
+    ref = plain.PlainModel(d).logits(toks)
+    for k, a in enumerate(got):
+        assert float((a - ref[19 + k]).abs().max()) < harness.TOL["bfloat16"] * float(ref.abs().max())
+    assert runner.graph_replays == 0
 
 
 def test_model_with_a_part_that_reads_the_host_is_not_recorded(model_dirs):

@@ -9,7 +9,7 @@ prefix cache, server, speculative decoding) are absent rather than accepted and 
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import List, Optional
+from typing import List, Optional, Tuple
 
 
 @dataclass
@@ -21,6 +21,7 @@ class GenerationConfig:
     top_k: Optional[int] = None
     frequency_penalty: Optional[float] = None
     presence_penalty: Optional[float] = None
+    eos_token_id: Tuple[int, ...] = ()     # one id or a list in the file; joined with config.json's (config.rs:360-375)
 
 
 @dataclass

@@ -19,11 +19,13 @@ import torch
 from ..config.engine_config import (EngineConfig, GenerationConfig, GenerationOutput, Message, SamplingParams,
                                     StreamItem)
 from ..sampling import Sampler, Strategy, resolve_strategy, uniform
-from ..sampling.sampler import PENALTY_CONTEXT
+from ..sampling.sampler import penalty_context
+from ..config.model_config import ConfigError
+from ..models import family_of
 from .loading import load_model, parse_dtype
 from .runner import ModelRunner, StepEntry
 from .scheduler import RequestTooLarge, Scheduler
-from .tokenizer import load_tokenizer
+from .tokenizer import IncrementalText, load_tokenizer
 
 DEFAULT_MAX_TOKENS = 16384      # /root/reference/src/core/engine.rs:650-678
 
@@ -69,9 +71,17 @@ class LLMEngine:
             self.dtype = model.dtype
         spec = self.model.spec
         self.max_model_len = min(econfig.max_model_len or spec.max_positions, spec.max_positions)
-        self.tokenizer = load_tokenizer(model_dir, spec.vocab_size)
-        self.eos_token_ids = set(spec.eos_token_ids) | set(self.tokenizer.eos_token_ids())
+        try:
+            default_template = family_of(spec.architecture).chat_template
+        except ConfigError:                # a model put together by hand, of no registered family
+            default_template = None
+        self.tokenizer = load_tokenizer(model_dir, spec.vocab_size, default_template)
         self.generation_cfg = econfig.generation_cfg or (_read_generation_config(model_dir) if model_dir else None)
+        # config.json's end-of-sequence ids and generation_config.json's together
+        # (Config::apply_generation_cfg, /root/reference/src/utils/config.rs:360-375), and the tokenizer's
+        self.eos_token_ids = set(spec.eos_token_ids) | set(self.tokenizer.eos_token_ids())
+        if self.generation_cfg is not None:
+            self.eos_token_ids |= set(self.generation_cfg.eos_token_id or ())
         self.seed = econfig.seed if econfig.seed is not None else int.from_bytes(os.urandom(4), "little")
         page = econfig.page_size
         num_pages = econfig.num_pages or self._plan_pages(page)
@@ -166,7 +176,7 @@ class LLMEngine:
             strategies = [r.strategy for r in sampled]
             recent = None
             if any(s.frequency_penalty or s.presence_penalty for s in strategies):
-                recent = [r.tokens[max(r.prompt_len, len(r.tokens) - PENALTY_CONTEXT):] for r in sampled]
+                recent = [penalty_context(r.tokens, r.prompt_len) for r in sampled]
             tokens = self.sampler.sample(
                 logits, strategies,
                 [0.0 if r.strategy.greedy else uniform(r.seed, r.stream, len(r.tokens) - r.prompt_len) for r in sampled],
@@ -217,9 +227,14 @@ class LLMEngine:
         if len(params) != len(prompts):
             raise ValueError("one SamplingParams per prompt is needed")
         rids = []
-        for p, sp in zip(prompts, params):
-            ids = self.tokenizer.encode(p) if isinstance(p, str) else list(p)
-            rids.append(self.add_request(ids, sp))
+        try:
+            for p, sp in zip(prompts, params):
+                ids = self.tokenizer.encode(p) if isinstance(p, str) else list(p)
+                rids.append(self.add_request(ids, sp))
+        except Exception:
+            for rid in rids:               # a later prompt was refused: the earlier ones do not stay behind
+                self.cancel(rid)
+            raise
         self.run_until_done()
         return [self._output(self._finished.pop(rid)) for rid in rids]
 
@@ -242,6 +257,7 @@ class LLMEngine:
         /root/reference/src/core/scheduler.rs:780-818)."""
         r = self._requests.pop(rid, None)
         if r is None:
+            self._finished.pop(rid, None)      # finished and never collected: forgotten now
             return
         self.scheduler.finish(rid)
         r.finish_reason = "cancelled"
@@ -271,8 +287,10 @@ def _completes_a_stop(stops: List[List[int]], generated: Sequence[int], token: i
 class EngineStream:
     """Tokens of one request as they are generated (the reference's EngineStream,
     xinfer.pyi:182-189).  Iterating drives the engine: every step also advances whatever other
-    requests are live.  Each token comes as a TOKEN_ID item followed by a TOKEN item with its
-    text; the last item is DONE."""
+    requests are live.  Each token comes as a TOKEN_ID item followed by a TOKEN item with the text
+    it adds (empty while a character that spans several tokens is incomplete: the text is
+    decoded from all tokens so far and handed on up to where it is final); the last item is
+    DONE.  A stream that is dropped unread takes its request's record with it."""
 
     def __init__(self, engine: "LLMEngine", rid: int, prompt_length: int):
         self._engine = engine
@@ -281,12 +299,19 @@ class EngineStream:
         self.finished = False
         self.cancelled = False
         self._sent = 0
+        self._text = IncrementalText(engine.tokenizer)
         self._pending: List[StreamItem] = []
 
     def cancel(self) -> None:
         if not self.finished and not self.cancelled:
             self._engine.cancel(self.seq_id)
             self.cancelled = True
+
+    def __del__(self):
+        try:
+            self.cancel()
+        except Exception:
+            pass
 
     def __iter__(self):
         return self
@@ -304,7 +329,7 @@ class EngineStream:
             if self._sent < len(gen):
                 tok = gen[self._sent]
                 self._sent += 1
-                self._pending = [StreamItem("TOKEN", eng.tokenizer.decode([tok]))]
+                self._pending = [StreamItem("TOKEN", self._text.add(gen[:self._sent]))]
                 return StreamItem("TOKEN_ID", tok)
             if self.seq_id in eng._finished:
                 eng._finished.pop(self.seq_id)
@@ -321,5 +346,11 @@ def _read_generation_config(model_dir: str) -> Optional[GenerationConfig]:
         return None
     with open(path, "r", encoding="utf-8") as f:
         raw = json.load(f)
+    eos = raw.get("eos_token_id")
+    if eos is None:
+        eos = ()
+    elif isinstance(eos, int):
+        eos = (eos,)
     return GenerationConfig(raw.get("temperature"), raw.get("top_p"), raw.get("top_k"),
-                            raw.get("frequency_penalty"), raw.get("presence_penalty"))
+                            raw.get("frequency_penalty"), raw.get("presence_penalty"),
+                            eos_token_id=tuple(int(t) for t in eos))

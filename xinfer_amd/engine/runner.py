@@ -109,10 +109,20 @@ class _DecodeGraph:
     keep: Tuple[Any, ...] = ()      # everything else the recorded kernels read: it must stay
                                     # allocated for as long as the graph may be replayed
 
+    @property
+    def nbytes(self) -> int:
+        """What the graph holds for itself between replays: its logits and its index arrays."""
+        return sum(t.numel() * t.element_size() for t in (self.dev32, self.dev64, self.logits))
+
+
+GRAPHS_MOST = 48                    # recorded decode graphs kept at a time, and
+GRAPH_BYTES_MOST = 1 << 30          # the bytes they may hold together; the least recently used goes first
+
 
 class ModelRunner:
     def __init__(self, model: CausalLM, page_size: int, num_pages, max_requests: int,
-                 use_graphs: bool = True, graph_max_batch: Optional[int] = None, graph_after: Optional[int] = None):
+                 use_graphs: bool = True, graph_max_batch: Optional[int] = None, graph_after: Optional[int] = None,
+                 graphs_most: int = GRAPHS_MOST, graph_bytes_most: int = GRAPH_BYTES_MOST):
         """`num_pages`: pages of every group's pool, or a list with one count per group.
         `use_graphs`: record decode steps of up to `graph_max_batch` requests as HIP graphs; a
         (batch size, context bucket) is recorded the `graph_after`-th time it is seen, so that
@@ -123,7 +133,10 @@ class ModelRunner:
         model, 0.1 to 0.2 ms a step for a large one, whose kernels outlast the launches.  Left to
         the runner, the count is 3 for a model whose step is bound by the host and 12 otherwise,
         and `graph_max_batch` 256 for such a model (its launches cost more than its kernels at
-        any batch size) and 64 otherwise."""
+        any batch size) and 64 otherwise.  At most `graphs_most` graphs holding `graph_bytes_most`
+        bytes (their logits, 39 MB at 64 rows of 151,936, and index arrays) are kept; beyond that
+        the least recently replayed one is dropped and its key starts counting sightings again
+        (the reference records batch sizes 1 to 32 once, /root/reference/src/utils/graph.rs:415-420)."""
         if not torch.cuda.is_available():
             raise RuntimeError("xinfer_amd runs on an AMD GPU only: no HIP device is visible")
         self.model = model
@@ -167,7 +180,10 @@ class ModelRunner:
             graph_max_batch = 256 if host_bound else 64
         self.graph_after = max(1, int(graph_after))
         self.graph_max_batch = int(graph_max_batch)
-        self._graphs: Dict[Tuple[int, int, bool], _DecodeGraph] = {}
+        self._graphs: Dict[Tuple[int, int, bool], _DecodeGraph] = {}     # in order of last use, oldest first
+        self.graphs_most = max(1, int(graphs_most))
+        self.graph_bytes_most = int(graph_bytes_most)
+        self.graphs_dropped = 0
         self._seen: Dict[Tuple[int, int, bool], int] = {}
         self._graph_pool = None
         # widest block table a request can have: the fixed width of a recorded step's tables
@@ -300,6 +316,7 @@ class ModelRunner:
         g = self._graphs.get((B, bucket, similar))
         if g is None:
             return None
+        self._used(g, (B, bucket, similar))
         self._staging.push(torch.int32, n32, g.dev32)
         self._staging.push(torch.int64, n64, g.dev64)
         self._staging.mark()
@@ -350,6 +367,24 @@ class ModelRunner:
         return d32, o32, d64, o64
 
     # ---- decode steps as HIP graphs ---------------------------------------------------
+    def _used(self, g: _DecodeGraph, key) -> None:
+        """Moves a graph to the young end of the order of last use."""
+        if next(reversed(self._graphs)) != key:
+            del self._graphs[key]
+            self._graphs[key] = g
+
+    def _drop_least_used(self, keep) -> None:
+        """Drops the least recently used graphs until count and bytes are within their bounds (the
+        one just recorded stays).  A dropped graph's memory goes back to the graphs' pool once its
+        last replay has finished."""
+        while len(self._graphs) > 1 and (len(self._graphs) > self.graphs_most
+                                         or sum(g.nbytes for g in self._graphs.values()) > self.graph_bytes_most):
+            key = next(k for k in self._graphs if k != keep)
+            torch.cuda.current_stream(self.device).synchronize()
+            del self._graphs[key]
+            self._seen.pop(key, None)
+            self.graphs_dropped += 1
+
     def _replay_decode(self, a: BatchArrays, ids32: np.ndarray, rows32: np.ndarray) -> torch.Tensor:
         """A step of single tokens.  The graph of (batch size, context bucket) computes the
         logits of every row; the wanted rows are gathered afterwards.  Kernels whose grid
@@ -385,7 +420,9 @@ class ModelRunner:
                 logits = self.model.forward(ids, ctx, self.layer_caches, every_row)
             g = _DecodeGraph(graph, d32, d64, logits, want, keep=(every_row, ctx, ids))
             self._graphs[key] = g
+            self._drop_least_used(keep=key)
         else:
+            self._used(g, key)
             self._upload(a, ids32, all_rows, g.dev32, g.dev64)
         g.graph.replay()
         self.graph_replays += 1

@@ -301,6 +301,14 @@ def mfma_attention_supported(nq: int, nkv: int, d: int, page: int) -> bool:
     return bool(lib().xi_attention_mfma_supported(nq, nkv, d, page))
 
 
+def decode_attention_takes(nq: int, nkv: int, d: int) -> bool:
+    """Whether the split-K decode kernel takes these head counts and this head size: up to 16 query
+    heads per kv head (the columns of one tile), and the waves' partial results of a group must
+    fit the LDS through which they are merged."""
+    g = nq // nkv
+    return g <= 16 and (4 * g * d + 8 * g) * 4 <= 64 * 1024
+
+
 def attention_prefill_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, scale, window=0, out=None,
                            small=False):
     """MFMA attention for any mix of portions.  tiles int32 [n, 2] = (sequence, first query
@@ -402,7 +410,7 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx
     bt = ctx.block_tables[group]
     if q.dtype == torch.bfloat16 and v_transposed and mfma_attention_supported(nq, nkv, d, page):
         g = nq // nkv
-        if ctx.max_q_len == 1 and g <= 16 and (4 * g * d + 8 * g) * 4 <= 64 * 1024:
+        if ctx.max_q_len == 1 and decode_attention_takes(nq, nkv, d):
             return attention_decode_bf16(q, k_cache, v_cache, bt, ctx.ctx_lens, ctx.max_ctx_len, scale, window,
                                          similar=getattr(ctx, "similar_lengths", False))
         key = ("attention_tiles", d, nq, nkv)
@@ -421,7 +429,7 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx
                 lead += 1
             lead_ctx = max(ctx.ctx_lens_host[:lead]) if lead else 0
             reads = g // (4 if g % 4 == 0 else 2 if g % 2 == 0 else 1)
-            if (lead < MIXED_DECODE_FROM or not (g <= 16 and (4 * g * d + 8 * g) * 4 <= 64 * 1024)
+            if (lead < MIXED_DECODE_FROM or not decode_attention_takes(nq, nkv, d)
                     or not (lead * lead_ctx * reads >= MIXED_DECODE_WORK or lead_ctx >= MIXED_DECODE_CONTEXT)):
                 lead = 0
             rows, small = prefill_tiles(q_lens, ctx.ctx_lens_host, d, nq, nkv, first_seq=lead)

@@ -60,7 +60,11 @@ def qwen3_spec(cfg: Qwen3Config, prefix: str = "model.", tied=None) -> ModelSpec
     )
 
 
-QWEN3 = ModelFamily("qwen3", Qwen3Config, qwen3_spec, qwen3_spec_for)
+# ChatML, the form Qwen3's own template reduces to for plain system/user/assistant turns
+CHATML = ("{% for message in messages %}<|im_start|>{{ message.role }}\n{{ message.content }}<|im_end|>\n{% endfor %}"
+          "{% if add_generation_prompt %}<|im_start|>assistant\n{% endif %}")
+
+QWEN3 = ModelFamily("qwen3", Qwen3Config, qwen3_spec, qwen3_spec_for, chat_template=CHATML)
 # The reference maps all of these names to ModelType::Qwen3 (utils/mod.rs:2357-2365);
 # only the Qwen3 name is registered here because Qwen2 differs (bias, no q/k norm).
 register_architecture("Qwen3ForCausalLM", QWEN3)

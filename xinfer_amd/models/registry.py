@@ -23,6 +23,8 @@ class ModelFamily:
     # (typed config, names of the tensors a checkpoint holds) -> ModelSpec, for a family whose
     # checkpoints come in more than one naming; None: `build_spec` whatever the names
     build_spec_for: Optional[Callable[[Any, Sequence[str]], ModelSpec]] = None
+    # the chat template (jinja) of a model folder whose tokenizer_config.json carries none
+    chat_template: Optional[str] = None
 
     def spec(self, config, tensor_names: Optional[Sequence[str]] = None) -> ModelSpec:
         if tensor_names is not None and self.build_spec_for is not None:

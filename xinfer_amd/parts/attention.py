@@ -24,7 +24,6 @@ from .linear import Linear
 @register_mixer("attention")
 class PagedAttention(Mixer):
     VECTOR_MIN_DECODE = 512      # decoded tokens lie in a page each: the form with one wave per head stays ahead up to here
-    graph_safe = True
 
     def __init__(self, spec: PartSpec, dtype: torch.dtype):
         super().__init__(spec, dtype)
@@ -39,6 +38,10 @@ class PagedAttention(Mixer):
         self.scale = float(spec.get("scale", self.d ** -0.5))
         if self.nq % self.nkv:
             raise ValueError(f"{self.nq} query heads are not a multiple of {self.nkv} kv heads")
+        # A step of single tokens reads nothing on the host where the split-K decode kernel or the
+        # generic kernel serves it; sizes that only the prefill kernel takes (more than 16 query heads
+        # per kv head) need the step's lengths on the host to lay out its tiles.
+        self.graph_safe = dtype != torch.bfloat16 or kernels.decode_attention_takes(self.nq, self.nkv, self.d)
         pos = spec.get("position")
         self.position = position_encoding_class(pos.kind)(pos, dtype) if pos is not None else None
         self.qkv: Optional[Linear] = None

@@ -7,7 +7,9 @@ top-k 32, top-p 0.95, temperature 0.7 (/root/reference/src/core/runner.rs:1803-1
 The reference picks one strategy per batch from its first sequence and draws from one
 shared generator; here every request has its own strategy and its own stream of random
 numbers (seed, request, number of tokens drawn so far), so a request's tokens do not
-depend on what it was batched with.
+depend on what it was batched with.  Frequency and presence penalties count what the
+reference counts (`penalty_context`, `penalties_apply`): the last 128 sampled tokens once
+more than 128 were sampled, never the prompt, and a penalty of exactly 1.0 counts as off.
 """
 from __future__ import annotations
 
@@ -22,7 +24,7 @@ from .. import kernels
 from ..config.engine_config import GenerationConfig, SamplingParams
 
 TOPK_FAST = 64             # largest top-k of the two-stage selection (`sampling_topk.hip`)
-PENALTY_CONTEXT = 128      # last generated tokens that penalties look at (runner.rs:1887-1912)
+PENALTY_CONTEXT = 128      # tokens that penalties look at (runner.rs:1887-1912)
 _MASK = (1 << 64) - 1
 
 
@@ -68,6 +70,26 @@ def resolve_strategy(params: SamplingParams, defaults: Optional[GenerationConfig
     return Strategy(s.temperature, s.top_k, s.top_p, float(freq or 0.0), float(pres or 0.0))
 
 
+def penalty_context(tokens: Sequence[int], prompt_len: int) -> List[int]:
+    """The tokens that frequency and presence penalties count for a request whose prompt and
+    generated tokens are `tokens`: the last PENALTY_CONTEXT of the tokens sampled so far (the
+    prompt is not among them: the reference's list holds what was sampled, runner.rs:1950-1962),
+    and none until more than PENALTY_CONTEXT have been sampled (runner.rs:1892-1897), so the
+    first token that penalties touch is the 130th generated one."""
+    generated = len(tokens) - prompt_len
+    if generated <= PENALTY_CONTEXT:
+        return []
+    return list(tokens[len(tokens) - PENALTY_CONTEXT:])
+
+
+def penalties_apply(strategy: Strategy, context: Sequence[int]) -> bool:
+    """Whether a row's penalties are applied (logits_processor.rs:399-401): more than one token
+    to count, and one of the two penalties neither 0 nor exactly 1 (the reference takes 1.0 for
+    "off" too); both values are then subtracted as they are."""
+    on = lambda v: v != 0.0 and v != 1.0
+    return len(context) > 1 and (on(strategy.frequency_penalty) or on(strategy.presence_penalty))
+
+
 def uniform(seed: int, request: int, draw: int) -> float:
     """The draw-th uniform number in [0, 1) of a request's stream: splitmix64 of the three
     counters, 24 bits kept so that the float32 value is exact."""
@@ -108,8 +130,8 @@ class Sampler:
     def sample(self, logits: torch.Tensor, strategies: Sequence[Strategy], uniforms: Sequence[float],
                recent: Optional[Sequence[Sequence[int]]] = None) -> List[int]:
         """logits float32 [R, V] (changed in place when penalties apply); one strategy and
-        one uniform number per row; `recent[r]` = the row's last generated tokens, for the
-        penalties.  Returns R token ids."""
+        one uniform number per row; `recent[r]` = the tokens the row's penalties count
+        (`penalty_context`).  Returns R token ids."""
         kernels._dev(logits)
         kernels._want(logits, torch.float32, "sample: logits")
         R, V = logits.shape
@@ -118,15 +140,14 @@ class Sampler:
         if R == 0:
             return []
         dev = logits.device
-        if recent is not None and any((s.frequency_penalty or s.presence_penalty) and len(rc) > 1
-                                      for s, rc in zip(strategies, recent)):
+        if recent is not None and any(penalties_apply(s, rc) for s, rc in zip(strategies, recent)):
             n = PENALTY_CONTEXT
             rec = np.full((R, n), -1, dtype=np.int32)
             fr = np.zeros(R, dtype=np.float32)
             pr = np.zeros(R, dtype=np.float32)
             for r, (s, rc) in enumerate(zip(strategies, recent)):
                 rc = list(rc)[-n:]
-                if len(rc) > 1:                      # logits_processor.rs:395
+                if penalties_apply(s, rc):
                     rec[r, :len(rc)] = rc
                     fr[r], pr[r] = s.frequency_penalty, s.presence_penalty
             rec_d, fr_d, pr_d = (torch.from_numpy(a).to(dev) for a in (rec, fr, pr))
