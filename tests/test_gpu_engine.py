@@ -737,6 +737,165 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
         harness.compare(run(steps), ref, harness.TOL["float32"], f"toy {what}")
 
 
+# ---- a toy mixer with one paged pool of its own, a scaled embedding, a head kind registered from here ----------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_one_pool_cache_scaled_embedding_and_a_head_kind(dtype, tmp_path):
+    """Data alone, beside part kinds registered here: (1) a mixer that keeps one pool of latent rows
+    (no keys and values: `KVNeed(window, (PoolNeed("latent", (PAGE, L), float32),))`) and answers
+    with the mean of the last `window` latents, read from the pages through the block table; (2)
+    the built-in embedding with a `scale`; (3) a head kind of its own (a bias, then the built-in soft
+    cap), registered from here; (4) tensor names of the layer's parts that are not the usual ones.
+    With an attention layer beside it the model has two cache groups of different pools.  Stepped
+    in every way of cutting with few pages, and generated from through the scheduler, whose window
+    group holds a window and a portion, not the whole request."""
+    from dataclasses import dataclass
+    from xinfer_amd import Engine, EngineConfig, SamplingParams, kernels
+    from xinfer_amd.config.spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+    from xinfer_amd.engine import ModelRunner, load_model
+    from xinfer_amd.models import ModelFamily, register_architecture
+    from xinfer_amd.parts import PAGE, KVNeed, Mixer, PoolNeed, register_head, register_mixer
+    from xinfer_amd.parts.embedding import LMHead
+    from xinfer_amd.weights import TensorDecl, write_random_model
+
+    H, L, WINDOW, V, SCALE, CAP = 48, 12, 11, 131, 7.0, 3.0
+
+    @register_mixer("latent_mean")
+    class LatentMean(Mixer):
+        def __init__(self, spec, dtype):
+            super().__init__(spec, dtype)
+            self.h, self.l, self.window = int(spec["hidden_size"]), int(spec["latent"]), int(spec["window"])
+
+        @classmethod
+        def declare(cls, spec, prefix):
+            h, l = int(spec["hidden_size"]), int(spec["latent"])
+            return [TensorDecl(f"{prefix}.down.weight", (l, h)), TensorDecl(f"{prefix}.up.weight", (h, l))]
+
+        def load(self, store, prefix, device):
+            self.down = store.get(f"{prefix}.down.weight", torch.float32, device)
+            self.up = store.get(f"{prefix}.up.weight", torch.float32, device)
+
+        def cache_need(self):
+            return KVNeed(self.window, (PoolNeed("latent", (PAGE, self.l), torch.float32),))
+
+        def forward(self, x, ctx, cache):
+            pool = cache.pools["latent"]                                    # [pages, page_size, L]
+            page = pool.shape[1]
+            z = kernels.gemm_tn(x.float().contiguous(), self.down)
+            pool.view(-1, self.l)[ctx.slots[cache.group]] = z               # this step's rows into their pages
+            out = torch.empty((ctx.num_tokens, self.l), dtype=torch.float32, device=x.device)
+            table = ctx.block_tables[cache.group]
+            for b in range(ctx.num_seqs):
+                lo, hi, n = ctx.cu_q_host[b], ctx.cu_q_host[b + 1], ctx.ctx_lens_host[b]
+                for t in range(lo, hi):
+                    p = n - (hi - t)                                         # the token's position
+                    first = max(0, p - self.window + 1)
+                    pos = torch.arange(first, p + 1, device=x.device)
+                    rows = table[b][pos // page].long() * page + pos % page    # pages behind the window are gone (-1)
+                    assert int(rows.min()) >= 0
+                    out[t] = pool.view(-1, self.l)[rows].mean(0)
+            return kernels.gemm_tn(out, self.up).to(self.dtype)
+
+    @register_head("biased_head")
+    class BiasedHead(LMHead):
+        @classmethod
+        def declare(cls, spec, prefix=""):
+            return LMHead.declare(spec) + [TensorDecl(spec["bias_name"], (int(spec["vocab_size"]),))]
+
+        def load(self, store, prefix, device, shared=None):
+            super().load(store, prefix, device, shared=shared)
+            self.bias = store.get(self.spec["bias_name"], torch.float32, device)
+
+        def forward(self, h):
+            logits = self.proj(h, out_dtype=torch.float32, skinny_rows=kernels.SKINNY_MAX_ROWS) + self.bias
+            return kernels.softcap_(logits, self.softcap)
+
+    @dataclass(frozen=True)
+    class LatentConfig:
+        vocab_size: int
+        architecture: str = "ToyLatentForCausalLM"
+
+        @classmethod
+        def from_dict(cls, raw, where="config.json"):
+            return cls(int(raw["vocab_size"]))
+
+        def to_dict(self):
+            return {"architectures": [self.architecture], "vocab_size": self.vocab_size}
+
+    def latent_spec(cfg):
+        norm = PartSpec("rmsnorm", dict(dim=H, eps=1e-5))
+        ffn = PartSpec("gated_mlp", dict(hidden_size=H, intermediate_size=64, activation="silu"))
+        rope = PartSpec("rope", dict(head_dim=16, rotary_dim=16, theta=10000.0, max_positions=256))
+        attn = PartSpec("attention", dict(hidden_size=H, num_heads=3, num_kv_heads=1, head_dim=16, qk_norm=False,
+                                          window=None, position=rope, scale=0.25))
+        layers = (LayerSpec("blocks.0", "prenorm", PartSpec("latent_mean", dict(hidden_size=H, latent=L, window=WINDOW)), ffn,
+                            {"ln_a": norm, "ln_b": norm}, mixer_name="mean", feed_forward_name="ff"),
+                  LayerSpec("blocks.1", "prenorm", attn, ffn, {"ln_a": norm, "ln_b": norm}, mixer_name="attn",
+                            feed_forward_name="ff"))
+        return ModelSpec(
+            architecture=cfg.architecture, vocab_size=cfg.vocab_size, hidden_size=H, max_positions=256,
+            embedding=PartSpec("embedding", dict(name="wte.weight", vocab_size=cfg.vocab_size, dim=H, scale=SCALE)),
+            layers=layers, schedule=(ScheduleEntry(0), ScheduleEntry(1)),
+            final_norm=PartSpec("rmsnorm", dict(dim=H, eps=1e-5, name="ln_f.weight")),
+            head=PartSpec("biased_head", dict(name="wte.weight", tied=True, vocab_size=cfg.vocab_size, dim=H,
+                                              bias_name="head.bias", softcap=CAP)))
+
+    register_architecture("ToyLatentForCausalLM", ModelFamily("toy_latent", LatentConfig, latent_spec))
+    d = write_random_model(str(tmp_path / "latent"), {"architectures": ["ToyLatentForCausalLM"], "vocab_size": V},
+                           seed=4, linear_std=0.15)
+    model = load_model(d, dtype, DEV)
+    assert [g.window for g in model.cache_groups] == [WINDOW, 0]
+    assert [p.name for p in model.kv_needs[0].pools] == ["latent"] and [p.name for p in model.kv_needs[1].pools] == ["k", "v"]
+
+    W = plain.read_weights(d)
+    assert set(W) >= {"wte.weight", "head.bias", "blocks.0.mean.down.weight", "blocks.0.ln_a.weight", "blocks.1.attn.q_proj.weight",
+                      "blocks.1.ff.down_proj.weight", "ln_f.weight"} and "lm_head.weight" not in W
+    cos, sin = plain.rope_tables(10000.0, 16, 256)
+
+    def toy_logits(ids):
+        T = len(ids)
+        x = W["wte.weight"][torch.tensor(ids)] * SCALE
+        z = plain.rms_norm(x, W["blocks.0.ln_a.weight"], 1e-5) @ W["blocks.0.mean.down.weight"].T
+        m = torch.stack([z[max(0, t - WINDOW + 1):t + 1].mean(0) for t in range(T)])
+        r = x + m @ W["blocks.0.mean.up.weight"].T
+        x = r + plain.mlp_block(plain.rms_norm(r, W["blocks.0.ln_b.weight"], 1e-5), W, "blocks.0.ff")
+        h = plain.rms_norm(x, W["blocks.1.ln_a.weight"], 1e-5)
+        pos = torch.arange(T)
+        q = plain.apply_rope((h @ W["blocks.1.attn.q_proj.weight"].T).reshape(T, 3, 16), pos, cos, sin)
+        k = plain.apply_rope((h @ W["blocks.1.attn.k_proj.weight"].T).reshape(T, 1, 16), pos, cos, sin)
+        v = (h @ W["blocks.1.attn.v_proj.weight"].T).reshape(T, 1, 16)
+        r = x + plain.attention(q, k, v, scale=0.25).reshape(T, 48) @ W["blocks.1.attn.o_proj.weight"].T
+        x = r + plain.mlp_block(plain.rms_norm(r, W["blocks.1.ln_b.weight"], 1e-5), W, "blocks.1.ff")
+        logits = plain.rms_norm(x, W["ln_f.weight"], 1e-5) @ W["wte.weight"].T + W["head.bias"]
+        return CAP * torch.tanh(logits / CAP)
+
+    rng = random.Random(19)
+    reqs = {f"q{i}": harness.random_prompt(rng, n, V) for i, n in enumerate([21, 60, 5, 37, 90])}
+    ref = {rid: toy_logits(t) for rid, t in reqs.items()}
+    assert float(max(r.abs().max() for r in ref.values())) > 0.8 * CAP            # the cap is at work
+    for what, steps in (("whole", harness.trace_whole(reqs)), ("mixed", harness.trace_mixed(reqs, 2, max_live=3)),
+                        ("portions", harness.trace_portions(reqs)), ("tail", harness.trace_tail_one_by_one(reqs, tail=20))):
+        need = harness.tokens_needed(steps, 8) // 8
+        runner = ModelRunner(model, page_size=8, num_pages=[need, need], max_requests=3)
+        got = harness.replay(runner, steps)
+        assert runner.cache.free_pages(0) == need and runner.cache.free_pages(1) == need
+        harness.compare(got, ref, harness.TOL[dtype], f"toy latent {dtype} {what}")
+
+    # through the scheduler: the window group's pool holds a window and a portion (11 - 1 + 16 tokens: 4 pages and
+    # one more), far less than the requests' lengths; greedy tokens are the plain model's
+    if dtype == "float32":
+        eng = Engine(EngineConfig(weight_path=d, page_size=8, num_pages=[2 * 5 + 1, 40], max_num_seqs=2, prefill_chunk_size=16,
+                                  max_num_batched_tokens=24), dtype)
+        prompts = [reqs["q1"], reqs["q4"][:70]]
+        outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True))
+        for p, o in zip(prompts, outs):
+            ids = list(p)
+            for tok in o.token_ids:
+                lg = toy_logits(ids)[-1]
+                assert float(lg.max() - lg[tok]) < 1e-4
+                ids.append(tok)
+        assert eng.runner.cache.free_pages(0) == 11 and eng.runner.cache.free_pages(1) == 40
+
+
 # ---- a toy feed-forward with routing and a toy position encoding, registered from here --------------------
 def test_toy_routed_feed_forward_and_position_encoding(tmp_path):
     """Two more part kinds defined in this test: a feed-forward that routes every token to the

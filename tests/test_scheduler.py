@@ -149,3 +149,40 @@ def test_random_workloads_finish_and_free_everything(seed):
     assert cm.live_requests() == 0
     for g, grp in enumerate(cm.groups):
         assert cm.free_pages(g) == grp.num_pages
+
+
+def test_a_window_group_holds_the_window_and_a_portion_not_the_whole_request():
+    """A prompt of 400 tokens on a model with a group that keeps the last 20 keys: that group's pool
+    of 5 pages of 16 tokens (window - 1 + a portion of 32 = 51 tokens, 4 pages, and one more for a start
+    inside a page) is enough, while the group that keeps every key needs all 26.  The request is
+    admitted, runs in portions without a preemption, and the window group never holds more than
+    its 5 pages; with 4 it is refused when added."""
+    cm, s = make(num_pages=26, page=16, max_seqs=2, budget=32, chunk=32, window_pages=5)
+    s.add(0, 400, 8)
+    most = [0]
+
+    def on_step(plan):
+        most[0] = max(most[0], 5 - cm.free_pages(1))
+    seen, steps = drive(s, cm, {0: (400, 8)}, on_step=on_step)
+    assert "preempted" not in seen[0]
+    assert [c for _, c in seen[0][:13]] == [32] * 12 + [16] and steps == 13 + 7
+    assert 4 <= most[0] <= 5
+    assert cm.free_pages(0) == 26 and cm.free_pages(1) == 5
+    cm, s = make(num_pages=26, page=16, max_seqs=2, budget=32, chunk=32, window_pages=4)
+    with pytest.raises(RequestTooLarge):
+        s.add(0, 400, 8)
+    s.add(1, 40, 8)             # 48 tokens at most: 3 pages hold them all
+
+
+def test_two_long_requests_share_a_small_window_pool():
+    """Two requests whose window pages would not fit if each held its whole length: both run to the
+    end; when the window pool is short the younger gives way and is recomputed."""
+    cm, s = make(num_pages=60, page=16, max_seqs=2, budget=48, chunk=24, window_pages=7)
+    reqs = {0: (300, 20), 1: (250, 30)}
+    for rid, (p, n) in reqs.items():
+        s.add(rid, p, n)
+    seen, _ = drive(s, cm, reqs)
+    for rid, (p, n) in reqs.items():
+        spans = [x for x in seen[rid] if x != "preempted"]
+        assert spans[-1][0] + spans[-1][1] == p + n - 1
+    assert cm.free_pages(0) == 60 and cm.free_pages(1) == 7

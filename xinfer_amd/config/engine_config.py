@@ -9,7 +9,7 @@ prefix cache, server, speculative decoding) are absent rather than accepted and 
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import List, Optional, Tuple
+from typing import List, Optional, Tuple, Union
 
 
 @dataclass
@@ -84,7 +84,7 @@ class EngineConfig:
     disable_cuda_graph: bool = False        # the reference's name; here it disables HIP graphs
     # --- this engine's own ---
     page_size: int = 64                     # tokens per cache page (the reference fixes 64)
-    num_pages: Optional[int] = None         # pages per cache group; default: from kv_fraction
+    num_pages: Union[int, List[int], None] = None   # pages of every cache group, or one count per group; default: from kv_fraction
     max_num_batched_tokens: Optional[int] = None   # token budget of a step; default: chunk size
     device: str = "cuda:0"
 

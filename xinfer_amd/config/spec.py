@@ -29,12 +29,26 @@ class PartSpec:
 @dataclass(frozen=True)
 class LayerSpec:
     """One decoder layer: which block arrangement, and the parts it is made of.
-    `prefix` is the tensor-name prefix of the layer's weights."""
+    Tensor names are data of the layer too: `prefix` is the prefix of all its weights,
+    `mixer_name` and `feed_forward_name` what follows it for those two parts, and the keys
+    of `norms` what follows it for each norm.  The order of `norms` says which is which:
+    the block arrangement takes them in the order in which it runs them (for "prenorm":
+    the norm before the mixer, then the norm before the feed-forward)."""
     prefix: str
     block: str
     mixer: PartSpec
     feed_forward: PartSpec
     norms: Mapping[str, PartSpec]
+    mixer_name: str = "self_attn"
+    feed_forward_name: str = "mlp"
+
+    def norm_items(self, count: int):
+        """The first `count` norms as (tensor name under the prefix, spec), in running order."""
+        items = list(self.norms.items())
+        if len(items) < count:
+            raise ValueError(f"layer {self.prefix!r} names {len(items)} norms; its block arrangement "
+                             f"{self.block!r} runs {count}")
+        return items[:count]
 
 
 @dataclass(frozen=True)

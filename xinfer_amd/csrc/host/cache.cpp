@@ -43,26 +43,31 @@ int CacheManager::pages_needed(int64_t id, int64_t n, int g) const {
   return (int)std::max<int64_t>(0, want - have);
 }
 
-bool CacheManager::can_reserve(int64_t id, int64_t n) const {
+// Tokens for which group g takes pages when n run next and `ahead` are known to follow.
+static inline int64_t tokens_of(const GroupSpec& grp, int64_t n, int64_t ahead) {
+  return grp.window > 0 ? n : std::max(n, ahead);
+}
+
+bool CacheManager::can_reserve(int64_t id, int64_t n, int64_t ahead) const {
   if (!find(id) || n < 0) return false;
   for (int g = 0; g < num_groups(); ++g)
-    if (pages_needed(id, n, g) > free_pages(g)) return false;
+    if (pages_needed(id, tokens_of(groups_[g], n, ahead), g) > free_pages(g)) return false;
   return true;
 }
 
-bool CacheManager::reserve(int64_t id, int64_t n) {
+bool CacheManager::reserve(int64_t id, int64_t n, int64_t ahead) {
   auto it = requests_.find(id);
   if (it == requests_.end()) {
     error_ = "reserve: unknown request " + std::to_string(id);
     return false;
   }
-  if (!can_reserve(id, n)) {
+  if (!can_reserve(id, n, ahead)) {
     error_ = "No free blocks available, retry later!";  // block_manager.rs:139
     return false;
   }
   RequestPages& r = it->second;
   for (int g = 0; g < num_groups(); ++g) {
-    const int need = pages_needed(id, n, g);
+    const int need = pages_needed(id, tokens_of(groups_[g], n, ahead), g);
     for (int i = 0; i < need; ++i) {
       const int32_t p = free_[g].front();
       free_[g].pop_front();

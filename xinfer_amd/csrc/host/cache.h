@@ -48,10 +48,13 @@ class CacheManager {
   int add_request(int64_t id);
   // Pages that `reserve(id, n)` would have to take from group g's pool.
   int pages_needed(int64_t id, int64_t n, int g) const;
-  bool can_reserve(int64_t id, int64_t n) const;
+  bool can_reserve(int64_t id, int64_t n, int64_t ahead = 0) const;
   // Reserves pages for the next n tokens of the request in every group, or changes
-  // nothing and returns false when a pool has too few free pages.
-  bool reserve(int64_t id, int64_t n);
+  // nothing and returns false when a pool has too few free pages.  `ahead` > n: groups that
+  // keep every key reserve for that many tokens at once (a prompt admitted whole, of which n
+  // tokens run first); a group with a window takes pages for the n tokens alone, since by the
+  // time the later ones run it has given earlier pages back.
+  bool reserve(int64_t id, int64_t n, int64_t ahead = 0);
   // The next n tokens are now in the cache.  Gives back window pages no later query needs.
   // Returns the number of pages given back, or -1 on misuse (see last_error()).
   int commit(int64_t id, int64_t n);

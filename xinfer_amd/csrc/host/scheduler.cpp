@@ -27,7 +27,16 @@ int Scheduler::add(int64_t id, int64_t prompt_len, int64_t max_new_tokens) {
   const int64_t max_len = prompt_len + max_new_tokens;
   for (int g = 0; g < cm_->num_groups(); ++g) {
     const GroupSpec& grp = cm_->group(g);
-    const int64_t pages = (max_len + grp.page_size - 1) / grp.page_size;
+    // A group that keeps every key holds the whole request at its end.  A group with a window
+    // holds, while a portion of n tokens runs, the window - 1 keys before it and its own n: one
+    // page more than those tokens fill, since they need not start at a page's edge.
+    int64_t held = max_len;
+    int64_t pages = (max_len + grp.page_size - 1) / grp.page_size;
+    if (grp.window > 0) {
+      const int64_t portion = std::min<int64_t>(chunk_size_, max_batched_tokens_);
+      held = std::min<int64_t>(max_len, (int64_t)grp.window - 1 + portion);
+      pages = std::min<int64_t>(pages, (held + grp.page_size - 1) / grp.page_size + 1);
+    }
     if (pages > grp.num_pages) {
       error_ = "request of " + std::to_string(prompt_len) + " prompt tokens and up to " +
                std::to_string(max_new_tokens) + " new tokens needs " + std::to_string(pages) +
@@ -93,14 +102,18 @@ const std::vector<SchedEntry>& Scheduler::schedule(std::vector<int64_t>* preempt
 
   // 3: admissions, in queue order, while everything allows.  A new request gets pages for
   // all of its known tokens at once (as the reference allocates a whole prompt,
-  // block_manager.rs:132-147), so its later portions cannot run out of pages.
+  // block_manager.rs:132-147), so its later portions cannot run out of pages, in the groups that
+  // keep every key; in a group with a window it gets the first portion's pages, and each later
+  // portion takes its own after the pages behind the window have gone back (if the pool is
+  // short then, the youngest request gives way as for any other growth).
   // Nothing is admitted in a step that had to preempt: pages are short.
   while (!preempted_any && !waiting_.empty() && budget > 0 && (int)running_.size() < max_num_seqs_ &&
          cm_->free_state_slots() > 0) {
     const int64_t id = waiting_.front();
     SchedRequest& r = requests_.at(id);
     if (cm_->add_request(id) < 0) break;
-    if (!cm_->reserve(id, r.total_len)) {
+    const int64_t n = std::min<int64_t>({r.total_len, (int64_t)chunk_size_, budget});
+    if (!cm_->reserve(id, n, r.total_len)) {
       cm_->release(id);
       break;
     }
@@ -108,7 +121,6 @@ const std::vector<SchedEntry>& Scheduler::schedule(std::vector<int64_t>* preempt
     r.running = true;
     r.order = next_order_++;
     running_.push_back(id);
-    const int64_t n = std::min<int64_t>({r.total_len, (int64_t)chunk_size_, budget});
     plan_.push_back(SchedEntry{id, 0, (int32_t)n, n == r.total_len ? 1 : 0});
     budget -= n;
   }

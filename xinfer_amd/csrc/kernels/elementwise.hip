@@ -3,6 +3,8 @@
 // All reductions are float32 in an order fixed by the row alone, so a row's
 // result does not depend on what else is in the batch.
 #include "common.h"
+
+#include <algorithm>
 #include <stdarg.h>
 #include <stdio.h>
 
@@ -17,16 +19,27 @@ void set_error(const char* fmt, ...) {
 }
 
 // ---------------------------------------------------------------------------------
-// Embedding: out[t, :] = float(table[ids[t], :])                (reference call site:
-// /root/reference/src/models/qwen3.rs:303, candle Embedding::forward)
+// Embedding: out[t, :] = float(table[ids[t], :]) * scale         (reference call site:
+// /root/reference/src/models/qwen3.rs:303, candle Embedding::forward; Qwen3 has no scale: 1)
 // ---------------------------------------------------------------------------------
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids,
-                             float* __restrict__ out, int H) {
+                             float* __restrict__ out, int H, float scale) {
   const int t = blockIdx.x;
   const T* row = table + (size_t)ids[t] * H;
   float* o = out + (size_t)t * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_float(row[i]);
+  if (scale == 1.0f) {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_float(row[i]);
+  } else {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_float(row[i]) * scale;
+  }
+}
+
+// Soft cap of logits in place: x = cap * tanh(x / cap), in float32.
+__global__ void softcap_kernel(float* __restrict__ x, size_t n, float cap) {
+  const float inv = 1.0f / cap;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+    x[i] = cap * tanhf(x[i] * inv);
 }
 
 // ---------------------------------------------------------------------------------
@@ -493,17 +506,26 @@ extern "C" {
 
 const char* xi_last_error() { return g_error; }
 
-int xi_embed(const void* table, int dtype, const int* ids, float* out, int n_tok, int H,
+int xi_embed(const void* table, int dtype, const int* ids, float* out, int n_tok, int H, float scale,
              hipStream_t stream) {
   XI_CHECK(n_tok >= 0 && H > 0, "embed: bad sizes T=%d H=%d", n_tok, H);
   if (n_tok == 0) return 0;
   if (dtype == kF32)
-    embed_kernel<float><<<n_tok, 256, 0, stream>>>((const float*)table, ids, out, H);
+    embed_kernel<float><<<n_tok, 256, 0, stream>>>((const float*)table, ids, out, H, scale);
   else if (dtype == kBF16)
-    embed_kernel<bf16><<<n_tok, 256, 0, stream>>>((const bf16*)table, ids, out, H);
+    embed_kernel<bf16><<<n_tok, 256, 0, stream>>>((const bf16*)table, ids, out, H, scale);
   else
     XI_CHECK(false, "embed: unknown dtype %d", dtype);
   XI_LAUNCH_CHECK("embed");
+  return 0;
+}
+
+int xi_softcap(float* x, int64_t n, float cap, hipStream_t stream) {
+  XI_CHECK(n >= 0 && cap > 0.f, "softcap: bad sizes n=%lld cap=%g", (long long)n, (double)cap);
+  if (n == 0) return 0;
+  const int blocks = (int)std::min<int64_t>((n + 255) / 256, 4096);
+  softcap_kernel<<<blocks, 256, 0, stream>>>(x, (size_t)n, cap);
+  XI_LAUNCH_CHECK("softcap");
   return 0;
 }
 

@@ -105,10 +105,8 @@ class LLMEngine:
         max_num_seqs requests of max_model_len tokens can use."""
         free, _ = torch.cuda.mem_get_info(self.model.device)
         frac = self.econfig.kv_fraction if self.econfig.kv_fraction is not None else 0.6
-        per_token = 0
         esize = torch.tensor([], dtype=self.dtype).element_size()
-        for kv in self.model.kv_needs.values():
-            per_token += 2 * kv.num_kv_heads * kv.head_dim * esize
+        per_token = sum(pool.bytes_per_token(esize) for kv in self.model.kv_needs.values() for pool in kv.pools)
         per_page = max(1, per_token * page)
         by_memory = int(free * frac) // per_page
         by_use = self.econfig.max_num_seqs * (-(-self.max_model_len // page))

@@ -15,8 +15,8 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 from ..config.spec import ModelSpec, ScheduleEntry
-from ..parts import (Embedding, KVNeed, LayerCache, LMHead, StateNeed, StepContext, Stream,
-                     block_class, norm_class)
+from ..parts import (KVNeed, LayerCache, StateNeed, StepContext, Stream, block_class, embedding_class,
+                     head_class, norm_class)
 from ..weights.store import TensorDecl, WeightStore
 
 
@@ -33,10 +33,10 @@ class CausalLM:
             raise ValueError(f"dtype {dtype} is not supported (float32 or bfloat16)")
         self.spec = spec
         self.dtype = dtype
-        self.embedding = Embedding(spec.embedding, dtype)
+        self.embedding = embedding_class(spec.embedding.kind)(spec.embedding, dtype)
         self.blocks = [block_class(l.block)(l, dtype) for l in spec.layers]
         self.final_norm = norm_class(spec.final_norm.kind)(spec.final_norm, dtype)
-        self.head = LMHead(spec.head, dtype)
+        self.head = head_class(spec.head.kind)(spec.head, dtype)
         for e in spec.schedule:
             if not (0 <= e.layer < len(self.blocks)):
                 raise ValueError(f"schedule names layer {e.layer} but the model has {len(self.blocks)}")
@@ -52,11 +52,11 @@ class CausalLM:
     # ---- weights -------------------------------------------------------------
     @classmethod
     def declare(cls, spec: ModelSpec) -> List[TensorDecl]:
-        decls = Embedding.declare(spec.embedding)
+        decls = embedding_class(spec.embedding.kind).declare(spec.embedding)
         for l in spec.layers:
             decls += block_class(l.block).declare(l)
         decls += norm_class(spec.final_norm.kind).declare(spec.final_norm, "")
-        decls += LMHead.declare(spec.head)
+        decls += head_class(spec.head.kind).declare(spec.head)
         seen, out = set(), []
         for d in decls:                      # a tied head names the embedding table again
             if d.name not in seen:
@@ -120,7 +120,7 @@ class CausalLM:
             if c is None:
                 c = LayerCache()
             elif e.cache_of is not None:
-                c = LayerCache(c.group, c.k, c.v, c.state, write=False)
+                c = LayerCache(c.group, c.pools, c.state, write=False)
             blk = self.blocks[e.layer]
             if getattr(blk, "folds", False):
                 # the block that runs next may let this one half do its first norm

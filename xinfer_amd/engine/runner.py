@@ -1,9 +1,11 @@
 """The step function: runs one mixed batch through the model from the cache.
 
-`ModelRunner` owns the model, the device memory of the paged cache (one K and one V
-pool per layer that owns pages, `[pages, kv_heads, page_size, head_dim]`), the
-per-request state arenas, and the cache manager that says which request holds which
-pages.  `step` takes a list of entries (request, its next tokens, the places whose
+`ModelRunner` owns the model, the device memory of the paged cache (per layer that owns
+pages the pools its mixer declares: for attention a K and a V pool,
+`[pages, kv_heads, page_size, head_dim]`), the per-request state arenas, and the cache
+manager that says which request holds which pages.  A state slot is cleared when the
+request it serves runs its first token (a request that starts, or starts again after it
+gave way), so a mixer finds zeros there, never another request's state.  `step` takes a list of entries (request, its next tokens, the places whose
 logits are wanted), runs exactly those tokens as one batch against what earlier steps
 left in the cache, and returns float32 logits for the wanted places.  A decode token is
 an entry with one token; prompt portions may be cut anywhere.
@@ -22,7 +24,7 @@ import numpy as np
 import torch
 
 from ..cache import DecodeStepError, BatchArrays, CacheGroup, OutOfPages, PagedCacheManager
-from ..parts import LayerCache, StepContext
+from ..parts import PAGE, LayerCache, StepContext
 from .model import CausalLM
 
 
@@ -155,14 +157,18 @@ class ModelRunner:
         self.layer_caches: Dict[int, LayerCache] = {}
         for layer, kv in model.kv_needs.items():
             g = model.group_of_layer[layer]
-            shape = (groups[g].num_pages, kv.num_kv_heads, self.page_size, kv.head_dim)
-            v_shape = (shape[0], shape[1], shape[3], shape[2]) if kv.v_transposed else shape
-            self.layer_caches[layer] = LayerCache(
-                group=g,
-                k=torch.zeros(shape, dtype=model.dtype, device=self.device),
-                v=torch.zeros(v_shape, dtype=model.dtype, device=self.device))
+            pools = {}
+            for pool in kv.pools:         # what the mixer declares, page by page
+                if pool.name in pools or sum(1 for s in pool.shape if s == PAGE) != 1:
+                    raise ValueError(f"layer {layer}: pool {pool.name!r} of shape {pool.shape} must have a name of its "
+                                     "own and exactly one axis of the page's length")
+                shape = (groups[g].num_pages, *(self.page_size if s == PAGE else int(s) for s in pool.shape))
+                pools[pool.name] = torch.zeros(shape, dtype=pool.dtype or model.dtype, device=self.device)
+            self.layer_caches[layer] = LayerCache(group=g, pools=pools)
+        self._state_arenas: List[torch.Tensor] = []
         for layer, st in model.state_needs.items():
             arena = torch.zeros((self.max_requests, *st.shape), dtype=st.dtype, device=self.device)
+            self._state_arenas.append(arena)
             if layer in self.layer_caches:
                 self.layer_caches[layer].state = arena
             else:
@@ -202,6 +208,12 @@ class ModelRunner:
     def length(self, rid: int) -> int:
         return self.cache.length(rid)
 
+    def _clear_state(self, slots: Sequence[int]) -> None:
+        """Zeroes the given state slots in every arena (a slot keeps what the request before left)."""
+        idx = torch.tensor([int(s) for s in slots], dtype=torch.int64, device=self.device)
+        for arena in self._state_arenas:
+            arena.index_fill_(0, idx, 0)
+
     # ---- the step -----------------------------------------------------------------
     def step(self, entries: Sequence[StepEntry], reserved: bool = False) -> torch.Tensor:
         """Runs the entries' tokens as one batch.  Returns float32 [wanted, vocab] in the
@@ -214,6 +226,11 @@ class ModelRunner:
         B = len(entries)
         single = all(len(e.tokens) == 1 for e in entries)
         if single and self.use_graphs and B <= self.graph_max_batch and self._graphs:
+            if self._state_arenas:       # a request whose first token this is gets a clean slot
+                ids_ = np.fromiter((e.request for e in entries), np.int64, B)
+                fresh = self.cache.lengths(ids_) == 0
+                if fresh.any():
+                    self._clear_state([self.cache.state_slot(int(r)) for r in ids_[fresh]])
             logits = self._decode_recorded(entries, reserved)
             if logits is not None:
                 return logits
@@ -272,6 +289,10 @@ class ModelRunner:
             self.cache.reserve_many(rid_arr, counts_arr)   # OutOfPages leaves every request's length as it was
         decode = self.use_graphs and int(counts_arr.max()) == 1 and B <= self.graph_max_batch
         arrays = self.cache.build_batch(rid_arr, counts_arr, max_pages=self._max_table if decode else None)
+        if self._state_arenas:           # requests that run their first token get a clean slot
+            fresh = (arrays.ctx_lens - np.diff(arrays.cu_q)) == 0
+            if fresh.any():
+                self._clear_state(arrays.state_slots[fresh].tolist())
         ids32 = ids_host.astype(np.int32)
         rows32 = np.asarray(rows, dtype=np.int32)
         if decode:

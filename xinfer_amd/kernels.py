@@ -84,8 +84,8 @@ def _want(t: torch.Tensor, dtype: torch.dtype, what: str) -> None:
 
 
 # ---------------------------------------------------------------------------------------
-def embed(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out[t] = float32(table[ids[t]]).  ids: int32 [T], values in [0, rows) (caller checks)."""
+def embed(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None, scale: float = 1.0) -> torch.Tensor:
+    """out[t] = float32(table[ids[t]]) * scale.  ids: int32 [T], values in [0, rows) (caller checks)."""
     _dev(table, ids, out)
     _want(ids, torch.int32, "embed: ids")
     if table.dim() != 2 or ids.dim() != 1:
@@ -95,8 +95,18 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = 
         out = torch.empty((T, H), dtype=torch.float32, device=table.device)
     elif out.shape != (T, H) or out.dtype != torch.float32:
         raise KernelError("embed: out must be float32 [T, H]")
-    _ok(lib().xi_embed(_p(table), _code(table, "embed"), _p(ids), _p(out), T, H, _stream()))
+    _ok(lib().xi_embed(_p(table), _code(table, "embed"), _p(ids), _p(out), T, H, ctypes.c_float(scale), _stream()))
     return out
+
+
+def softcap_(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    """logits = cap * tanh(logits / cap), in place, float32."""
+    _dev(logits)
+    _want(logits, torch.float32, "softcap: logits")
+    if not cap > 0:
+        raise KernelError(f"softcap: the cap must be positive, got {cap}")
+    _ok(lib().xi_softcap(_p(logits), ctypes.c_int64(logits.numel()), ctypes.c_float(cap), _stream()))
+    return logits
 
 
 def add_rmsnorm(resid: torch.Tensor, y: Optional[torch.Tensor], weight: torch.Tensor, eps: float,

@@ -41,7 +41,8 @@ def qwen3_spec(cfg: Qwen3Config, prefix: str = "model.", tied=None) -> ModelSpec
         norm = PartSpec("rmsnorm", dict(dim=cfg.hidden_size, eps=cfg.rms_norm_eps))
         layers.append(LayerSpec(
             prefix=layer_prefix, block="prenorm", mixer=mixer, feed_forward=ffn,
-            norms={"input_layernorm": norm, "post_attention_layernorm": norm}))
+            norms={"input_layernorm": norm, "post_attention_layernorm": norm},       # qwen3.rs:81,93
+            mixer_name="self_attn", feed_forward_name="mlp"))                         # qwen3.rs:41,54
     return ModelSpec(
         architecture=cfg.architecture,
         vocab_size=cfg.vocab_size,

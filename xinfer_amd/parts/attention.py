@@ -85,7 +85,7 @@ class PagedAttention(Mixer):
     # ---- cache ---------------------------------------------------------------
     def cache_need(self) -> KVNeed:
         # the matrix-core kernels of the bfloat16 path read V transposed
-        return KVNeed(self.nkv, self.d, self.window, v_transposed=self.dtype == torch.bfloat16)
+        return KVNeed.keys_values(self.nkv, self.d, self.window, v_transposed=self.dtype == torch.bfloat16)
 
     # ---- step ----------------------------------------------------------------
     takes_sink = True

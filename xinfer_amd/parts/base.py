@@ -17,6 +17,10 @@ runs on the tokens of one step.  A part never learns which model it is in.
   PositionEncoding data for the mixer's fused kernel (for "rope": cos/sin tables)
   Block            forward(stream, ctx, cache) -> stream, the arrangement of the above
                    around the residual stream.
+  TokenEmbedding   forward(ids) -> float32 [T, hidden], the start of the residual stream;
+                   `table` is what a tied head shares
+  Head             forward(h) -> float32 logits [R, vocab]; load(..., shared=) takes the
+                   embedding's table when the spec says `tied`
 
 New kinds register themselves with the decorators below; a `PartSpec.kind` then selects
 them.  Nothing else in the engine has to change.
@@ -33,15 +37,40 @@ from ..weights.store import TensorDecl, WeightStore
 
 
 # ---- what a layer may ask of the cache ------------------------------------------------
+PAGE = -1      # in a pool's shape: the axis that is as long as a page has tokens
+
+
+@dataclass(frozen=True)
+class PoolNeed:
+    """One paged pool of a layer: the runner allocates [pages, *shape] with PAGE replaced by the
+    page size, in `dtype` (None: the activation dtype), and hands it to the mixer under `name`."""
+    name: str
+    shape: Tuple[int, ...]
+    dtype: Optional[torch.dtype] = None
+
+    def bytes_per_token(self, element_size: int) -> int:
+        n = 1
+        for s in self.shape:
+            n *= 1 if s == PAGE else int(s)
+        return n * (element_size if self.dtype is None else torch.tensor([], dtype=self.dtype).element_size())
+
+
 @dataclass(frozen=True)
 class KVNeed:
-    """Paged keys and values: `window` = 0 keeps every key, w > 0 the last w.  The K pool
-    is [pages, kv_heads, page_size, head_dim]; the V pool the same, or with `v_transposed`
-    [pages, kv_heads, head_dim, page_size]."""
-    num_kv_heads: int
-    head_dim: int
+    """What a mixer keeps in pages: `window` = 0 keeps every token's entry, w > 0 the last w (pages
+    that the window has passed go back to the pool while the request runs); `pools` names the
+    pools and the shape of a page in each.  `KVNeed.keys_values` is the pair that attention keeps;
+    a mixer of another kind may keep one pool (a latent), or pools of different widths."""
     window: int = 0
-    v_transposed: bool = False
+    pools: Tuple[PoolNeed, ...] = ()
+
+    @staticmethod
+    def keys_values(num_kv_heads: int, head_dim: int, window: int = 0, v_transposed: bool = False) -> "KVNeed":
+        """K pool "k" [pages, kv_heads, page_size, head_dim]; V pool "v" the same, or with
+        `v_transposed` [pages, kv_heads, head_dim, page_size]."""
+        k = PoolNeed("k", (num_kv_heads, PAGE, head_dim))
+        v = PoolNeed("v", (num_kv_heads, head_dim, PAGE) if v_transposed else (num_kv_heads, PAGE, head_dim))
+        return KVNeed(window, (k, v))
 
 
 @dataclass(frozen=True)
@@ -56,10 +85,17 @@ class LayerCache:
     """What one run of a layer gets from the cache.  `write` is False when the run reads
     the cache that another layer's run owns."""
     group: int = -1
-    k: Optional[torch.Tensor] = None          # [pages, kv_heads, page_size, head_dim]
-    v: Optional[torch.Tensor] = None
+    pools: Dict[str, torch.Tensor] = field(default_factory=dict)   # by PoolNeed.name: [pages, *shape]
     state: Optional[torch.Tensor] = None      # [max_requests, *StateNeed.shape]
     write: bool = True
+
+    @property
+    def k(self) -> Optional[torch.Tensor]:
+        return self.pools.get("k")
+
+    @property
+    def v(self) -> Optional[torch.Tensor]:
+        return self.pools.get("v")
 
 
 @dataclass
@@ -178,6 +214,23 @@ class PositionEncoding(Part):
     (2i, 2i+1) instead of (i, i + rotary_dim / 2)); its kernels apply them to q and k."""
 
 
+class TokenEmbedding(Part):
+    table: Optional[torch.Tensor] = None
+
+    def forward(self, ids: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Head(Part):
+    tied = False
+
+    def load(self, store: WeightStore, prefix: str, device, shared: Optional[torch.Tensor] = None) -> None:
+        raise NotImplementedError
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
 class Block:
     """Arrangement of a layer's parts around the residual stream."""
 
@@ -210,6 +263,8 @@ FEED_FORWARDS: Dict[str, type] = {}
 NORMS: Dict[str, type] = {}
 POSITION_ENCODINGS: Dict[str, type] = {}
 BLOCKS: Dict[str, type] = {}
+EMBEDDINGS: Dict[str, type] = {}
+HEADS: Dict[str, type] = {}
 
 
 def _register(table: Dict[str, type], what: str) -> Callable[[str], Callable[[type], type]]:
@@ -227,6 +282,8 @@ register_feed_forward = _register(FEED_FORWARDS, "feed-forward")
 register_norm = _register(NORMS, "norm")
 register_position_encoding = _register(POSITION_ENCODINGS, "position encoding")
 register_block = _register(BLOCKS, "block")
+register_embedding = _register(EMBEDDINGS, "embedding")
+register_head = _register(HEADS, "head")
 
 
 def _lookup(table: Dict[str, type], what: str, kind: str) -> type:
@@ -254,3 +311,11 @@ def position_encoding_class(kind: str) -> type:
 
 def block_class(kind: str) -> type:
     return _lookup(BLOCKS, "block", kind)
+
+
+def embedding_class(kind: str) -> type:
+    return _lookup(EMBEDDINGS, "embedding", kind)
+
+
+def head_class(kind: str) -> type:
+    return _lookup(HEADS, "head", kind)

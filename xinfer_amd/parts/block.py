@@ -17,39 +17,34 @@ from ..weights.store import TensorDecl, WeightStore
 from .base import (Block, Folded, KVNeed, LayerCache, NormSink, StateNeed, StepContext, Stream,
                    feed_forward_class, mixer_class, norm_class, register_block)
 
-# tensor-name infixes of a pre-norm decoder layer's parts (HF naming, qwen3.rs:41,54,81,93)
-_MIXER, _FFN = "self_attn", "mlp"
-
-
 @register_block("prenorm")
 class PreNormBlock(Block):
-    NORM_BEFORE_MIXER = "input_layernorm"
-    NORM_BEFORE_FFN = "post_attention_layernorm"
+    """Runs two norms: `layer.norms` names the one before the mixer first, then the one before
+    the feed-forward.  Every tensor name comes from the `LayerSpec`."""
 
     def __init__(self, layer: LayerSpec, dtype: torch.dtype):
         super().__init__(layer, dtype)
         self.mixer = mixer_class(layer.mixer.kind)(layer.mixer, dtype)
         self.ffn = feed_forward_class(layer.feed_forward.kind)(layer.feed_forward, dtype)
-        n1, n2 = layer.norms[self.NORM_BEFORE_MIXER], layer.norms[self.NORM_BEFORE_FFN]
+        (self._name1, n1), (self._name2, n2) = layer.norm_items(2)
         self.norm1 = norm_class(n1.kind)(n1, dtype)
         self.norm2 = norm_class(n2.kind)(n2, dtype)
 
     @classmethod
     def declare(cls, layer: LayerSpec) -> List[TensorDecl]:
         p = layer.prefix
-        out = mixer_class(layer.mixer.kind).declare(layer.mixer, f"{p}.{_MIXER}")
-        out += feed_forward_class(layer.feed_forward.kind).declare(layer.feed_forward, f"{p}.{_FFN}")
-        for name in (cls.NORM_BEFORE_MIXER, cls.NORM_BEFORE_FFN):
-            n = layer.norms[name]
+        out = mixer_class(layer.mixer.kind).declare(layer.mixer, f"{p}.{layer.mixer_name}")
+        out += feed_forward_class(layer.feed_forward.kind).declare(layer.feed_forward, f"{p}.{layer.feed_forward_name}")
+        for name, n in layer.norm_items(2):
             out += norm_class(n.kind).declare(n, f"{p}.{name}")
         return out
 
     def load(self, store: WeightStore, device) -> None:
         p = self.layer.prefix
-        self.mixer.load(store, f"{p}.{_MIXER}", device)
-        self.ffn.load(store, f"{p}.{_FFN}", device)
-        self.norm1.load(store, f"{p}.{self.NORM_BEFORE_MIXER}", device)
-        self.norm2.load(store, f"{p}.{self.NORM_BEFORE_FFN}", device)
+        self.mixer.load(store, f"{p}.{self.layer.mixer_name}", device)
+        self.ffn.load(store, f"{p}.{self.layer.feed_forward_name}", device)
+        self.norm1.load(store, f"{p}.{self._name1}", device)
+        self.norm2.load(store, f"{p}.{self._name2}", device)
 
     @property
     def graph_safe(self) -> bool:
