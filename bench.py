@@ -9,6 +9,9 @@ decode step through the engine's own step function (mixed-batch path, paged cach
 kernels) followed by greedy sampling on the GPU.  Beside it: the prefill of one
 2,048-token prompt, the decode step's bandwidth roofline, and decode at batch 1 and 64.
 
+`--peaks` adds what this card itself reaches (a read-only stream, one large square product) and
+the fractions of those, beside the fractions of the published peaks that the line always has.
+
 Data is synthetic: weights are seeded random values of the architecture's shapes made
 on the GPU, token ids are seeded uniform, and the cache contents the decode steps read
 are random values (decode timing does not depend on what the cache holds).
@@ -125,6 +128,41 @@ def serve(workload: str, layers) -> int:
     return 0
 
 
+def measured_peaks(dev="cuda:0"):
+    """(GB/s of a read-only stream over 4 GiB, TFLOP/s of one square bfloat16 product of 8192 in the
+    vendor library): what this card reaches, beside the published peaks.  Best of five runs each."""
+    import torch
+    from xinfer_amd import kernels
+    buf = torch.empty(1 << 30, dtype=torch.int32, device=dev)         # 4 GiB: sixteen times the memory-side cache
+    buf.zero_()
+    best = None
+    for workgroups, chunk in ((256, 1 << 18), (256, 1 << 16), (1024, 1 << 14)):     # the shapes that read fastest
+        for _ in range(5):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            kernels.stream_read(buf, workgroups, chunk)
+            b.record()
+            torch.cuda.synchronize()
+            ms = a.elapsed_time(b)
+            best = ms if best is None else min(best, ms)
+    gbps = buf.numel() * 4 / (best * 1e-3) / 1e9
+    del buf
+    n = 8192
+    x = torch.randn(n, n, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    w = torch.randn(n, n, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    best = None
+    for _ in range(6):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        torch.nn.functional.linear(x, w)
+        b.record()
+        torch.cuda.synchronize()
+        ms = a.elapsed_time(b)
+        best = ms if best is None else min(best, ms)
+    tflops = 2.0 * n * n * n / (best * 1e-3) / 1e12
+    return gbps, tflops
+
+
 def main() -> int:
     global CONTEXT, PREFILL_TOKENS
     ap = argparse.ArgumentParser()
@@ -143,6 +181,10 @@ def main() -> int:
     ap.add_argument("--skip-points", action="store_true", help="only the default decode run")
     ap.add_argument("--only", choices=["all", "decode", "prefill"], default="all",
                     help="run one phase only (for profiling); the JSON line then lacks the other")
+    ap.add_argument("--peaks", action="store_true",
+                    help="also measure what this card reaches on a read-only stream of 4 GiB and on one square "
+                         "bfloat16 product of 8192, and report the fractions of those beside the fractions of the "
+                         "published peaks")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -255,6 +297,13 @@ def main() -> int:
                      "frac": round(achieved / HBM_GBPS, 4)},
     }
     print(f"[bench] decode b{args.batch}: {sec * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
+    peaks = None
+    if args.peaks:
+        peaks = measured_peaks(dev)
+        out["peaks_measured"] = {"hbm_read_GBps": round(peaks[0], 1), "bf16_product_TFLOPs": round(peaks[1], 1)}
+        out["roofline"]["frac_of_measured"] = round(achieved / peaks[0], 4)
+        print(f"[bench] measured peaks: {peaks[0]:.0f} GB/s read-only stream, {peaks[1]:.0f} TFLOP/s square bf16 product",
+              file=sys.stderr, flush=True)
     if args.only == "decode":
         print(json.dumps(out), flush=True)
         return 0
@@ -263,6 +312,8 @@ def main() -> int:
     out["prefill"] = {"value": round(PREFILL_TOKENS / psec, 1), "tokens": PREFILL_TOKENS,
                       "ms": round(psec * 1e3, 3),
                       "frac": round(flops / psec / (PEAK_TFLOPS["bf16"] * 1e12), 4)}
+    if peaks is not None:
+        out["prefill"]["frac_of_measured"] = round(flops / psec / (peaks[1] * 1e12), 4)
     print(f"[bench] prefill {PREFILL_TOKENS}: {psec * 1e3:.2f} ms", file=sys.stderr, flush=True)
     if not args.skip_points:
         points = {}

@@ -11,7 +11,11 @@ import torch
 # both sides compute in 32 bits and differ only in the order of sums.  bfloat16: weights
 # are the same bfloat16 values on both sides; activations between kernels are rounded to
 # 8 mantissa bits (relative 2^-9 each), a handful of times per layer.
-TOL = {"float32": 5e-5, "bfloat16": 2e-2}
+# The worst errors the tests print on an MI355X: float32 5.9e-6 (tiny and real sizes, every way
+# of cutting); bfloat16 1.1e-2 at real layer sizes and 1.4e-2 on the long-context model, whose
+# sharpened scores make the rounding of q and k show more.  The bounds are about three times
+# the float32 figure and one and a half times the bfloat16 one.
+TOL = {"float32": 2e-5, "bfloat16": 2e-2}
 
 
 def random_prompt(rng: random.Random, n: int, vocab: int) -> List[int]:

@@ -143,13 +143,16 @@ def test_tiny_b_workload_chunked_and_sampled(model_dirs):
     for i in (4, 0, 2):
         alone = eng2.generate([prompts[i]], sps[i])[0]             # the same seed, another request id
         assert alone.token_ids == together[i].token_ids, i
-    # each token is a token the plain model gives non-negligible probability at that point
+    # each token is the one the plain model draws at that point from its own logits with the same
+    # uniform number (a request with a seed of its own draws from that seed's first stream)
+    from xinfer_amd.sampling import uniform
     pm = plain.PlainModel(model_dirs["B"])
-    ids = list(prompts[1])
-    for t in together[1].token_ids:
-        pr = torch.softmax(pm.logits(ids)[-1].double() / 0.8, -1)
-        assert float(pr[t]) > 1e-5
-        ids.append(t)
+    for i in (1, 2):
+        ids = list(prompts[i])
+        for n, t in enumerate(together[i].token_ids):
+            kept = plain_sampling.kept_probabilities(pm.logits(ids)[-1], 0.8)
+            assert plain_sampling.draw(kept, uniform(100 + i, 0, n)) == t, (i, n)
+            ids.append(t)
 
 
 def test_preemption_gives_the_same_tokens(model_dirs):

@@ -35,6 +35,32 @@ __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict_
   }
 }
 
+// Reads `n16` 16-byte words and keeps nothing: the read-only stream against which the
+// weight-streaming kernels are measured (bench.py --peaks).  A workgroup takes whole chunks of
+// `chunk16` words (consecutive addresses stay with one compute unit, as the rows of a weight do in
+// the products); a wave reads 1 KB an instruction and keeps eight of them in flight.
+__global__ __launch_bounds__(512) void stream_read_kernel(const uint4* __restrict__ p, size_t n16, size_t chunk16,
+                                                          unsigned* __restrict__ sink) {
+  unsigned acc = 0;
+  const size_t chunks = (n16 + chunk16 - 1) / chunk16;
+  for (size_t c = blockIdx.x; c < chunks; c += gridDim.x) {
+    const size_t lo = c * chunk16, hi = lo + chunk16 < n16 ? lo + chunk16 : n16;
+    size_t i = lo + threadIdx.x;
+    for (; i + 7 * 512 < hi; i += 8 * 512) {
+      uint4 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = p[i + u * 512];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    for (; i < hi; i += 512) {
+      const uint4 v = p[i];
+      acc ^= v.x ^ v.y ^ v.z ^ v.w;
+    }
+  }
+  if (acc == 0x9e3779b9u && sink != nullptr) *sink = acc;      // keeps the loads alive; `sink` is null in use
+}
+
 // Soft cap of logits in place: x = cap * tanh(x / cap), in float32.
 __global__ void softcap_kernel(float* __restrict__ x, size_t n, float cap) {
   const float inv = 1.0f / cap;
@@ -517,6 +543,18 @@ int xi_embed(const void* table, int dtype, const int* ids, float* out, int n_tok
   else
     XI_CHECK(false, "embed: unknown dtype %d", dtype);
   XI_LAUNCH_CHECK("embed");
+  return 0;
+}
+
+int xi_stream_read(const void* p, int64_t bytes, int workgroups, int64_t chunk_bytes, hipStream_t stream) {
+  XI_CHECK(bytes >= 0 && workgroups > 0 && workgroups <= 65535 && chunk_bytes >= 8192 && chunk_bytes % 8192 == 0 &&
+               ((uintptr_t)p & 15) == 0,
+           "stream_read: bad arguments bytes=%lld workgroups=%d chunk=%lld", (long long)bytes, workgroups,
+           (long long)chunk_bytes);
+  if (bytes < 16) return 0;
+  stream_read_kernel<<<workgroups, 512, 0, stream>>>((const uint4*)p, (size_t)(bytes / 16), (size_t)(chunk_bytes / 16),
+                                                     nullptr);
+  XI_LAUNCH_CHECK("stream_read");
   return 0;
 }
 

@@ -99,6 +99,15 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = 
     return out
 
 
+def stream_read(t: torch.Tensor, workgroups: int = 2048, chunk_bytes: int = 1 << 18) -> None:
+    """Reads all of a tensor's memory and keeps nothing: the plain read-only stream that the
+    weight-streaming kernels are measured against.  A workgroup reads whole chunks of
+    `chunk_bytes` (a multiple of 8 KB)."""
+    _dev(t)
+    _ok(lib().xi_stream_read(_p(t), ctypes.c_int64(t.numel() * t.element_size()), int(workgroups),
+                             ctypes.c_int64(chunk_bytes), _stream()))
+
+
 def softcap_(logits: torch.Tensor, cap: float) -> torch.Tensor:
     """logits = cap * tanh(logits / cap), in place, float32."""
     _dev(logits)
