@@ -111,16 +111,32 @@ def serve(workload: str, layers) -> int:
     sp = SamplingParams(temperature=0.0, max_tokens=w["new_tokens"], ignore_eos=True)
     eng.generate(prompts[:2], SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True))   # warm-up
     steps0 = eng.steps
+    eng.step_log = []
     torch.cuda.synchronize()
     t = time.perf_counter()
     outs = eng.generate(prompts, sp)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t
     new = sum(o.decoded_length for o in outs)
+    # The least time the steps that ran could take: a step reads every weight once and the cache of its
+    # requests, and computes its tokens' products and its attention's pairs; it is bound by the slower
+    # of the two at the published peaks.
+    h, i_, nq, nkv, d, L = (cfg.hidden_size, cfg.intermediate_size, cfg.num_attention_heads, cfg.num_key_value_heads,
+                            cfg.head_dim, cfg.num_hidden_layers)
+    per_layer = (nq + 2 * nkv) * d * h + h * nq * d + 3 * i_ * h
+    wb, kvb = weight_bytes(cfg), kv_bytes_per_token(cfg)
+    least = mem_s = 0.0
+    for tokens, keys, pairs in eng.step_log:
+        mem = (wb + keys * kvb) / (HBM_GBPS * 1e9)
+        flop = (2.0 * tokens * L * per_layer + L * 4.0 * nq * d * pairs) / (PEAK_TFLOPS["bf16"] * 1e12)
+        least += max(mem, flop)
+        mem_s += mem
     print(json.dumps({
         "metric": f"generated tok/s, {workload} workload, bf16", "value": round(new / dt, 1), "unit": "tokens/s",
         "n_gpus": 1, "seconds": round(dt, 3), "engine_steps": eng.steps - steps0, "higher_is_better": True,
         "vs_reference_published": round(new / dt / w["reference_tok_s"], 2) if "reference_tok_s" in w else None,
+        "roofline": {"bound": "hbm or mfma, step by step", "least_seconds": round(least, 3),
+                     "least_seconds_memory_alone": round(mem_s, 3), "frac": round(least / dt, 4)},
         "dtype": "bf16", "data": "synthetic: seeded random weights, uniform random token ids",
         "config": {"model": w["name"], "layers": cfg.num_hidden_layers, "layers_of_model": full, "requests": n,
                    "prompt_tokens": sum(lens), "new_tokens": new, "prefill_chunk": w["chunk"],

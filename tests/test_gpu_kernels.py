@@ -754,6 +754,10 @@ def _cu_ctx(seqs):
 
 PREFILL_CASES = ATTN_CASES + [
     (8, 2, 128, 64, 0, [(2048, 300), (129, 129), (640, 2)]),     # a cached prefix before the portion
+    (8, 2, 128, 16, 0, [(700, 300), (65, 64)]),                  # pages smaller than a tile of 64 keys
+    (4, 4, 64, 128, 0, [(1000, 500), (200, 1)]),                 # pages larger than a tile
+    (4, 2, 32, 8, 40, [(333, 333)]),                              # head size 32, a window
+    (2, 1, 256, 64, 0, [(450, 200)]),                             # head size 256 behind a prefix
     (4, 1, 64, 16, 100, [(500, 260), (99, 99), (101, 3)]),       # window crossing block borders
     (6, 3, 96, 8, 0, [(257, 257)]),
     (2, 1, 16, 8, 5, [(40, 40), (6, 1)]),
@@ -772,21 +776,32 @@ def test_attention_prefill_mfma(nq, nkv, d, page, window, seqs):
     ref = _attention_ref(case, seqs, window, scale)
     q, kc, vt, bt = _mfma_inputs(case)
     cu, ctx = _cu_ctx(seqs)
-    for small in (False, True):          # both workgroup shapes
-        qb = kernels.prefill_block(d, nq // nkv, small)
-        tiles = torch.tensor([(b, q0) for b, (_, n) in enumerate(seqs) for q0 in range(0, n, qb)], dtype=torch.int32)
-        out = kernels.attention_prefill_bf16(q, kc, vt, bt, tiles.to(DEV), cu.to(DEV), ctx.to(DEV), scale, window,
-                                             small=small)
-        err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
-        assert err < _tol(torch.bfloat16, 2), (small, err)
-    # the launch order the engine uses: every block once
-    rows, small = kernels.prefill_tiles([n for _, n in seqs], [c for c, _ in seqs], d, nq, nkv)
-    qb = kernels.prefill_block(d, nq // nkv, small)
-    assert sorted(rows) == sorted((b, q0) for b, (_, n) in enumerate(seqs) for q0 in range(0, n, qb))
-    out = kernels.attention_prefill_bf16(q, kc, vt, bt, torch.tensor(rows, dtype=torch.int32).to(DEV), cu.to(DEV),
-                                         ctx.to(DEV), scale, window, small=small)
-    err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
-    assert err < _tol(torch.bfloat16, 2), err
+    # every workgroup shape of both kernels: the one whose tiles reach LDS through a ring of direct
+    # loads (head sizes 32, 64, 128, 256) and the one that copies them through registers
+    for ring in (True, False):
+        kernels.PREFILL_RING = ring
+        try:
+            shapes = (0, 1, 2) if ring and kernels.prefill_ring_supported(d) else (0, 1)
+            for small in shapes:
+                qb = kernels.prefill_block(d, nq // nkv, small)
+                tiles = torch.tensor([(b, q0) for b, (_, n) in enumerate(seqs) for q0 in range(0, n, qb)], dtype=torch.int32)
+                out = kernels.attention_prefill_bf16(q, kc, vt, bt, tiles.to(DEV), cu.to(DEV), ctx.to(DEV), scale, window,
+                                                     small=small)
+                err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
+                assert err < _tol(torch.bfloat16, 2), (ring, small, err)
+            # the launch order the engine uses: every block once
+            rows, small = kernels.prefill_tiles([n for _, n in seqs], [c for c, _ in seqs], d, nq, nkv)
+            qb = kernels.prefill_block(d, nq // nkv, small)
+            assert sorted(rows) == sorted((b, q0) for b, (_, n) in enumerate(seqs) for q0 in range(0, n, qb))
+            out = kernels.attention_prefill_bf16(q, kc, vt, bt, torch.tensor(rows, dtype=torch.int32).to(DEV), cu.to(DEV),
+                                                 ctx.to(DEV), scale, window, small=small)
+            err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
+            assert err < _tol(torch.bfloat16, 2), (ring, err)
+        finally:
+            kernels.PREFILL_RING = True
+    if not kernels.prefill_ring_supported(d):
+        with pytest.raises(kernels.KernelError, match="two groups"):
+            kernels.attention_prefill_bf16(q, kc, vt, bt, tiles.to(DEV), cu.to(DEV), ctx.to(DEV), scale, window, small=2)
     # the generic kernel reads the transposed pool too
     out2 = kernels.attention_generic(q, kc, vt, bt, case["tok_seq"].to(DEV), case["positions"].to(DEV), scale,
                                      window, v_transposed=True)
@@ -946,5 +961,6 @@ def test_attention_mfma_far_key_and_page_edges():
         assert (out.cpu().double() - ref).abs().max() / ref.abs().max() < _tol(torch.bfloat16, 2), far
         cu = torch.tensor([0, 1], dtype=torch.int32)
         tiles = torch.tensor([[0, 0]], dtype=torch.int32)
-        out = kernels.attention_prefill_bf16(q, kc, vt, bt, tiles.to(DEV), cu.to(DEV), ctx.to(DEV), scale, 0)
-        assert (out.cpu().double() - ref).abs().max() / ref.abs().max() < _tol(torch.bfloat16, 2), far
+        for small in (0, 1, 2):
+            out = kernels.attention_prefill_bf16(q, kc, vt, bt, tiles.to(DEV), cu.to(DEV), ctx.to(DEV), scale, 0, small=small)
+            assert (out.cpu().double() - ref).abs().max() / ref.abs().max() < _tol(torch.bfloat16, 2), (far, small)

@@ -218,7 +218,7 @@ def test_reference_attention_probe_cases(prefix, append, hq, hkv, page_map):
 
     cu = torch.tensor([0, append], dtype=torch.int32, device=DEV)
     cl = torch.tensor([kv_len], dtype=torch.int32, device=DEV)
-    for small in (False, True):
+    for small in (0, 1, 2):           # every workgroup shape of the prefill kernel
         qb = kernels.prefill_block(d, grp, small)
         tiles = torch.tensor([(0, q0) for q0 in range(0, append, qb)], dtype=torch.int32, device=DEV)
         out = kernels.attention_prefill_bf16(q_dev, kc, vt, bt, tiles, cu, cl, scale, 0, small=small)

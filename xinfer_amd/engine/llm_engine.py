@@ -96,6 +96,9 @@ class LLMEngine:
         self._next_id = 0
         self.steps = 0
         self.num_preemptions = 0
+        # set to a list to have every step's work recorded in it for a measurement: (tokens run,
+        # keys in the cache of the step's requests after it, query-key pairs of its attention)
+        self.step_log: Optional[list] = None
 
     # ---- memory -------------------------------------------------------------------
     def _plan_pages(self, page: int) -> int:
@@ -168,6 +171,9 @@ class LLMEngine:
         logits = self.runner.step(entries, reserved=True)
         self.scheduler.commit()
         self.steps += 1
+        if self.step_log is not None:
+            self.step_log.append((sum(e.count for e in plan), sum(e.start + e.count for e in plan),
+                                  sum(e.count * e.start + e.count * (e.count + 1) // 2 for e in plan)))
         done: List[int] = []
         if sampled:
             # (a request's generated tokens are tokens[prompt_len:]; no copies of them on this path)

@@ -332,7 +332,9 @@ def attention_prefill_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_
                            small=False):
     """MFMA attention for any mix of portions.  tiles int32 [n, 2] = (sequence, first query
     token of a block of `prefill_block(d, nq // nkv, small)` tokens within the sequence's
-    portion); `small` selects the four-wave workgroup shape (see `prefill_tiles`)."""
+    portion); `small` selects the workgroup shape (see `prefill_tiles`): 0 eight waves, 1 four
+    waves and half the block, 2 (head sizes 32, 64, 128, 256) eight waves in two groups that split
+    a tile's keys, the block of shape 1."""
     _dev(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_lens, out)
     T, nq, d = q.shape
     nkv, page = k_cache.shape[1], k_cache.shape[2]
@@ -345,17 +347,29 @@ def attention_prefill_bf16(q, k_cache, vt_cache, block_tables, tiles, cu_q, ctx_
         raise KernelError("attention_prefill: block_tables [B, pages], cu_q [B+1], ctx_lens [B], tiles [n, 2] expected")
     if out is None:
         out = torch.empty((T, nq * d), dtype=q.dtype, device=q.device)
-    _ok(lib().xi_attention_prefill_bf16(
+    # head sizes 32, 64, 128, 256: the kernel whose tiles reach LDS through a ring of direct loads
+    ring = PREFILL_RING and prefill_ring_supported(d)
+    if int(small) == 2 and not ring:
+        raise KernelError(f"attention_prefill: the shape of two groups of waves needs a head size of 32, 64, 128 or 256, got {d}")
+    entry = lib().xi_attention_prefill_ring_bf16 if ring else lib().xi_attention_prefill_bf16
+    _ok(entry(
         _p(q), _p(k_cache), _p(vt_cache), _p(block_tables), int(block_tables.shape[1]), _p(tiles),
         int(tiles.shape[0]), _p(cu_q), _p(ctx_lens), _p(out), ctypes.c_float(scale), int(window), int(page),
-        nq, nkv, d, int(bool(small)), _stream()))
+        nq, nkv, d, int(small), _stream()))
     return out
+
+
+PREFILL_RING = True       # False: every head size goes to the kernel that copies tiles through registers
+
+
+def prefill_ring_supported(d: int) -> bool:
+    return bool(lib().xi_attention_prefill_ring_supported(int(d)))
 
 
 def prefill_block(d: int, group: int = 1, small: bool = False) -> int:
     """Query positions per workgroup of the prefill kernel for a head size, a number of
     query heads per kv head and a workgroup shape."""
-    return int(lib().xi_attention_prefill_block(int(d), int(group), int(bool(small))))
+    return int(lib().xi_attention_prefill_block(int(d), int(group), int(small)))
 
 
 COMPUTE_UNITS = 256
@@ -365,20 +379,31 @@ MIXED_DECODE_CONTEXT = 4096    # or the longest context this (measured on MI355X
                                # 40 query heads on 8 kv heads, 64 sequences at 1,500 keys: 450 -> 155 us a layer)
 
 
-def prefill_tiles(q_lens, ctx_lens, d: int, nq: int, nkv: int, small: Optional[bool] = None, first_seq: int = 0):
-    """The query blocks of a batch of portions for the prefill kernel: (rows, small).
+def prefill_tiles(q_lens, ctx_lens, d: int, nq: int, nkv: int, small=None, first_seq: int = 0):
+    """The query blocks of a batch of portions for the prefill kernel: (rows, shape).
     rows = [(sequence, first query of the block)] in launch order.  A block's work grows
     with the keys it sees, and the compute units take workgroups in launch order, so the
     blocks are sorted by work and laid out in a zigzag over rounds of one workgroup per
-    compute unit.  With few blocks the four-wave shape is used (`small`; chosen here unless
-    given): it doubles the workgroups and lets two of them share a compute unit, and the
-    zigzag gives a unit that got a long block in the first round a short one in the second.
-    The eight-wave shape has one workgroup per unit at a time: longest first."""
+    compute unit.  The shape (chosen here unless given) is 0, eight waves and the full block,
+    where that makes two workgroups a compute unit or more; with fewer blocks 1, four waves and
+    half the block: twice the workgroups, two of them resident on a compute unit, and the
+    zigzag gives a unit that got a long block in the first round a short one in the second; and
+    with so few blocks that even those leave compute units with one workgroup (a prompt of 2,048
+    tokens on 8 kv heads) 2, where the head size allows: eight waves in two groups that split a
+    tile's keys, so that the longest block, which ends up alone on its unit, walks its keys with
+    twice the waves (2,048 tokens, 32 query heads: 60 -> 56 us; 1,024: 31 -> 28).  Shape 0 has one
+    workgroup per unit at a time: longest first."""
     g = nq // nkv
     heads = nkv * (g // (4 if g % 4 == 0 else 2 if g % 2 == 0 else 1))     # workgroups per query block
     big = prefill_block(d, g, False)
     if small is None:
-        small = sum(-(-n // big) for n in q_lens[first_seq:]) * heads < 2 * COMPUTE_UNITS
+        blocks = sum(-(-n // big) for n in q_lens[first_seq:])
+        small = 0 if blocks * heads >= 2 * COMPUTE_UNITS else 1
+        if small and PREFILL_RING and prefill_ring_supported(d):
+            half = prefill_block(d, g, 1)
+            if sum(-(-n // half) for n in q_lens[first_seq:]) * heads <= 2 * COMPUTE_UNITS:
+                small = 2
+    small = int(small)
     qb = prefill_block(d, g, small)
     rows = [(b, q0) for b, n in enumerate(q_lens) if b >= first_seq for q0 in range(0, n, qb)]
     rows.sort(key=lambda t: -(ctx_lens[t[0]] - q_lens[t[0]] + t[1]))
@@ -386,7 +411,7 @@ def prefill_tiles(q_lens, ctx_lens, d: int, nq: int, nkv: int, small: Optional[b
     out = []
     for i in range(0, len(rows), per_round):
         chunk = rows[i:i + per_round]
-        out += chunk if (not small or (i // per_round) % 2 == 0) else chunk[::-1]
+        out += chunk if (small != 1 or (i // per_round) % 2 == 0) else chunk[::-1]
     return out, small
 
 
