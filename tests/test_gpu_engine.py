@@ -1044,6 +1044,177 @@ def test_toy_routed_feed_forward_and_position_encoding(tmp_path):
         harness.compare(harness.replay(runner, steps), ref, harness.TOL["float32"], f"toy routed {what}")
 
 
+# ---- a toy norm and a toy block arrangement, registered from here -----------------------------------------
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_norm_and_block_arrangement(dtype, tmp_path):
+    """Two more part kinds defined in this test: a norm that centres its rows and has a bias
+    (nothing a product could carry, so it is not foldable), and a block arrangement in which the
+    mixer and the feed-forward read the same normed rows and their sum goes through a second norm
+    before it joins the stream.  The architecture runs a built-in "prenorm" layer, the toy
+    arrangement, and the prenorm layer again (so a block that folds norms runs before and after
+    one that does not), and ends in the toy norm as its final norm (which norms the wanted rows
+    only).  Registered, written, loaded and stepped in every way of cutting, without a change to
+    the framework's files."""
+    from dataclasses import dataclass
+    from xinfer_amd.config.spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+    from xinfer_amd.engine import ModelRunner, load_model
+    from xinfer_amd.models import ModelFamily, register_architecture
+    from xinfer_amd.parts import (Block, Norm, Stream, feed_forward_class, mixer_class, norm_class, register_block,
+                                  register_norm)
+    from xinfer_amd.weights import TensorDecl, write_random_model
+
+    H, D, V, EPS = 48, 16, 83, 3e-4
+
+    @register_norm("centered")
+    class Centered(Norm):
+        """out = (s - mean(s)) * rsqrt(var(s) + eps) * weight + bias, s = resid (+ add), in float32.  The
+        contract of a norm: without `rows` the sum is written back into `resid` and every row is
+        normed; with `rows` only those rows are made and `resid` is left alone; `add` may be a stack
+        [P, T, H] of float32 partial sums."""
+
+        def __init__(self, spec, dtype):
+            super().__init__(spec, dtype)
+            self.dim, self.eps = int(spec["dim"]), float(spec["eps"])
+
+        @classmethod
+        def declare(cls, spec, prefix):
+            return [TensorDecl(f"{prefix}.weight", (int(spec["dim"]),), "norm"), TensorDecl(f"{prefix}.bias", (int(spec["dim"]),))]
+
+        def load(self, store, prefix, device):
+            self.weight = store.get(f"{prefix}.weight", torch.float32, device)
+            self.bias = store.get(f"{prefix}.bias", torch.float32, device)
+
+        def forward(self, resid, add, out_dtype, rows=None, out=None):
+            if add is not None:
+                add = add.sum(0) if add.dim() == 3 else add.float()
+            if rows is None:
+                if add is not None:
+                    resid += add
+                s = resid
+            else:
+                s = resid[rows.long()] + (add[rows.long()] if add is not None else 0.0)
+            c = s - s.mean(1, keepdim=True)
+            y = (c * torch.rsqrt((c * c).mean(1, keepdim=True) + self.eps) * self.weight + self.bias).to(out_dtype)
+            if out is not None:
+                out.copy_(y)
+                return out
+            return y
+
+    @register_block("parallel_then_norm")
+    class ParallelThenNorm(Block):
+        """r = x + norm_b(mixer(norm_a(x)) + feed_forward(norm_a(x)))"""
+
+        def __init__(self, layer, dtype):
+            super().__init__(layer, dtype)
+            self.mixer = mixer_class(layer.mixer.kind)(layer.mixer, dtype)
+            self.ffn = feed_forward_class(layer.feed_forward.kind)(layer.feed_forward, dtype)
+            (self.name_a, a), (self.name_b, b) = layer.norm_items(2)
+            self.norm_a, self.norm_b = norm_class(a.kind)(a, dtype), norm_class(b.kind)(b, dtype)
+
+        @classmethod
+        def declare(cls, layer):
+            p = layer.prefix
+            out = mixer_class(layer.mixer.kind).declare(layer.mixer, f"{p}.{layer.mixer_name}")
+            out += feed_forward_class(layer.feed_forward.kind).declare(layer.feed_forward, f"{p}.{layer.feed_forward_name}")
+            for name, n in layer.norm_items(2):
+                out += norm_class(n.kind).declare(n, f"{p}.{name}")
+            return out
+
+        def load(self, store, device):
+            p = self.layer.prefix
+            self.mixer.load(store, f"{p}.{self.layer.mixer_name}", device)
+            self.ffn.load(store, f"{p}.{self.layer.feed_forward_name}", device)
+            self.norm_a.load(store, f"{p}.{self.name_a}", device)
+            self.norm_b.load(store, f"{p}.{self.name_b}", device)
+
+        def cache_need(self):
+            return self.mixer.cache_need()
+
+        def forward(self, stream, ctx, cache):
+            def whole(y):                    # a part may answer with a stack of float32 partial sums
+                return y.sum(0) if y.dim() == 3 else y.float()
+            h = self.norm_a.forward(stream.resid, stream.pending, self.dtype)
+            branch = (whole(self.mixer.forward(h, ctx, cache)) + whole(self.ffn.forward(h, ctx))).contiguous()
+            return Stream(stream.resid, self.norm_b.forward(branch, None, torch.float32))
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        vocab_size: int
+        architecture: str = "ToyParallelForCausalLM"
+
+        @classmethod
+        def from_dict(cls, raw, where="config.json"):
+            return cls(int(raw["vocab_size"]))
+
+        def to_dict(self):
+            return {"architectures": [self.architecture], "vocab_size": self.vocab_size}
+
+    def toy_spec(cfg):
+        rms = PartSpec("rmsnorm", dict(dim=H, eps=1e-5))
+        cen = PartSpec("centered", dict(dim=H, eps=EPS))
+        rope = PartSpec("rope", dict(head_dim=D, rotary_dim=D, theta=10000.0, max_positions=256))
+        attn = PartSpec("attention", dict(hidden_size=H, num_heads=3, num_kv_heads=1, head_dim=D, qk_norm=True, qk_norm_eps=1e-5,
+                                          window=None, position=rope, scale=0.25))
+        ffn = PartSpec("gated_mlp", dict(hidden_size=H, intermediate_size=80, activation="silu"))
+        layers = (LayerSpec("model.layers.0", "prenorm", attn, ffn, {"input_layernorm": rms, "post_attention_layernorm": rms}),
+                  LayerSpec("model.layers.1", "parallel_then_norm", attn, ffn, {"ln_in": cen, "ln_out": rms}))
+        return ModelSpec(
+            architecture=cfg.architecture, vocab_size=cfg.vocab_size, hidden_size=H, max_positions=256,
+            embedding=PartSpec("embedding", dict(name="model.embed_tokens.weight", vocab_size=cfg.vocab_size, dim=H)),
+            # the prenorm layer runs again after the toy arrangement and reads the cache of its first run
+            layers=layers, schedule=(ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0, cache_of=0)),
+            final_norm=PartSpec("centered", dict(dim=H, eps=EPS, prefix="model.norm")),
+            head=PartSpec("lm_head", dict(name="lm_head.weight", tied=False, vocab_size=cfg.vocab_size, dim=H)))
+
+    register_architecture("ToyParallelForCausalLM", ModelFamily("toy_parallel", ToyConfig, toy_spec))
+    d = write_random_model(str(tmp_path / "toy"), {"architectures": ["ToyParallelForCausalLM"], "vocab_size": V},
+                           seed=6, linear_std=0.15)
+    model = load_model(d, dtype, DEV)
+    assert not model.blocks[1].graph_safe and model.blocks[0].graph_safe
+
+    W = plain.read_weights(d)
+    cos, sin = plain.rope_tables(10000.0, D, 256)
+
+    def centered(x, name):
+        c = x - x.mean(1, keepdim=True)
+        return c / torch.sqrt((c * c).mean(1, keepdim=True) + EPS) * W[f"{name}.weight"] + W[f"{name}.bias"]
+
+    def qkv(h, p, T):
+        def heads(name, n, norm):
+            y = (h @ W[f"{p}.{name}_proj.weight"].T).reshape(T, n, D)
+            return plain.apply_rope(plain.rms_norm(y, W[f"{p}.{norm}.weight"], 1e-5), torch.arange(T), cos, sin) if norm else y
+        return heads("q", 3, "q_norm"), heads("k", 1, "k_norm"), heads("v", 1, None)
+
+    def toy_logits(ids):
+        T = len(ids)
+        x = W["model.embed_tokens.weight"][torch.tensor(ids)]
+        kv = None
+        for run in (0, 1, 2):
+            if run == 1:
+                p = "model.layers.1"
+                h = centered(x, f"{p}.ln_in")
+                q, k, v = qkv(h, f"{p}.self_attn", T)
+                a = plain.attention(q, k, v, scale=0.25).reshape(T, 3 * D) @ W[f"{p}.self_attn.o_proj.weight"].T
+                x = x + plain.rms_norm(a + plain.mlp_block(h, W, f"{p}.mlp"), W[f"{p}.ln_out.weight"], 1e-5)
+                continue
+            p = "model.layers.0"
+            h = plain.rms_norm(x, W[f"{p}.input_layernorm.weight"], 1e-5)
+            q, k, v = qkv(h, f"{p}.self_attn", T)
+            if kv is None:
+                kv = (k, v)
+            r = x + plain.attention(q, kv[0], kv[1], scale=0.25).reshape(T, 3 * D) @ W[f"{p}.self_attn.o_proj.weight"].T
+            x = r + plain.mlp_block(plain.rms_norm(r, W[f"{p}.post_attention_layernorm.weight"], 1e-5), W, f"{p}.mlp")
+        return centered(x, "model.norm") @ W["lm_head.weight"].T
+
+    rng = random.Random(12)
+    reqs = {f"q{i}": harness.random_prompt(rng, n, V) for i, n in enumerate([27, 50, 6, 38])}
+    ref = {rid: toy_logits(t) for rid, t in reqs.items()}
+    for what, steps in (("whole", harness.trace_whole(reqs)), ("mixed", harness.trace_mixed(reqs, 1, max_live=2)),
+                        ("portions", harness.trace_portions(reqs)), ("tail", harness.trace_tail_one_by_one(reqs, tail=20))):
+        runner = ModelRunner(model, page_size=8, num_pages=harness.tokens_needed(steps, 8) // 8, max_requests=2)
+        harness.compare(harness.replay(runner, steps), ref, harness.TOL[dtype], f"toy parallel {dtype} {what}")
+
+
 # ---- the measurement script -------------------------------------------------------------------------------
 def test_bench_line_keeps_its_contract():
     """`bench.py` with two layers: one JSON line with the contract's fields, a flat `config` of at

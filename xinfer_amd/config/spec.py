@@ -69,6 +69,6 @@ class ModelSpec:
     embedding: PartSpec
     layers: Tuple[LayerSpec, ...]
     schedule: Tuple[ScheduleEntry, ...]
-    final_norm: PartSpec
+    final_norm: PartSpec                  # its parameter "prefix" (default "") is the prefix of its tensors' names
     head: PartSpec
     eos_token_ids: Tuple[int, ...] = ()

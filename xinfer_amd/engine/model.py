@@ -55,7 +55,7 @@ class CausalLM:
         decls = embedding_class(spec.embedding.kind).declare(spec.embedding)
         for l in spec.layers:
             decls += block_class(l.block).declare(l)
-        decls += norm_class(spec.final_norm.kind).declare(spec.final_norm, "")
+        decls += norm_class(spec.final_norm.kind).declare(spec.final_norm, str(spec.final_norm.get("prefix", "")))
         decls += head_class(spec.head.kind).declare(spec.head)
         seen, out = set(), []
         for d in decls:                      # a tied head names the embedding table again
@@ -75,7 +75,7 @@ class CausalLM:
         self.embedding.load(store, "", device)
         for b in self.blocks:
             b.load(store, device)
-        self.final_norm.load(store, "", device)
+        self.final_norm.load(store, str(self.spec.final_norm.get("prefix", "")), device)
         self.head.load(store, "", device, shared=self.embedding.table if self.head.tied else None)
         return self
 
