@@ -81,7 +81,7 @@ def prefill_flops(cfg, T):
     return linear + attn
 
 
-def serve(workload: str, layers) -> int:
+def serve(workload: str, layers, run_ahead: bool = True) -> int:
     """One of the serving workloads through the whole engine."""
     import torch
     from xinfer_amd import EngineConfig, SamplingParams
@@ -102,7 +102,7 @@ def serve(workload: str, layers) -> int:
     n = w["requests"]
     pages = n * (-(-w["max_model_len"] // page)) + 8
     eng = LLMEngine(EngineConfig(max_num_seqs=n, max_model_len=w["max_model_len"], num_pages=pages, page_size=page,
-                                 prefill_chunk_size=w["chunk"], seed=1),     # a step's token budget is the chunk
+                                 prefill_chunk_size=w["chunk"], seed=1, run_ahead=run_ahead),     # a step's token budget is the chunk
                     model=model)
     g = torch.Generator().manual_seed(4)
     lo, hi = w["prompt"]
@@ -197,6 +197,8 @@ def main() -> int:
     ap.add_argument("--skip-points", action="store_true", help="only the default decode run")
     ap.add_argument("--only", choices=["all", "decode", "prefill"], default="all",
                     help="run one phase only (for profiling); the JSON line then lacks the other")
+    ap.add_argument("--no-run-ahead", action="store_true",
+                    help="serving workloads: read every step's tokens on the host before the next step is planned")
     ap.add_argument("--peaks", action="store_true",
                     help="also measure what this card reaches on a read-only stream of 4 GiB and on one square "
                          "bfloat16 product of 8192, and report the fractions of those beside the fractions of the "
@@ -206,7 +208,7 @@ def main() -> int:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
     if args.workload != "decode":
-        return serve(args.workload, args.layers)
+        return serve(args.workload, args.layers, not args.no_run_ahead)
     if args.layers is None:
         args.layers = FULL_LAYERS
     CONTEXT, PREFILL_TOKENS = args.context, args.prefill_tokens     # the sizes of this run

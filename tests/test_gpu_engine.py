@@ -175,6 +175,62 @@ def test_preemption_gives_the_same_tokens(model_dirs):
         small.generate([harness.random_prompt(rng, 60, 256)], SamplingParams(max_tokens=30))
 
 
+def test_running_ahead_gives_the_same_tokens(model_dirs):
+    """The engine launches a step before it has read the tokens of the step before it (they reach the
+    step on the device) and applies the finishing rules a step late; with `run_ahead=False` it
+    reads every step's tokens first.  Both give the same tokens and reasons: greedy and sampled,
+    with so few pages that requests are preempted and recomputed, with stop tokens and
+    end-of-sequence ids (a request that ends has one token computed for nothing, which must not
+    show), with length limits of 1 and 2 tokens, with penalties (whose steps wait for the tokens),
+    and with requests cancelled while a step is on its way."""
+    from xinfer_amd import SamplingParams
+    rng = random.Random(3)
+    prompts = [harness.random_prompt(rng, n, 509) for n in (1, 9, 64, 130, 200, 33, 77, 5)]
+    stops = [[7], [100, 101], [3]] + [[t] for t in range(200, 260)]
+    cases = [
+        ("greedy", SamplingParams(temperature=0.0, max_tokens=24, ignore_eos=True), dict(num_pages=200)),
+        ("sampled, few pages", SamplingParams(temperature=0.8, top_k=20, max_tokens=60, ignore_eos=True),
+         dict(num_pages=36, max_num_seqs=6)),
+        ("whole distribution", SamplingParams(temperature=1.1, top_p=0.9, max_tokens=20, ignore_eos=True), dict(num_pages=200)),
+        ("stops", SamplingParams(temperature=0.9, max_tokens=60, ignore_eos=True, stop_token_ids=stops),
+         dict(num_pages=200, max_num_seqs=8)),
+        ("end of sequence", SamplingParams(temperature=0.9, max_tokens=60), dict(num_pages=200, eos=set(range(0, 509, 9)))),
+        ("one token", SamplingParams(temperature=0.0, max_tokens=1, ignore_eos=True), dict(num_pages=200)),
+        ("two tokens", SamplingParams(temperature=0.7, max_tokens=2, ignore_eos=True), dict(num_pages=200)),
+        ("penalties", SamplingParams(temperature=0.7, max_tokens=30, ignore_eos=True, frequency_penalty=0.5), dict(num_pages=200)),
+    ]
+    for name, sp, kw in cases:
+        kw = dict(kw)
+        eos = kw.pop("eos", None)
+        results = []
+        for ahead in (False, True):
+            eng = _engine(model_dirs["B"], "B", "f32", prefill_chunk_size=48, max_num_batched_tokens=64,
+                          run_ahead=ahead, **{"max_num_seqs": 4, **kw})
+            if eos is not None:
+                eng.eos_token_ids = eos
+            outs = eng.generate(prompts, sp)
+            results.append(([(o.token_ids, o.finish_reason) for o in outs], eng.num_preemptions))
+            assert eng.runner.cache.free_pages(0) == kw["num_pages"] and eng._launched is None, name
+        assert results[0][0] == results[1][0], name
+        if name == "sampled, few pages":
+            assert results[0][1] > 0 and results[1][1] > 0
+        if name in ("stops", "end of sequence"):
+            reasons = {r for _, r in results[1][0]}
+            assert ("stop" if name == "stops" else "eos") in reasons, reasons
+    # cancelling while a step is on its way: the others go on as if nothing had happened
+    sp = SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True)
+    alone = _engine(model_dirs["B"], "B", "f32", max_num_seqs=4, num_pages=200).generate([prompts[2], prompts[5]], sp)
+    eng = _engine(model_dirs["B"], "B", "f32", max_num_seqs=4, num_pages=200)
+    rids = [eng.add_request(p, sp) for p in (prompts[2], prompts[3], prompts[5])]
+    for _ in range(6):
+        eng.step()
+    assert eng._launched is not None
+    eng.cancel(rids[1])
+    eng.run_until_done()
+    assert [eng._finished[r].generated for r in (rids[0], rids[2])] == [o.token_ids for o in alone]
+    assert rids[1] not in eng._finished and eng.runner.cache.free_pages(0) == 200
+
+
 def test_eos_and_limits(model_dirs):
     from xinfer_amd import SamplingParams
     eng = _engine(model_dirs["A"], "A", "f32", max_num_seqs=2, num_pages=16, max_model_len=40)

@@ -87,6 +87,9 @@ class EngineConfig:
     num_pages: Union[int, List[int], None] = None   # pages of every cache group, or one count per group; default: from kv_fraction
     max_num_batched_tokens: Optional[int] = None   # token budget of a step; default: chunk size
     device: str = "cuda:0"
+    # launch a step before the tokens of the step before it have been read on the host (they
+    # reach it on the device); False: every step's tokens are read before the next is planned
+    run_ahead: bool = True
 
     def model_dir(self) -> str:
         if self.model_id and self.weight_path:

@@ -50,10 +50,22 @@ class _Request:
     finish_reason: str = ""
     preemptions: int = 0
     stops: List[List[int]] = field(default_factory=list)    # token sequences that end the generation
+    pending: int = 0                   # tokens sampled on the GPU that the host has not read yet
+    closed: bool = False               # the scheduler has let go of it already (its last token is on its way)
 
     @property
     def generated(self) -> List[int]:
         return self.tokens[self.prompt_len:]
+
+
+@dataclass
+class _Launched:
+    """A step that has been launched and whose sampled tokens the host has not read yet."""
+    sampled: List[_Request]            # the requests of its wanted rows, in row order
+    tokens: torch.Tensor               # int32 [rows] on the device
+    host: torch.Tensor                 # the same in pinned memory once `ready` has happened
+    ready: torch.cuda.Event
+    row_of: Dict[int, int]             # request id -> its row
 
 
 class LLMEngine:
@@ -99,6 +111,16 @@ class LLMEngine:
         # set to a list to have every step's work recorded in it for a measurement: (tokens run,
         # keys in the cache of the step's requests after it, query-key pairs of its attention)
         self.step_log: Optional[list] = None
+        # Running ahead: a step is launched with the tokens that the step before it is still
+        # sampling (they are handed over on the device), and only then are that earlier step's
+        # tokens read and its requests' stop rules applied, while the GPU works.  A request that
+        # turns out to have ended (end-of-sequence, a stop sequence) has one more token computed
+        # for nothing; one that reaches its length limit is known beforehand and is not planned again.
+        self.run_ahead = bool(econfig.run_ahead)
+        self._launched: Optional[_Launched] = None
+        rows = max(1, econfig.max_num_seqs)
+        self._token_pins = [torch.empty((rows,), dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self._pin_turn = 0
 
     # ---- memory -------------------------------------------------------------------
     def _plan_pages(self, page: int) -> int:
@@ -153,65 +175,128 @@ class LLMEngine:
     # ---- the loop ------------------------------------------------------------------------
     def step(self) -> List[int]:
         """One iteration: plan, run the batch, sample, finish.  Returns the ids that finished."""
+        done: List[int] = []
         plan, preempted = self.scheduler.schedule()
         for rid in preempted:
             self._requests[rid].preemptions += 1
             self.num_preemptions += 1
+        if self._launched is not None and (not plan or not self.run_ahead or self._needs_host_tokens(plan)):
+            # the earlier step's tokens are needed before this one can be launched (or there is nothing to launch)
+            done += self._collect()
+            plan = [e for e in plan if e.request in self._requests]    # (the scheduler dropped the ended ones from its plan too)
         if not plan:
-            if not self.scheduler.idle():
+            if not done and not self.scheduler.idle():
                 raise RuntimeError("the scheduler planned nothing although requests are waiting")
-            return []
+            return done
         entries, sampled = [], []
+        places, rows = [], []              # tokens of this step that the launched step is still sampling
+        at = 0
         for e in plan:
             r = self._requests[e.request]
-            toks = r.tokens[e.start:e.start + e.count]
+            end = e.start + e.count
+            if end > len(r.tokens):        # the entry's last token is on its way
+                if self._launched is None or end != len(r.tokens) + 1 or r.rid not in self._launched.row_of:
+                    raise RuntimeError(f"request {r.rid}: the plan runs ahead of its known tokens")
+                toks = r.tokens[e.start:] + [0]
+                places.append(at + e.count - 1)
+                rows.append(self._launched.row_of[r.rid])
+            else:
+                toks = r.tokens[e.start:end]
             entries.append(StepEntry(e.request, toks, [e.count - 1] if e.sample else []))
             if e.sample:
                 sampled.append(r)
-        logits = self.runner.step(entries, reserved=True)
+            at += e.count
+        device_tokens = (self._launched.tokens, places, rows) if places else None
+        logits = self.runner.step(entries, reserved=True, device_tokens=device_tokens)
         self.scheduler.commit()
         self.steps += 1
         if self.step_log is not None:
             self.step_log.append((sum(e.count for e in plan), sum(e.start + e.count for e in plan),
                                   sum(e.count * e.start + e.count * (e.count + 1) // 2 for e in plan)))
-        done: List[int] = []
+        launched = None
         if sampled:
             # (a request's generated tokens are tokens[prompt_len:]; no copies of them on this path)
             strategies = [r.strategy for r in sampled]
             recent = None
             if any(s.frequency_penalty or s.presence_penalty for s in strategies):
-                recent = [penalty_context(r.tokens, r.prompt_len) for r in sampled]
-            tokens = self.sampler.sample(
+                recent = [penalty_context(r.tokens, r.prompt_len) for r in sampled]     # (nothing is pending then)
+            tokens = self.sampler.sample_device(
                 logits, strategies,
-                [0.0 if r.strategy.greedy else uniform(r.seed, r.stream, len(r.tokens) - r.prompt_len) for r in sampled],
+                [0.0 if r.strategy.greedy else uniform(r.seed, r.stream, len(r.tokens) + r.pending - r.prompt_len)
+                 for r in sampled],
                 recent=recent)         # (a greedy row draws nothing)
-            now = _now_ms()
-            for r, tok in zip(sampled, tokens):
-                if len(r.tokens) == r.prompt_len:
-                    r.decode_start = now
-                reason = ""
-                if r.stops and _completes_a_stop(r.stops, r.generated, int(tok)):
-                    reason = "stop"
-                elif tok in self.eos_token_ids and not r.params.ignore_eos:
-                    reason = "eos"
-                else:
-                    r.tokens.append(int(tok))
-                    if len(r.tokens) - r.prompt_len >= r.max_tokens:
-                        reason = "length"
-                    elif len(r.tokens) >= self.max_model_len:
-                        reason = "max_model_len"
-                    else:
-                        self.scheduler.append_token(r.rid)
-                if reason:
-                    r.finish_reason = reason
-                    r.decode_finish = now
+            n = len(sampled)
+            if self._token_pins[self._pin_turn].numel() < n:
+                self._token_pins[self._pin_turn] = torch.empty((n,), dtype=torch.int32, pin_memory=True)
+            host = self._token_pins[self._pin_turn][:n]
+            self._pin_turn ^= 1
+            host.copy_(tokens, non_blocking=True)
+            ready = torch.cuda.Event()
+            ready.record()
+            launched = _Launched(sampled, tokens, host, ready, {r.rid: i for i, r in enumerate(sampled)})
+            # what the scheduler needs to plan the next step is known without the tokens: every
+            # sampled request grows by one, unless this token is the last it may have
+            for r in sampled:
+                r.pending += 1
+                known = len(r.tokens) + r.pending
+                if known - r.prompt_len >= r.max_tokens or known >= self.max_model_len:
                     self.scheduler.finish(r.rid)
-                    self._finished[r.rid] = self._requests.pop(r.rid)
-                    done.append(r.rid)
+                    r.closed = True
+                else:
+                    self.scheduler.append_token(r.rid)
+        if self._launched is not None:
+            done += self._collect()        # the step before, while the GPU runs this one
+        self._launched = launched
+        if launched is not None and not self.run_ahead:
+            done += self._collect()
+        return done
+
+    def _needs_host_tokens(self, plan) -> bool:
+        """Whether a step cannot be launched before the launched step's tokens are read: a request
+        it samples for counts its recent tokens (penalties)."""
+        for e in plan:
+            if e.sample:
+                s = self._requests[e.request].strategy
+                if s.frequency_penalty or s.presence_penalty:
+                    return True
+        return False
+
+    def _collect(self) -> List[int]:
+        """Reads the launched step's tokens and applies the finishing rules.  Returns the ids that finished."""
+        launched, self._launched = self._launched, None
+        launched.ready.synchronize()
+        done: List[int] = []
+        now = _now_ms()
+        for r, tok in zip(launched.sampled, launched.host.tolist()):
+            if self._requests.get(r.rid) is not r:
+                continue                   # ended or cancelled since: the token was computed for nothing
+            r.pending -= 1
+            if len(r.tokens) == r.prompt_len:
+                r.decode_start = now
+            reason = ""
+            if r.stops and _completes_a_stop(r.stops, r.generated, int(tok)):
+                reason = "stop"
+            elif tok in self.eos_token_ids and not r.params.ignore_eos:
+                reason = "eos"
+            else:
+                r.tokens.append(int(tok))
+                if len(r.tokens) - r.prompt_len >= r.max_tokens:
+                    reason = "length"
+                elif len(r.tokens) >= self.max_model_len:
+                    reason = "max_model_len"
+            if reason:
+                r.finish_reason = reason
+                r.decode_finish = now
+                if not r.closed:
+                    self.scheduler.finish(r.rid)
+                self._finished[r.rid] = self._requests.pop(r.rid)
+                done.append(r.rid)
+            elif r.closed and r.pending == 0:
+                raise RuntimeError(f"request {r.rid} was closed but did not finish")
         return done
 
     def run_until_done(self) -> None:
-        while not self.scheduler.idle():
+        while not self.scheduler.idle() or self._launched is not None:
             self.step()
 
     # ---- outputs ---------------------------------------------------------------------------
@@ -263,7 +348,8 @@ class LLMEngine:
         if r is None:
             self._finished.pop(rid, None)      # finished and never collected: forgotten now
             return
-        self.scheduler.finish(rid)
+        if not r.closed:                       # (else the scheduler let go of it when its last token was launched)
+            self.scheduler.finish(rid)
         r.finish_reason = "cancelled"
         r.decode_finish = _now_ms()
 

@@ -192,6 +192,9 @@ class ModelRunner:
         self.graphs_dropped = 0
         self._seen: Dict[Tuple[int, int, bool], int] = {}
         self._graph_pool = None
+        self._device_tokens = None          # the step's tokens that live on the device (see `step`)
+        self._tok_pin: Optional[torch.Tensor] = None
+        self._tok_pin_free = None
         # widest block table a request can have: the fixed width of a recorded step's tables
         self._max_table = max(1, -(-model.spec.max_positions // self.page_size))
         self.graph_replays = 0
@@ -215,11 +218,51 @@ class ModelRunner:
             arena.index_fill_(0, idx, 0)
 
     # ---- the step -----------------------------------------------------------------
-    def step(self, entries: Sequence[StepEntry], reserved: bool = False) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], reserved: bool = False,
+             device_tokens: Optional[Tuple[torch.Tensor, Sequence[int], Sequence[int]]] = None) -> torch.Tensor:
         """Runs the entries' tokens as one batch.  Returns float32 [wanted, vocab] in the
         order of the entries and of each entry's `want`.  With `reserved` the caller (the
         scheduler) has reserved the pages already and also records afterwards that the
-        tokens are in the cache; without it this call does both."""
+        tokens are in the cache; without it this call does both.
+        `device_tokens` = (ids, places, rows): tokens that are not known on the host yet.  The
+        token at place `places[i]` of the step's tokens (counted over all entries, in order) is
+        `ids[rows[i]]`, an int32 tensor on the device that an earlier step's sampling wrote (the
+        entries hold any valid id there); it is put in place on the device, in stream order, and
+        nothing waits for it."""
+        self._device_tokens = device_tokens
+        try:
+            return self._step(entries, reserved)
+        finally:
+            self._device_tokens = None
+
+    def _put_device_tokens(self, ids: torch.Tensor) -> None:
+        """Overwrites the places of `ids` (the step's token ids on the device) that `step` was
+        given device tokens for."""
+        if self._device_tokens is None:
+            return
+        src, places, rows = self._device_tokens
+        n = len(places)
+        if n == 0:
+            return
+        if max(places) >= ids.numel() or max(rows) >= src.numel() or min(places) < 0 or min(rows) < 0:
+            raise StepError("a device token's place or row is outside the step")
+        if n == ids.numel() == src.numel() and list(places) == list(rows) == list(range(n)):
+            ids.copy_(src)               # every token, in order: the usual step of decoding requests
+            return
+        # the two index arrays go up through pinned memory (a copy from ordinary memory would wait for the GPU)
+        if self._tok_pin is None or self._tok_pin.numel() < 2 * n:
+            self._tok_pin = torch.empty((max(1024, 2 * n),), dtype=torch.int64, pin_memory=True)
+        if self._tok_pin_free is not None:
+            self._tok_pin_free.synchronize()
+        host = self._tok_pin[:2 * n].view(2, n)
+        host.copy_(torch.tensor([list(places), list(rows)], dtype=torch.int64))
+        idx = torch.empty((2, n), dtype=torch.int64, device=self.device)
+        idx.copy_(host, non_blocking=True)
+        self._tok_pin_free = torch.cuda.Event()
+        self._tok_pin_free.record()
+        ids.index_copy_(0, idx[0], src.index_select(0, idx[1]))
+
+    def _step(self, entries: Sequence[StepEntry], reserved: bool) -> torch.Tensor:
         spec = self.model.spec
         if not entries:
             return torch.empty((0, spec.vocab_size), dtype=torch.float32, device=self.device)
@@ -299,6 +342,7 @@ class ModelRunner:
             logits = self._replay_decode(arrays, ids32, rows32)
         else:
             ctx, ids, want_rows, _, _ = self._context(arrays, ids32, rows32)
+            self._put_device_tokens(ids)
             logits = self.model.forward(ids, ctx, self.layer_caches, want_rows)
         if not reserved:
             self.cache.commit_many(rid_arr, counts_arr)
@@ -341,6 +385,7 @@ class ModelRunner:
         self._staging.push(torch.int32, n32, g.dev32)
         self._staging.push(torch.int64, n64, g.dev64)
         self._staging.mark()
+        self._put_device_tokens(g.dev32[:B])        # the token ids lead the 32-bit arrays
         g.graph.replay()
         self.graph_replays += 1
         if not reserved:
@@ -424,8 +469,10 @@ class ModelRunner:
             self._seen[key] = self._seen.get(key, 0) + 1
             if self._seen[key] < self.graph_after:         # not yet: launch by launch
                 ctx, ids, want_rows, _, _ = self._context(a, ids32, rows32)
+                self._put_device_tokens(ids)
                 return self.model.forward(ids, ctx, self.layer_caches, want_rows)
             ctx, ids, want, d32, d64 = self._context(a, ids32, all_rows, max_ctx_len=bucket, host_lengths=False)
+            self._put_device_tokens(ids)
             every_row = torch.arange(B, dtype=torch.int32, device=self.device)
             cur = torch.cuda.current_stream(self.device)
             side = torch.cuda.Stream(self.device)
@@ -445,6 +492,7 @@ class ModelRunner:
         else:
             self._used(g, key)
             self._upload(a, ids32, all_rows, g.dev32, g.dev64)
+            self._put_device_tokens(g.dev32[:B])
         g.graph.replay()
         self.graph_replays += 1
         if rows32.size == B and np.array_equal(rows32, np.arange(B)):

@@ -110,6 +110,8 @@ class Sampler:
         self.device = torch.device(device)
         lib = kernels.lib()
         self._lib = lib
+        self._pin: Optional[torch.Tensor] = None
+        self._pin_free = None
 
     def argmax(self, logits: torch.Tensor) -> torch.Tensor:
         kernels._dev(logits)
@@ -132,14 +134,36 @@ class Sampler:
         """logits float32 [R, V] (changed in place when penalties apply); one strategy and
         one uniform number per row; `recent[r]` = the tokens the row's penalties count
         (`penalty_context`).  Returns R token ids."""
+        return self.sample_device(logits, strategies, uniforms, recent).tolist()
+
+    def _params(self, rows: Sequence[Sequence[float]]) -> torch.Tensor:
+        """Per-row numbers as a float32 tensor [len(rows), R] on the device, by way of pinned memory:
+        a copy from ordinary memory makes the host wait for the GPU's earlier work."""
+        n, R = len(rows), len(rows[0])
+        if self._pin is None or self._pin.numel() < n * R:
+            self._pin = torch.empty((max(1024, n * R),), dtype=torch.float32, pin_memory=True)
+        if self._pin_free is not None:
+            self._pin_free.synchronize()         # the copy before has left the buffer
+        host = self._pin[:n * R].view(n, R)
+        host.copy_(torch.tensor(rows, dtype=torch.float32))
+        out = torch.empty((n, R), dtype=torch.float32, device=self.device)
+        out.copy_(host, non_blocking=True)
+        self._pin_free = torch.cuda.Event()
+        self._pin_free.record()
+        return out
+
+    def sample_device(self, logits: torch.Tensor, strategies: Sequence[Strategy], uniforms: Sequence[float],
+                      recent: Optional[Sequence[Sequence[int]]] = None) -> torch.Tensor:
+        """`sample` without the copy to the host: the R token ids as an int32 tensor on the device;
+        nothing here waits for the GPU (unless penalties apply)."""
         kernels._dev(logits)
         kernels._want(logits, torch.float32, "sample: logits")
         R, V = logits.shape
         if R != len(strategies) or R != len(uniforms):
             raise kernels.KernelError("sample: one strategy and one uniform number per row are needed")
-        if R == 0:
-            return []
         dev = logits.device
+        if R == 0:
+            return torch.empty((0,), dtype=torch.int32, device=dev)
         if recent is not None and any(penalties_apply(s, rc) for s, rc in zip(strategies, recent)):
             n = PENALTY_CONTEXT
             rec = np.full((R, n), -1, dtype=np.int32)
@@ -154,25 +178,24 @@ class Sampler:
             kernels._ok(self._lib.xi_apply_penalties(kernels._p(logits), R, V, kernels._p(rec_d), n,
                                                      kernels._p(fr_d), kernels._p(pr_d), kernels._stream()))
         if all(s.greedy for s in strategies):
-            return self.argmax(logits).tolist()
+            return self.argmax(logits)
         chunks = int(self._lib.xi_sample_topk_chunks(V))
         if chunks > 0 and all(s.greedy or 1 <= s.top_k <= TOPK_FAST for s in strategies):
             # a small top-k everywhere (the default strategy has 32): the k most probable of a row
             # are found by many workgroups, the rest is about k numbers
-            par = torch.tensor([[s.temperature for s in strategies], [float(s.top_k) for s in strategies],
-                                [s.top_p for s in strategies], list(uniforms)], dtype=torch.float32).to(dev)
+            par = self._params([[s.temperature for s in strategies], [float(s.top_k) for s in strategies],
+                                [s.top_p for s in strategies], list(uniforms)])
             cand_v = torch.empty((R, chunks, TOPK_FAST), dtype=torch.float32, device=dev)
             cand_i = torch.empty((R, chunks, TOPK_FAST), dtype=torch.int32, device=dev)
             out = torch.empty((R,), dtype=torch.int32, device=dev)
             kernels._ok(self._lib.xi_sample_topk(kernels._p(logits), R, V, kernels._p(par), kernels._p(cand_v),
                                                  kernels._p(cand_i), kernels._p(out), kernels._stream()))
-            return out.tolist()
-        t = torch.tensor([s.temperature for s in strategies], dtype=torch.float32, device=dev)
-        k = torch.tensor([s.top_k for s in strategies], dtype=torch.int32, device=dev)
-        p = torch.tensor([s.top_p for s in strategies], dtype=torch.float32, device=dev)
-        u = torch.tensor(list(uniforms), dtype=torch.float32, device=dev)
+            return out
+        t, kf, p, u = self._params([[s.temperature for s in strategies], [float(s.top_k) for s in strategies],
+                                    [s.top_p for s in strategies], list(uniforms)])
+        k = kf.to(torch.int32)              # (a row's top_k is far below 2^24: exact as float32)
         probs = torch.empty_like(logits)
         out = torch.empty((R,), dtype=torch.int32, device=dev)
         kernels._ok(self._lib.xi_sample(kernels._p(logits), R, V, kernels._p(t), kernels._p(k), kernels._p(p),
                                         kernels._p(u), kernels._p(probs), kernels._p(out), kernels._stream()))
-        return out.tolist()
+        return out
