@@ -1,6 +1,7 @@
 """Tiny Qwen3 configurations for tests.  A and B differ in every size and option; W adds
 a sliding window on some layers (two cache groups), a head size that is no power of
-two and biases on the q, k and v projections; all have widths and vocabularies that are
+two and biases on the q, k and v projections; Y scales its rotation (YaRN) and rotates half of
+a head; all have widths and vocabularies that are
 no power of two where they can."""
 
 def _cfg(**kw):
@@ -36,6 +37,18 @@ TINY["O"] = dict(
                 head_dim=16, intermediate_size=182, vocab_size=257, rope_theta=777.0,
                 rms_norm_eps=3e-6, tie_word_embeddings=True, max_position_embeddings=256),
     seed=5, linear_std=0.04, norm_std=0.15, page_size=8)
+
+# Y: YaRN scaling over a given original length (so the model runs further than
+# max_position_embeddings: round(40 * 4) = 160 positions), with bounds of the blend that fall
+# inside its 8 frequencies, and half of every head rotated.
+TINY["Y"] = dict(
+    config=_cfg(num_hidden_layers=2, hidden_size=72, num_attention_heads=6, num_key_value_heads=3,
+                head_dim=32, intermediate_size=104, vocab_size=211, rope_theta=5000.0,
+                rms_norm_eps=2e-6, tie_word_embeddings=True, max_position_embeddings=64,
+                partial_rotary_factor=0.5,
+                rope_scaling=dict(rope_type="yarn", factor=4.0, original_max_position_embeddings=40,
+                                  beta_fast=4.0, beta_slow=1.0, attn_factor=1.25)),
+    seed=8, linear_std=0.05, norm_std=0.1, page_size=16)
 
 
 # Real layer sizes (Qwen3-0.6B, 4B, 8B, 14B and 32B) with few layers and a small vocabulary: the

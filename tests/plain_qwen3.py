@@ -77,17 +77,107 @@ def rope_tables(theta: float, rot: int, max_pos: int):
     return freqs.cos(), freqs.sin()
 
 
+def _f32(v) -> torch.Tensor:
+    return torch.tensor(v, dtype=torch.float32)
+
+
+def scaled_rope_tables(c: dict):
+    """cos and sin [positions, rot / 2] under config.json's `rope_scaling` (or `rope_parameters`)
+    and `partial_rotary_factor`, after ScalingRotaryEmbedding::new,
+    /root/reference/src/models/layers/rotary_emb.rs:126-415 and (YaRN) 440-540.  rot =
+    int(partial_rotary_factor * head_dim) (:138-141).  The length the model was trained at is
+    `original_max_position_embeddings`, else max_position_embeddings / factor, else
+    max_position_embeddings (:152-166).  Rows: the positions the model can run, which for YaRN
+    over a given original length is round(original * factor) if that is more
+    (/root/reference/src/utils/mod.rs:873-897); the reference builds more rows than it can reach."""
+    d, theta, max_pos = c["head_dim"], float(c["rope_theta"]), int(c["max_position_embeddings"])
+    rot = int(c["partial_rotary_factor"] * d) if c.get("partial_rotary_factor") is not None else d
+    rs = c.get("rope_scaling") or c.get("rope_parameters")
+    kind = None if rs is None else rs.get("rope_type", rs.get("type"))
+    if kind in (None, "default"):
+        return rope_tables(theta, rot, max_pos)
+    factor = rs.get("factor")
+    if rs.get("original_max_position_embeddings") is not None:
+        orig = float(rs["original_max_position_embeddings"])
+    elif factor is not None:
+        orig = max_pos / float(factor)
+    else:
+        orig = float(max_pos)
+
+    def plain_inv(base: float):          # :116-121
+        return [_f32(1.0) / torch.tensor(base ** (i / rot), dtype=torch.float64).to(torch.float32) for i in range(0, rot, 2)]
+
+    rows, mscale = max_pos, None
+    if kind == "linear":                 # :172-206: the tensor of frequencies times (f32)(1 / factor)
+        inv = [f * _f32(1.0 / float(factor)) for f in plain_inv(theta)]
+    elif kind == "llama3":               # :208-282
+        lo, hi = float(rs["low_freq_factor"]), float(rs["high_freq_factor"])
+        low_wavelen, high_wavelen = _f32(orig / lo), _f32(orig / hi)
+        inv = []
+        for f in plain_inv(theta):
+            wavelen = _f32(2.0) * _f32(math.pi) / f
+            if wavelen < high_wavelen:
+                inv.append(f)
+            elif wavelen > low_wavelen:
+                inv.append(f / _f32(float(factor)))
+            else:
+                smooth = (_f32(orig) / wavelen - _f32(lo)) / _f32(hi - lo)
+                inv.append((_f32(1.0) - smooth) * f / _f32(float(factor)) + smooth * f)
+    elif kind == "dynamic":              # :284-335
+        if rs.get("alpha") is not None:
+            base = (theta * float(rs["alpha"])) ** (rot / (rot - 2))
+        else:
+            fct = float(factor)
+            max_len = int(orig * fct)
+            base = (theta * ((fct * max_len / orig) - (fct - 1.0))) ** (rot / (rot - 2))
+        inv = plain_inv(base)
+    elif kind == "yarn":                 # :336-401 and 482-540: everything in float32
+        fct = _f32(float(factor))
+        beta_fast, beta_slow = float(rs.get("beta_fast", 32.0)), float(rs.get("beta_slow", 1.0))
+        extrapolation, attn = float(rs.get("extrapolation_factor", 1.0)), float(rs.get("attn_factor", 1.0))
+        base = _f32(theta)
+        pw = [torch.pow(base, _f32(float(i)) / _f32(float(rot))) for i in range(0, rot, 2)]
+        extra = [_f32(1.0) / p_ for p_ in pw]
+        inter = [_f32(1.0) / (fct * p_) for p_ in pw]
+
+        def correction_dim(num_rot: float):      # :441-449
+            return (_f32(float(rot)) * torch.log(_f32(orig) / (_f32(num_rot) * _f32(2.0) * _f32(math.pi)))) / (_f32(2.0) * torch.log(base))
+
+        low = max(float(torch.floor(correction_dim(beta_fast))), 0.0)            # :451-463
+        high = min(float(torch.ceil(correction_dim(beta_slow))), rot - 1.0)
+        if low == high:                                                            # :465-468
+            high += 0.001
+        inv = []
+        for j in range(rot // 2):
+            ramp = torch.clamp((_f32(float(j)) - _f32(low)) * _f32(1.0 / (high - low)), 0.0, 1.0)
+            mask = (_f32(1.0) - ramp) * _f32(extrapolation)
+            inv.append(inter[j] * (_f32(1.0) - mask) + extra[j] * mask)
+        mscale = (_f32(1.0) if float(fct) <= 1.0 else _f32(0.1) * torch.log(fct) + _f32(1.0)) * _f32(attn)   # :474-479, 531
+        if rs.get("original_max_position_embeddings") is not None and float(factor) > 1.0:
+            rows = max(max_pos, int(round(orig * float(factor))))
+    else:
+        raise ValueError(f"Unknown rope_type: {kind}")
+    inv_freq = torch.stack([torch.as_tensor(f, dtype=torch.float32) for f in inv])
+    freqs = torch.arange(rows, dtype=torch.float32)[:, None] * inv_freq[None, :]
+    cos, sin = freqs.cos(), freqs.sin()
+    if mscale is not None:
+        cos, sin = cos * mscale, sin * mscale
+    return cos, sin
+
+
 def apply_rope(x: torch.Tensor, positions: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
-    """Non-interleaved ("neox") rotation: for i < d/2,
-    o[i] = x[i]*cos - x[i+d/2]*sin;  o[i+d/2] = x[i]*sin + x[i+d/2]*cos.
-    x: [T, heads, d].  Golden formula of the reference's own probe:
+    """Non-interleaved ("neox") rotation of the first rot = 2 * cos.shape[1] dims: for i < rot/2,
+    o[i] = x[i]*cos - x[i+rot/2]*sin;  o[i+rot/2] = x[i]*sin + x[i+rot/2]*cos; dims from rot on
+    pass unchanged.  x: [T, heads, d].  Golden formula of the reference's own probe:
     /root/reference/tests/probes/compare_attention_misc_probe.py:33-49 (else branch);
-    Qwen3 uses this layout (is_rope_i = false, /root/reference/src/utils/mod.rs:2303)."""
+    Qwen3 uses this layout (is_rope_i = false, /root/reference/src/utils/mod.rs:2303).  The partial
+    form is applied by a kernel outside the reference's tree (rotary_emb.rs:87-98): rotating the
+    leading dims is the convention of the models that have the factor; parity unpinned."""
     c = cos[positions].to(x.dtype)[:, None, :]
     s = sin[positions].to(x.dtype)[:, None, :]
-    h = x.shape[-1] // 2
-    a, b = x[..., :h], x[..., h:]
-    return torch.cat([a * c - b * s, a * s + b * c], dim=-1)
+    h = cos.shape[-1]
+    a, b, rest = x[..., :h], x[..., h:2 * h], x[..., 2 * h:]
+    return torch.cat([a * c - b * s, a * s + b * c, rest], dim=-1)
 
 
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: Optional[int] = None,
@@ -174,7 +264,7 @@ def model_logits(c: dict, W: Dict[str, torch.Tensor], ids: List[int], start: int
     tied).  /root/reference/src/models/qwen3.rs:311-374."""
     dtype = W["model.embed_tokens.weight"].dtype
     d = c["head_dim"]
-    cos, sin = rope_tables(float(c["rope_theta"]), d, c["max_position_embeddings"])
+    cos, sin = scaled_rope_tables(c)
     positions = torch.arange(start, start + len(ids))
     x = W["model.embed_tokens.weight"][torch.tensor(ids)]
     for i in range(c["num_hidden_layers"]):

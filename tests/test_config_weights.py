@@ -42,7 +42,16 @@ def test_defaults_follow_the_reference():
     (dict(num_key_value_heads=3), "multiple"),
     (dict(head_dim=15), "even"),
     (dict(hidden_act="gelu"), "hidden_act"),
-    (dict(rope_scaling={"rope_type": "yarn", "factor": 4.0}), "rope_scaling"),
+    (dict(rope_scaling={"rope_type": "su", "factor": 4.0}), "Unknown rope_type: su"),
+    (dict(rope_scaling={"rope_type": "yarn"}), "yarn rope_type requires factor"),
+    (dict(rope_scaling={"type": "linear"}), "Linear rope_type requires factor"),
+    (dict(rope_scaling={"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0}), "Llama3 rope_type requires"),
+    (dict(rope_scaling={"rope_type": "dynamic"}), "Dynamic rope_type requires either alpha or factor"),
+    (dict(rope_scaling={"rope_type": "yarn", "factor": "4"}), "rope_scaling.factor"),
+    (dict(rope_scaling={"rope_type": "yarn", "factor": -1.0}), "positive"),
+    (dict(rope_scaling=[1, 2]), "rope_scaling"),
+    (dict(partial_rotary_factor=1.5), "partial_rotary_factor"),
+    (dict(partial_rotary_factor=0.1), "even number"),
     (dict(sliding_window=0), "sliding_window"),
     (dict(layer_types=["full_attention"]), "layer_types"),
     (dict(hidden_size="64"), "integer"),
@@ -248,3 +257,61 @@ def test_bench_refuses_more_than_one_gpu():
     assert r.returncode == 2
     lines = [l for l in r.stdout.splitlines() if l.strip()]
     assert len(lines) == 1 and "one GPU" in lines[0]
+
+
+# ---- rope scaling ----------------------------------------------------------------------------
+ROPE_SCALINGS = [
+    (dict(rope_type="yarn", factor=4.0, original_max_position_embeddings=32), None),
+    (dict(type="yarn", factor=8.0, beta_fast=16, beta_slow=2, attn_factor=1.3, extrapolation_factor=0.9), 0.5),
+    (dict(rope_type="linear", factor=3.0), None),
+    (dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=16), None),
+    (dict(rope_type="dynamic", factor=2.5), 0.75),
+    (dict(rope_type="dynamic", alpha=3.0), None),
+    (dict(rope_type="default"), None),
+    (None, 0.25),
+]
+
+
+@pytest.mark.parametrize("scaling,partial", ROPE_SCALINGS)
+def test_rope_scaling_tables_are_the_plain_ones(scaling, partial):
+    """The position encoding part alone, on the CPU: for every kind of rope_scaling and a partial
+    rotation its tables equal the plain implementation's, which is written from the reference
+    on its own (tests/plain_qwen3.py: scaled_rope_tables), and the model's positions are the
+    table's rows."""
+    import torch
+    import plain_qwen3 as plain
+    from xinfer_amd.parts import position_encoding_class
+    raw = dict(TINY["A"]["config"], max_position_embeddings=128)
+    if scaling is not None:
+        raw["rope_scaling"] = scaling
+    if partial is not None:
+        raw["partial_rotary_factor"] = partial
+    fam, cfg = config_from_dict(raw)
+    spec = fam.build_spec(cfg)
+    pe = spec.layers[0].mixer["position"]
+    part = position_encoding_class(pe.kind)(pe, torch.float32)
+    part.load(None, "", "cpu")
+    cos, sin = plain.scaled_rope_tables(dict(raw))
+    assert part.cos.shape == cos.shape == (spec.max_positions, int((partial or 1.0) * 32) // 2)
+    assert torch.equal(part.cos, cos) and torch.equal(part.sin, sin)
+    assert part.rotary_dim == 2 * cos.shape[1] and part.head_dim == 32
+    # the configuration survives being written out and read again
+    assert config_from_dict(cfg.to_dict())[1] == cfg
+
+
+def test_yarn_scaling_factor_option():
+    """The option puts YaRN over the file's own length in place of whatever the file says, with the
+    derived parameters of /root/reference/src/utils/mod.rs:806-871: beta_fast 32 up to a factor of
+    4 and 32 sqrt(factor / 4) beyond, the extrapolation factor 1 + 0.05 sqrt(factor - 8) above 8;
+    the model then runs round(length * factor) positions."""
+    from xinfer_amd.config.model_config import derive_yarn_scaling
+    _, cfg = config_from_dict(dict(TINY["A"]["config"], rope_scaling=dict(rope_type="linear", factor=2.0)))
+    assert cfg.positions == 128
+    y = cfg.with_yarn_scaling(4.0)
+    rs = y.rope_scaling
+    assert (rs.kind, rs.factor, rs.original_max_position_embeddings, rs.beta_fast, rs.beta_slow,
+            rs.extrapolation_factor, rs.attn_factor) == ("yarn", 4.0, 128.0, 32.0, 1.0, 1.0, 1.0)
+    assert y.positions == 512 and y.max_position_embeddings == 128
+    big = derive_yarn_scaling(16.0, 4096)
+    assert big.beta_fast == 64.0 and abs(big.extrapolation_factor - (1 + 0.05 * 8 ** 0.5)) < 1e-12
+    assert derive_yarn_scaling(0.5, 4096).factor == 1.0          # a factor below 1 is 1

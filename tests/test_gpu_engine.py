@@ -231,6 +231,33 @@ def test_running_ahead_gives_the_same_tokens(model_dirs):
     assert rids[1] not in eng._finished and eng.runner.cache.free_pages(0) == 200
 
 
+def test_yarn_scaling_factor_stretches_the_positions(model_dirs):
+    """`yarn_scaling_factor=2` (the reference's --yarn-scaling-factor) on the model of 128 positions:
+    prompts of 150 and 200 tokens are taken, and the greedy tokens are those of the plain model under
+    the rope_scaling that the option stands for (YaRN over 128 positions, beta_fast 32, beta_slow 1);
+    without the option such a prompt is refused."""
+    from xinfer_amd import SamplingParams
+    rng = random.Random(6)
+    prompts = [harness.random_prompt(rng, n, 256) for n in (150, 200, 9)]
+    sp = SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True)
+    with pytest.raises(ValueError, match="max_model_len"):
+        _engine(model_dirs["A"], "A", "f32", max_num_seqs=4, num_pages=40).generate(prompts, sp)
+    eng = _engine(model_dirs["A"], "A", "f32", max_num_seqs=4, num_pages=40, prefill_chunk_size=64, yarn_scaling_factor=2.0)
+    assert eng.max_model_len == 256 and eng.model.spec.max_positions == 256
+    outs = eng.generate(prompts, sp)
+    pm = plain.PlainModel(model_dirs["A"])
+    pm.config["rope_scaling"] = dict(rope_type="yarn", factor=2.0, original_max_position_embeddings=128,
+                                     beta_fast=32.0, beta_slow=1.0, extrapolation_factor=1.0, attn_factor=1.0)
+    for p, o in zip(prompts, outs):
+        ids = list(p)
+        for tok in o.token_ids:
+            lg = pm.logits(ids)[-1]
+            assert float(lg.max() - lg[tok]) < 1e-4
+            ids.append(tok)
+    plain_unscaled = plain.PlainModel(model_dirs["A"]).logits(prompts[2])
+    assert not torch.allclose(pm.logits(prompts[2]), plain_unscaled, atol=1e-3)      # the scaling is at work from the start
+
+
 def test_eos_and_limits(model_dirs):
     from xinfer_amd import SamplingParams
     eng = _engine(model_dirs["A"], "A", "f32", max_num_seqs=2, num_pages=16, max_model_len=40)

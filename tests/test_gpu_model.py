@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 
 DTYPES = ["float32", "bfloat16"]
 LENGTHS = {"A": [5, 17, 33, 100, 128], "B": [1, 9, 64, 130, 200], "W": [3, 24, 25, 77, 150, 61],
-           "O": [2, 31, 70, 129, 8]}
+           "O": [2, 31, 70, 129, 8], "Y": [4, 64, 65, 160, 41, 100]}
 
 
 def _requests(name):

@@ -72,6 +72,110 @@ def test_rope_on_the_reference_probe_shapes():
                 assert torch.allclose(out[t, h, i + 4], q[t, h, i] * s + q[t, h, i + 4] * c)
 
 
+def _scaled(scaling=None, **kw):
+    c = dict(head_dim=128, rope_theta=1e6, max_position_embeddings=4096)
+    c.update(kw)
+    if scaling is not None:
+        c["rope_scaling"] = scaling
+    return plain.scaled_rope_tables(c)
+
+
+def test_rope_scaling_linear_and_dynamic_reduce_to_plain_tables():
+    """Linear scaling by a power of two puts the plain table's row p at row factor * p, exactly
+    (a product with the factor instead of its inverse fails); dynamic scaling is the plain table of
+    a larger base, (theta * alpha)^(rot / (rot - 2)) or, from a factor, the value of the NTK rule at
+    the scaled length (/root/reference/src/models/layers/rotary_emb.rs:172-206, 284-335)."""
+    cos0, sin0 = plain.rope_tables(1e6, 128, 4096)
+    cos, sin = _scaled(dict(rope_type="linear", factor=4.0))
+    assert cos.shape == cos0.shape
+    assert torch.equal(cos[0:4096:4], cos0[:1024]) and torch.equal(sin[0:4096:4], sin0[:1024])
+    assert not torch.equal(cos[:1024], cos0[:1024])
+    cos, sin = _scaled(dict(type="dynamic", alpha=3.0))
+    want = plain.rope_tables((1e6 * 3.0) ** (128 / 126), 128, 4096)
+    assert torch.equal(cos, want[0]) and torch.equal(sin, want[1])
+    # from a factor: the original length is max / factor = 1024, the scaled one 4096
+    cos, sin = _scaled(dict(rope_type="dynamic", factor=4.0))
+    want = plain.rope_tables((1e6 * (4.0 * 4096 / 1024 - 3.0)) ** (128 / 126), 128, 4096)
+    assert torch.equal(cos, want[0]) and torch.equal(sin, want[1])
+    assert torch.equal(_scaled(dict(rope_type="default"))[0], cos0) and torch.equal(_scaled(None)[0], cos0)
+    with pytest.raises(ValueError, match="Unknown rope_type"):
+        _scaled(dict(rope_type="su", factor=2.0))
+
+
+def test_rope_scaling_llama3_bands():
+    """With the published parameters of that rule (factor 8, low 1, high 4 over 8,192 positions,
+    base 500,000) wavelengths under 2,048 positions keep their frequency, those over 8,192 have an
+    eighth of it, and the ratio falls from one to the other in between: a blend the wrong way
+    round jumps at both edges (/root/reference/src/models/layers/rotary_emb.rs:208-282)."""
+    c = dict(head_dim=128, rope_theta=500000.0, max_position_embeddings=16384,
+             rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                               original_max_position_embeddings=8192))
+    cos, sin = plain.scaled_rope_tables(c)
+    cos0, sin0 = plain.rope_tables(500000.0, 128, 16384)
+    ang, ang0 = torch.atan2(sin[1], cos[1]).double(), torch.atan2(sin0[1], cos0[1]).double()     # row 1 holds the frequencies
+    ratio = ang / ang0
+    wavelen = 2 * math.pi / ang0
+    assert torch.all(ratio[wavelen < 2048] == 1.0) and int((wavelen < 2048).sum()) > 10
+    assert torch.allclose(ratio[wavelen > 8192], torch.tensor(0.125, dtype=torch.float64), rtol=1e-5) and int((wavelen > 8192).sum()) > 10
+    mid = (wavelen >= 2048) & (wavelen <= 8192)
+    assert int(mid.sum()) >= 3
+    r = ratio[mid]
+    assert torch.all(r[1:] < r[:-1]) and float(r[0]) < 1.0 and float(r[-1]) > 0.125
+    # continuous at the edges: the first blended ratio is near 1, the last near 1/8
+    smooth = (8192 / wavelen[mid] - 1.0) / 3.0
+    assert torch.allclose(r, (1 - smooth) / 8 + smooth, rtol=1e-4)
+
+
+def test_rope_scaling_yarn_bands_and_magnitude():
+    """Qwen3's own long-context setting (base 1e6, head size 128, factor 4 over 32,768 positions):
+    the blend runs over frequencies 23 to 40 (floor and ceil of 128 ln(32768 / (2 pi b)) / (2 ln 1e6)
+    for b = 32 and 1).  Below it a frequency stays as it is, above it is a quarter, at 31 it is
+    9/17 + (8/17)/4 of itself; cos and sin are scaled by 0.1 ln 4 + 1, times attn_factor.  A ramp the
+    wrong way round, a missing magnitude or an original length taken for the scaled one fails
+    (/root/reference/src/models/layers/rotary_emb.rs:336-401, 440-540)."""
+    rs = dict(rope_type="yarn", factor=4.0, original_max_position_embeddings=32768)
+    c = dict(head_dim=128, rope_theta=1e6, max_position_embeddings=40960, rope_scaling=rs)
+    cos, sin = plain.scaled_rope_tables(c)
+    assert cos.shape == (131072, 64)              # round(32768 * 4) positions, more than max_position_embeddings
+    m = 0.1 * math.log(4.0) + 1.0
+    assert torch.allclose(cos[:4096] ** 2 + sin[:4096] ** 2, torch.full((4096, 64), m * m), rtol=1e-5)
+    cos0, sin0 = plain.rope_tables(1e6, 128, 8)
+    freq = torch.atan2(sin[1], cos[1]).double()                      # the angle of position 1
+    freq0 = torch.atan2(sin0[1], cos0[1]).double()
+    ratio = freq / freq0
+    assert torch.allclose(ratio[:24], torch.ones(24, dtype=torch.float64), rtol=1e-5)
+    assert torch.allclose(ratio[40:], torch.full((24,), 0.25, dtype=torch.float64), rtol=1e-5)
+    assert abs(float(ratio[31]) - (9 / 17 + (8 / 17) / 4)) < 1e-5
+    assert torch.all(ratio[24:40][1:] < ratio[24:40][:-1])
+    # attn_factor multiplies the magnitude; a factor of 1 is plain RoPE (to the float32 power's rounding)
+    cos_a, _ = plain.scaled_rope_tables(dict(c, rope_scaling=dict(rs, attn_factor=1.5)))
+    assert torch.allclose(cos_a[:64], cos[:64] * 1.5, rtol=1e-6)
+    one = plain.scaled_rope_tables(dict(c, rope_scaling=dict(rope_type="yarn", factor=1.0)))
+    ref = plain.rope_tables(1e6, 128, 40960)
+    assert one[0].shape == ref[0].shape and torch.allclose(one[0][:512], ref[0][:512], atol=2e-4)
+    # without an original length it is max / factor, and the table keeps max_position_embeddings rows
+    short = plain.scaled_rope_tables(dict(c, max_position_embeddings=131072, rope_scaling=dict(rope_type="yarn", factor=4.0)))
+    assert short[0].shape == (131072, 64) and torch.equal(short[0][:1000], cos[:1000])
+
+
+def test_partial_rotary_leaves_the_rest_of_a_head_alone(tmp_path):
+    """partial_rotary_factor 0.5 of a head of 32: 8 frequencies, dims 16.. pass unchanged and
+    dims (i, i + 8) turn together; and a whole model under YaRN and partial rotation still gives
+    the same logits wherever the sequence starts (only distances count, also with the scaled
+    magnitude)."""
+    cos, sin = plain.scaled_rope_tables(dict(head_dim=32, rope_theta=1e4, max_position_embeddings=64, partial_rotary_factor=0.5))
+    assert cos.shape == (64, 8) and torch.equal(cos, plain.rope_tables(1e4, 16, 64)[0])
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(3, 2, 32, generator=g, dtype=torch.float64)
+    out = plain.apply_rope(x, torch.tensor([5, 9, 60]), cos.double(), sin.double())
+    assert torch.equal(out[..., 16:], x[..., 16:]) and not torch.allclose(out[..., :16], x[..., :16])
+    assert torch.allclose(out[..., :8] ** 2 + out[..., 8:16] ** 2, x[..., :8] ** 2 + x[..., 8:16] ** 2)
+    pm = _tiny_weights("Y", tmp_path)
+    ids = [5, 77, 200, 41, 9, 150, 123, 8]
+    assert torch.allclose(pm.logits(ids), plain.model_logits(pm.config, pm.weights, ids, start=140), atol=2e-4)
+    assert plain.scaled_rope_tables(pm.config)[0].shape == (160, 8)
+
+
 def test_attention_is_the_library_routine():
     g = torch.Generator().manual_seed(10)
     T, nq, nkv, d = 12, 6, 2, 8

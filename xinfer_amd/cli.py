@@ -39,6 +39,8 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--prefill-chunk-size", type=int, default=8192,
                    help="most prompt tokens of one request in a step")
     p.add_argument("--disable-cuda-graph", action="store_true", help="disable HIP graph replay of decode steps")
+    p.add_argument("--yarn-scaling-factor", type=float, default=None,
+                   help="stretch the model's positions by this factor with YaRN")
     p.add_argument("--i", dest="interactive", action="store_true",
                    help="interactive chat: prompts are read line by line, the conversation so far is the context")
     p.add_argument("--page-size", type=int, default=64, help="tokens per cache page")
@@ -85,7 +87,8 @@ def run(args) -> int:
         model_id=args.m, weight_path=args.w, max_num_seqs=max_num_seqs, max_model_len=max_model_len,
         max_tokens=min(args.max_tokens, max_model_len), generation_cfg=gen_cfg, seed=args.seed,
         kv_fraction=args.kv_fraction, prefill_chunk_size=args.prefill_chunk_size,
-        disable_cuda_graph=args.disable_cuda_graph, page_size=args.page_size, num_pages=args.num_pages)
+        disable_cuda_graph=args.disable_cuda_graph, page_size=args.page_size, num_pages=args.num_pages,
+        yarn_scaling_factor=args.yarn_scaling_factor)
     engine = LLMEngine(cfg, args.dtype)
     params = SamplingParams(temperature=args.temperature, top_k=args.top_k, top_p=args.top_p,
                             frequency_penalty=args.frequency_penalty,

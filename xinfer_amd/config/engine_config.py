@@ -75,13 +75,14 @@ class EngineConfig:
     model_id: Optional[str] = None          # a local model folder (there is no hub download here)
     weight_path: Optional[str] = None       # the same, under the reference's legacy name
     max_num_seqs: int = 32                  # most requests live at a time
-    max_model_len: Optional[int] = None     # default: the model's max_position_embeddings
+    max_model_len: Optional[int] = None     # default: the positions the model can encode (max_position_embeddings, more under YaRN)
     max_tokens: Optional[int] = None        # default per request: 16384, clipped to max_model_len
     generation_cfg: Optional[GenerationConfig] = None
     seed: Optional[int] = None
     kv_fraction: Optional[float] = None     # share of free GPU memory given to the cache (0.6)
     prefill_chunk_size: int = 8192          # most prompt tokens of one request in a step (any >= 1)
     disable_cuda_graph: bool = False        # the reference's name; here it disables HIP graphs
+    yarn_scaling_factor: Optional[float] = None   # YaRN over the model's own length, in place of its rope_scaling
     # --- this engine's own ---
     page_size: int = 64                     # tokens per cache page (the reference fixes 64)
     num_pages: Union[int, List[int], None] = None   # pages of every cache group, or one count per group; default: from kv_fraction

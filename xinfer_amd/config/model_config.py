@@ -69,6 +69,96 @@ def _typed(v, key: str, typ, where: str):
     raise TypeError(typ)
 
 
+ROPE_SCALING_KINDS = ("default", "linear", "llama3", "dynamic", "yarn")
+
+
+@dataclass(frozen=True)
+class RopeScaling:
+    """config.json's `rope_scaling` (or `rope_parameters`), typed.  The kinds and their keys are
+    those of the reference's ScalingRotaryEmbedding::new
+    (/root/reference/src/models/layers/rotary_emb.rs:126-415): "linear" (factor), "llama3"
+    (factor, low_freq_factor, high_freq_factor), "dynamic" (alpha, or factor), "yarn" (factor;
+    beta_fast 32, beta_slow 1, extrapolation_factor 1, attn_factor 1 unless given); "default" is
+    plain RoPE.  `original_max_position_embeddings` as the file gives it, or None."""
+    kind: str
+    factor: Optional[float] = None
+    original_max_position_embeddings: Optional[float] = None
+    low_freq_factor: Optional[float] = None
+    high_freq_factor: Optional[float] = None
+    alpha: Optional[float] = None
+    beta_fast: float = 32.0
+    beta_slow: float = 1.0
+    extrapolation_factor: float = 1.0
+    attn_factor: float = 1.0
+
+    @classmethod
+    def from_dict(cls, raw: Any, where: str) -> Optional["RopeScaling"]:
+        if raw is None:
+            return None
+        if not isinstance(raw, dict):
+            raise ConfigError(f"{where}: 'rope_scaling' must be an object")
+        kind = raw.get("rope_type", raw.get("type"))       # rotary_emb.rs:146-150
+        if kind is None and "rope_theta" in raw and len(raw) == 1:
+            return None                                        # `rope_parameters` that only repeats the base
+        if not isinstance(kind, str):
+            raise ConfigError(f"{where}: rope_scaling needs a string 'rope_type'")
+        if kind not in ROPE_SCALING_KINDS:
+            raise ConfigError(f"{where}: Unknown rope_type: {kind} (known: {', '.join(ROPE_SCALING_KINDS)})")
+
+        def num(key, default=None):
+            v = raw.get(key)
+            return default if v is None else _typed(v, f"rope_scaling.{key}", float, where)
+
+        rs = cls(kind=kind, factor=num("factor"),
+                 original_max_position_embeddings=num("original_max_position_embeddings"),
+                 low_freq_factor=num("low_freq_factor"), high_freq_factor=num("high_freq_factor"),
+                 alpha=num("alpha"), beta_fast=num("beta_fast", 32.0), beta_slow=num("beta_slow", 1.0),
+                 extrapolation_factor=num("extrapolation_factor", 1.0), attn_factor=num("attn_factor", 1.0))
+        if kind == "linear" and rs.factor is None:
+            raise ConfigError(f"{where}: Linear rope_type requires factor to be set")
+        if kind == "llama3" and None in (rs.factor, rs.low_freq_factor, rs.high_freq_factor):
+            raise ConfigError(f"{where}: Llama3 rope_type requires factor, low_freq_factor, high_freq_factor to be set")
+        if kind == "llama3" and rs.high_freq_factor == rs.low_freq_factor:
+            raise ConfigError(f"{where}: llama3 rope_type needs high_freq_factor and low_freq_factor to differ")
+        if kind == "dynamic" and rs.alpha is None and rs.factor is None:
+            raise ConfigError(f"{where}: Dynamic rope_type requires either alpha or factor to be set")
+        if kind == "yarn" and rs.factor is None:
+            raise ConfigError(f"{where}: yarn rope_type requires factor to be set")
+        for key in ("factor", "alpha", "original_max_position_embeddings"):
+            v = getattr(rs, key)
+            if v is not None and not v > 0.0:
+                raise ConfigError(f"{where}: rope_scaling.{key} must be positive, got {v}")
+        return rs
+
+    def to_dict(self) -> Dict[str, Any]:
+        out: Dict[str, Any] = {"rope_type": self.kind}
+        defaults = RopeScaling(self.kind)
+        for f in fields(self):
+            v = getattr(self, f.name)
+            if f.name != "kind" and v is not None and v != getattr(defaults, f.name):
+                out[f.name] = v
+        return out
+
+    def original_positions(self, max_position_embeddings: int) -> float:
+        """The length the model was trained at: as given, else max / factor, else max (rotary_emb.rs:152-166)."""
+        if self.original_max_position_embeddings is not None:
+            return self.original_max_position_embeddings
+        if self.factor is not None:
+            return max_position_embeddings / self.factor
+        return float(max_position_embeddings)
+
+
+def derive_yarn_scaling(factor: float, max_position_embeddings: int) -> RopeScaling:
+    """The `rope_scaling` that the reference's --yarn-scaling-factor option puts in place of the
+    file's (/root/reference/src/utils/mod.rs:806-871): YaRN over the file's length, beta_fast grown
+    with sqrt(factor / 4) and the extrapolation factor a little above 1 for large factors."""
+    factor = max(float(factor), 1.0)
+    beta_fast = 32.0 if factor <= 4.0 else 32.0 * (factor / 4.0) ** 0.5
+    extrapolation = 1.0 + 0.05 * (factor - 8.0) ** 0.5 if factor > 8.0 else 1.0
+    return RopeScaling("yarn", factor=factor, original_max_position_embeddings=float(max_position_embeddings),
+                       beta_fast=beta_fast, beta_slow=1.0, extrapolation_factor=extrapolation, attn_factor=1.0)
+
+
 @dataclass(frozen=True)
 class Qwen3Config:
     """Qwen3 dense (`Qwen3ForCausalLM`).
@@ -81,7 +171,9 @@ class Qwen3Config:
     ("load the bias if the tensor exists" in the reference; here an explicit flag,
     default false as in Qwen3 checkpoints), `sliding_window` (passed to every
     layer when present, qwen3.rs:46) and `layer_types`, which restricts the window
-    to the layers it names "sliding_attention".
+    to the layers it names "sliding_attention"; `rope_scaling` (see `RopeScaling`) and
+    `partial_rotary_factor` (the first int(factor * head_dim) dims of a head are rotated,
+    rotary_emb.rs:138-141).
     """
     vocab_size: int
     hidden_size: int
@@ -100,6 +192,8 @@ class Qwen3Config:
     layer_types: Optional[Tuple[str, ...]] = None
     eos_token_id: Optional[Tuple[int, ...]] = None
     bos_token_id: Optional[int] = None
+    rope_scaling: Optional[RopeScaling] = None
+    partial_rotary_factor: Optional[float] = None
     architecture: str = "Qwen3ForCausalLM"
 
     # ---- construction -------------------------------------------------
@@ -136,14 +230,10 @@ class Qwen3Config:
         sw = raw.get("sliding_window")
         if sw is not None:
             sw = _typed(sw, "sliding_window", int, where)
-        scaling = raw.get("rope_scaling", raw.get("rope_parameters"))
-        if scaling is not None:
-            kind = None
-            if isinstance(scaling, dict):
-                kind = scaling.get("rope_type", scaling.get("type"))
-            if kind not in (None, "default"):
-                raise ConfigError(
-                    f"{where}: rope_scaling of type {kind!r} is not supported (plain RoPE only)")
+        scaling = RopeScaling.from_dict(raw.get("rope_scaling", raw.get("rope_parameters")), where)
+        prf = raw.get("partial_rotary_factor")
+        if prf is not None:
+            prf = _typed(prf, "partial_rotary_factor", float, where)
         cfg = cls(
             vocab_size=_typed(raw["vocab_size"], "vocab_size", int, where),
             hidden_size=h,
@@ -167,6 +257,8 @@ class Qwen3Config:
             eos_token_id=eos_t,
             bos_token_id=_typed(raw["bos_token_id"], "bos_token_id", int, where)
             if raw.get("bos_token_id") is not None else None,
+            rope_scaling=scaling,
+            partial_rotary_factor=prf,
             architecture=raw.get("architectures", ["Qwen3ForCausalLM"])[0],
         )
         cfg.validate(where)
@@ -192,6 +284,14 @@ class Qwen3Config:
             raise ConfigError(f"{where}: rms_norm_eps must not be negative")
         if self.rope_theta <= 0.0:
             raise ConfigError(f"{where}: rope_theta must be positive")
+        if self.partial_rotary_factor is not None:
+            if not (0.0 < self.partial_rotary_factor <= 1.0):
+                raise ConfigError(f"{where}: partial_rotary_factor must be in (0, 1], got {self.partial_rotary_factor}")
+            if self.rotary_dim < 2 or self.rotary_dim % 2:
+                raise ConfigError(f"{where}: partial_rotary_factor {self.partial_rotary_factor} of head_dim "
+                                  f"{self.head_dim} gives {self.rotary_dim} rotated dims; an even number of at least 2 is needed")
+        if self.rope_scaling is not None and self.rope_scaling.kind == "dynamic" and self.rotary_dim <= 2:
+            raise ConfigError(f"{where}: dynamic rope scaling needs more than 2 rotated dims")
         if self.sliding_window is not None and self.sliding_window <= 0:
             raise ConfigError(f"{where}: sliding_window must be positive or null")
         if self.layer_types is not None:
@@ -213,11 +313,42 @@ class Qwen3Config:
             if f.name == "architecture":
                 continue
             v = getattr(self, f.name)
+            if f.name in ("rope_scaling", "partial_rotary_factor") and v is None:
+                continue
+            if isinstance(v, RopeScaling):
+                v = v.to_dict()
             if isinstance(v, tuple):
                 v = list(v)
             if f.name == "eos_token_id" and v is not None and len(v) == 1:
                 v = v[0]
             out[f.name] = v
+        return out
+
+    @property
+    def rotary_dim(self) -> int:
+        """Dims of a head that are rotated (rotary_emb.rs:138-141)."""
+        if self.partial_rotary_factor is None:
+            return self.head_dim
+        return int(self.partial_rotary_factor * self.head_dim)
+
+    @property
+    def positions(self) -> int:
+        """Positions the model can encode.  YaRN over a given original length reaches
+        round(original * factor) if that is more than max_position_embeddings
+        (effective_max_position_embeddings, /root/reference/src/utils/mod.rs:873-897)."""
+        rs = self.rope_scaling
+        if (rs is not None and rs.kind == "yarn" and rs.factor is not None and rs.factor > 1.0
+                and rs.original_max_position_embeddings is not None):
+            return max(self.max_position_embeddings, int(round(rs.original_max_position_embeddings * rs.factor)))
+        return self.max_position_embeddings
+
+    def with_yarn_scaling(self, factor: float) -> "Qwen3Config":
+        """The configuration under the --yarn-scaling-factor option: YaRN over this file's length,
+        in place of whatever rope_scaling the file has (apply_runtime_rope_overrides,
+        /root/reference/src/utils/mod.rs:862-869)."""
+        import dataclasses
+        out = dataclasses.replace(self, rope_scaling=derive_yarn_scaling(factor, self.max_position_embeddings))
+        out.validate("config.json with yarn_scaling_factor")
         return out
 
     def window_of_layer(self, i: int) -> Optional[int]:

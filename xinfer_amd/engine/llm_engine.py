@@ -76,7 +76,7 @@ class LLMEngine:
         if model is None:
             self.dtype = parse_dtype(dtype)
             model_dir = econfig.model_dir()
-            self.model = load_model(model_dir, self.dtype, econfig.device)
+            self.model = load_model(model_dir, self.dtype, econfig.device, econfig.yarn_scaling_factor)
         else:
             model_dir = None
             self.model = model

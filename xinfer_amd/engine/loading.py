@@ -26,8 +26,14 @@ def parse_dtype(name) -> torch.dtype:
         raise ValueError(f"dtype {name!r} is not supported (bf16/bfloat16 or f32/float32)") from None
 
 
-def load_model(model_dir: str, dtype, device="cuda:0") -> CausalLM:
+def load_model(model_dir: str, dtype, device="cuda:0", yarn_scaling_factor: Optional[float] = None) -> CausalLM:
+    """`yarn_scaling_factor`: stretch the model's positions by this factor with YaRN, whatever the
+    folder's config.json says about rope scaling (the reference's --yarn-scaling-factor)."""
     fam, cfg = load_config(model_dir)
+    if yarn_scaling_factor is not None:
+        if not hasattr(cfg, "with_yarn_scaling"):
+            raise ValueError(f"yarn_scaling_factor: the {fam.name} family has no rope scaling to set")
+        cfg = cfg.with_yarn_scaling(float(yarn_scaling_factor))
     store = SafetensorsStore(model_dir)
     try:
         return build_model(cfg, store, dtype, device)

@@ -23,9 +23,16 @@ def qwen3_spec_for(cfg: Qwen3Config, tensor_names) -> ModelSpec:
 
 def qwen3_spec(cfg: Qwen3Config, prefix: str = "model.", tied=None) -> ModelSpec:
     tied = cfg.tie_word_embeddings if tied is None else bool(tied)
-    rope = PartSpec("rope", dict(
-        head_dim=cfg.head_dim, rotary_dim=cfg.head_dim, theta=cfg.rope_theta,
-        max_positions=cfg.max_position_embeddings, interleaved=False))
+    rope_params = dict(head_dim=cfg.head_dim, rotary_dim=cfg.rotary_dim, theta=cfg.rope_theta,
+                       max_positions=cfg.positions, interleaved=False)
+    rs = cfg.rope_scaling
+    if rs is not None and rs.kind != "default":
+        rope_params["scaling"] = dict(
+            kind=rs.kind, original=rs.original_positions(cfg.max_position_embeddings), factor=rs.factor,
+            low_freq_factor=rs.low_freq_factor, high_freq_factor=rs.high_freq_factor, alpha=rs.alpha,
+            beta_fast=rs.beta_fast, beta_slow=rs.beta_slow, extrapolation_factor=rs.extrapolation_factor,
+            attn_factor=rs.attn_factor)
+    rope = PartSpec("rope", rope_params)
     layers = []
     for i in range(cfg.num_hidden_layers):
         layer_prefix = f"{prefix}layers.{i}"
@@ -47,7 +54,7 @@ def qwen3_spec(cfg: Qwen3Config, prefix: str = "model.", tied=None) -> ModelSpec
         architecture=cfg.architecture,
         vocab_size=cfg.vocab_size,
         hidden_size=cfg.hidden_size,
-        max_positions=cfg.max_position_embeddings,
+        max_positions=cfg.positions,
         embedding=PartSpec("embedding", dict(
             name=f"{prefix}embed_tokens.weight", vocab_size=cfg.vocab_size, dim=cfg.hidden_size)),
         layers=tuple(layers),
