@@ -226,7 +226,10 @@ def attention_block(x, W, prefix, c, positions, cos, sin, window):
     q = x @ W[f"{prefix}.q_proj.weight"].T
     k = x @ W[f"{prefix}.k_proj.weight"].T
     v = x @ W[f"{prefix}.v_proj.weight"].T
-    if c.get("attention_bias"):
+    has = c.get("qkv_bias") if c.get("qkv_bias") is not None else c.get("attention_bias")
+    if has is None:                      # neither key: the biases are taken if they are there (attention.rs:472-476, 388-399)
+        has = f"{prefix}.q_proj.bias" in W
+    if has:
         q = q + W[f"{prefix}.q_proj.bias"]
         k = k + W[f"{prefix}.k_proj.bias"]
         v = v + W[f"{prefix}.v_proj.bias"]

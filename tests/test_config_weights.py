@@ -51,6 +51,8 @@ def test_defaults_follow_the_reference():
     (dict(rope_scaling={"rope_type": "yarn", "factor": -1.0}), "positive"),
     (dict(rope_scaling=[1, 2]), "rope_scaling"),
     (dict(partial_rotary_factor=1.5), "partial_rotary_factor"),
+    (dict(attn_logit_softcapping=30.0), "attn_logit_softcapping"),
+    (dict(attn_output_gate=True), "attn_output_gate"),
     (dict(partial_rotary_factor=0.1), "even number"),
     (dict(sliding_window=0), "sliding_window"),
     (dict(layer_types=["full_attention"]), "layer_types"),
@@ -315,3 +317,28 @@ def test_yarn_scaling_factor_option():
     big = derive_yarn_scaling(16.0, 4096)
     assert big.beta_fast == 64.0 and abs(big.extrapolation_factor - (1 + 0.05 * 8 ** 0.5)) < 1e-12
     assert derive_yarn_scaling(0.5, 4096).factor == 1.0          # a factor below 1 is 1
+
+
+def test_biases_follow_the_checkpoint_when_the_config_is_silent(tmp_path):
+    """`qkv_bias` goes before `attention_bias`; with neither key the q, k and v biases are taken if
+    the checkpoint has them (/root/reference/src/models/layers/attention.rs:472-476, 388-399): the
+    same tensors give a model with biases under a config.json without the key, one without them
+    (and three ignored tensors a layer) when the key says false."""
+    from xinfer_amd.engine.loading import build_model
+    raw = dict(TINY["W"]["config"])
+    assert raw["attention_bias"] is True
+    d = write_random_model(str(tmp_path / "w"), raw, seed=2)
+    store = SafetensorsStore(d)
+    silent = {k: v for k, v in raw.items() if k != "attention_bias"}
+    fam, cfg = config_from_dict(silent)
+    assert cfg.attention_bias is None
+    assert fam.spec(cfg, store.names()).layers[0].mixer["bias"] is True
+    assert fam.spec(cfg, [n for n in store.names() if not n.endswith(".bias")]).layers[0].mixer["bias"] is False
+    assert fam.build_spec(cfg).layers[0].mixer["bias"] is False                     # random weights: none
+    assert config_from_dict(dict(silent, qkv_bias=True, attention_bias=False))[1].attention_bias is True
+    assert config_from_dict(dict(silent, qkv_bias=False, attention_bias=True))[1].attention_bias is False
+    with_bias = build_model(cfg, store, "f32", device="cpu")
+    assert with_bias.ignored_tensors == [] and with_bias.blocks[0].mixer.qkv_bias is not None
+    _, off = config_from_dict(dict(silent, attention_bias=False))
+    without = build_model(off, store, "f32", device="cpu")
+    assert len(without.ignored_tensors) == 3 * raw["num_hidden_layers"] and without.blocks[0].mixer.qkv_bias is None

@@ -251,3 +251,32 @@ def test_extra_tensors_and_a_checkpoint_without_prefix_give_the_same_logits(mode
     assert torch.equal(logits(str(bare), 8), logits(str(tied), 8))
     ref = plain.PlainModel(str(tied)).logits(toks)
     assert float((logits(str(bare), 8) - ref).abs().max()) < harness.TOL["float32"] * float(ref.abs().max())
+
+
+def test_a_config_that_is_silent_about_biases_takes_the_checkpoints(model_dirs, tmp_path):
+    """Configuration W's folder with `attention_bias` taken out of config.json: the q, k and v
+    biases in the checkpoint are used all the same (/root/reference/src/models/layers/attention.rs:
+    472-476, 388-399), the logits are those of the folder that names them, and the plain model's."""
+    import json
+    import shutil
+    from xinfer_amd.engine import ModelRunner, StepEntry, load_model
+    toks = harness.random_prompt(random.Random(4), 50, 300)
+
+    def logits(folder):
+        runner = ModelRunner(load_model(folder, "float32", "cuda:0"), page_size=16, num_pages=[8, 8], max_requests=1)
+        runner.add_request(0)
+        return runner.step([StepEntry(0, toks, list(range(len(toks))))]).cpu()
+
+    silent = tmp_path / "silent"
+    silent.mkdir()
+    with open(model_dirs["W"] + "/config.json") as f:
+        raw = json.load(f)
+    assert raw.pop("attention_bias") is True
+    (silent / "config.json").write_text(json.dumps(raw))
+    shutil.copy(model_dirs["W"] + "/model.safetensors", silent / "model.safetensors")
+    got = logits(str(silent))
+    assert torch.equal(got, logits(model_dirs["W"]))
+    ref = plain.PlainModel(str(silent)).logits(toks)
+    assert float((got - ref).abs().max()) < harness.TOL["float32"] * float(ref.abs().max())
+    (silent / "config.json").write_text(json.dumps(dict(raw, qkv_bias=False)))
+    assert not torch.allclose(logits(str(silent)), got, atol=1e-3)          # switched off, the biases are missed

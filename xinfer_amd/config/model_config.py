@@ -167,9 +167,10 @@ class Qwen3Config:
     counts, hidden size, layer count, eps, max positions and activation.  Optional
     keys and their defaults: `head_dim = hidden_size / num_attention_heads`
     (attention.rs:446), `rope_theta = 10000` (rotary_emb.rs:49),
-    `tie_word_embeddings = false` (qwen3.rs:200-209), `attention_bias`
-    ("load the bias if the tensor exists" in the reference; here an explicit flag,
-    default false as in Qwen3 checkpoints), `sliding_window` (passed to every
+    `tie_word_embeddings = false` (qwen3.rs:200-209), `qkv_bias` or else `attention_bias`
+    (when neither is given the reference loads the q, k and v biases if the checkpoint has them,
+    attention.rs:472-476 and 388-399: here None, decided by the tensors' names when a
+    checkpoint is read and off for random weights), `sliding_window` (passed to every
     layer when present, qwen3.rs:46) and `layer_types`, which restricts the window
     to the layers it names "sliding_attention"; `rope_scaling` (see `RopeScaling`) and
     `partial_rotary_factor` (the first int(factor * head_dim) dims of a head are rotated,
@@ -186,7 +187,7 @@ class Qwen3Config:
     rms_norm_eps: float
     rope_theta: float = 10000.0
     tie_word_embeddings: bool = False
-    attention_bias: bool = False
+    attention_bias: Optional[bool] = None
     hidden_act: str = "silu"
     sliding_window: Optional[int] = None
     layer_types: Optional[Tuple[str, ...]] = None
@@ -230,6 +231,12 @@ class Qwen3Config:
         sw = raw.get("sliding_window")
         if sw is not None:
             sw = _typed(sw, "sliding_window", int, where)
+        # what the reference's attention reads of a configuration and this engine does not compute
+        # (attention.rs:477-481, 698): refused rather than left out of the result
+        if raw.get("attn_logit_softcapping") is not None:
+            raise ConfigError(f"{where}: attn_logit_softcapping is not supported")
+        if raw.get("attn_output_gate"):
+            raise ConfigError(f"{where}: attn_output_gate is not supported")
         scaling = RopeScaling.from_dict(raw.get("rope_scaling", raw.get("rope_parameters")), where)
         prf = raw.get("partial_rotary_factor")
         if prf is not None:
@@ -248,8 +255,9 @@ class Qwen3Config:
                               else 10000.0, "rope_theta", float, where),
             tie_word_embeddings=_typed(raw["tie_word_embeddings"], "tie_word_embeddings", bool, where)
             if raw.get("tie_word_embeddings") is not None else False,
-            attention_bias=_typed(raw["attention_bias"], "attention_bias", bool, where)
-            if raw.get("attention_bias") is not None else False,
+            attention_bias=_typed(raw["qkv_bias"], "qkv_bias", bool, where) if raw.get("qkv_bias") is not None
+            else _typed(raw["attention_bias"], "attention_bias", bool, where) if raw.get("attention_bias") is not None
+            else None,
             hidden_act=_typed(raw.get("hidden_act", raw.get("hidden_activation", "silu")),
                               "hidden_act", str, where),
             sliding_window=sw,

@@ -16,13 +16,19 @@ def qwen3_spec_for(cfg: Qwen3Config, tensor_names) -> ModelSpec:
     anywhere and no head of its own: the reference then reads every tensor without the prefix
     and ties the head to the table (embedding checkpoints, qwen3.rs:200-209)."""
     names = set(tensor_names)
+    # a configuration that says nothing about biases takes them if the checkpoint has them
+    # (attention.rs:472-476, 388-399)
+    bias = cfg.attention_bias
+    if bias is None:
+        bias = any(n.endswith(".self_attn.q_proj.bias") for n in names)
     if "embed_tokens.weight" in names and "model.embed_tokens.weight" not in names:
-        return qwen3_spec(cfg, prefix="", tied=True)
-    return qwen3_spec(cfg)
+        return qwen3_spec(cfg, prefix="", tied=True, bias=bias)
+    return qwen3_spec(cfg, bias=bias)
 
 
-def qwen3_spec(cfg: Qwen3Config, prefix: str = "model.", tied=None) -> ModelSpec:
+def qwen3_spec(cfg: Qwen3Config, prefix: str = "model.", tied=None, bias=None) -> ModelSpec:
     tied = cfg.tie_word_embeddings if tied is None else bool(tied)
+    bias = bool(cfg.attention_bias) if bias is None else bool(bias)
     rope_params = dict(head_dim=cfg.head_dim, rotary_dim=cfg.rotary_dim, theta=cfg.rope_theta,
                        max_positions=cfg.positions, interleaved=False)
     rs = cfg.rope_scaling
@@ -39,7 +45,7 @@ def qwen3_spec(cfg: Qwen3Config, prefix: str = "model.", tied=None) -> ModelSpec
         mixer = PartSpec("attention", dict(
             hidden_size=cfg.hidden_size, num_heads=cfg.num_attention_heads,
             num_kv_heads=cfg.num_key_value_heads, head_dim=cfg.head_dim,
-            bias=cfg.attention_bias, qk_norm=True, qk_norm_eps=cfg.rms_norm_eps,
+            bias=bias, qk_norm=True, qk_norm_eps=cfg.rms_norm_eps,
             window=cfg.window_of_layer(i), position=rope,
             scale=float(cfg.head_dim) ** -0.5))
         ffn = PartSpec("gated_mlp", dict(
