@@ -56,7 +56,7 @@ WORKLOADS = {
     "long32b": dict(model=QWEN3_32B, name="Qwen3-32B layer sizes", requests=16, prompt=(8192, 8192), new_tokens=512,
                     chunk=2048, max_model_len=8704),
 }
-FULL_LAYERS = QWEN3_8B["num_hidden_layers"]
+MODELS = {"0.6b": QWEN3_0_6B, "8b": QWEN3_8B, "14b": QWEN3_14B, "32b": QWEN3_32B}
 CONTEXT = 4096
 PREFILL_TOKENS = 2048
 
@@ -194,6 +194,8 @@ def main() -> int:
                     help="context length at the end of the decode run (default: the contract's)")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
                     help="length of the prefilled prompt (default: the contract's)")
+    ap.add_argument("--model", choices=sorted(MODELS), default="8b",
+                    help="layer sizes of the decode and prefill runs (default: the contract's Qwen3-8B)")
     ap.add_argument("--skip-points", action="store_true", help="only the default decode run")
     ap.add_argument("--only", choices=["all", "decode", "prefill"], default="all",
                     help="run one phase only (for profiling); the JSON line then lacks the other")
@@ -209,8 +211,10 @@ def main() -> int:
         return 2
     if args.workload != "decode":
         return serve(args.workload, args.layers, not args.no_run_ahead)
+    full_layers = MODELS[args.model]["num_hidden_layers"]
+    model_name = {"0.6b": "Qwen3-0.6B", "8b": "Qwen3-8B", "14b": "Qwen3-14B", "32b": "Qwen3-32B"}[args.model]
     if args.layers is None:
-        args.layers = FULL_LAYERS
+        args.layers = full_layers
     CONTEXT, PREFILL_TOKENS = args.context, args.prefill_tokens     # the sizes of this run
 
     import torch
@@ -220,7 +224,7 @@ def main() -> int:
     from xinfer_amd.weights.random_init import random_store_for
 
     dev = "cuda:0"
-    raw = dict(QWEN3_8B, num_hidden_layers=args.layers)
+    raw = dict(MODELS[args.model], num_hidden_layers=args.layers)
     _, cfg = config_from_dict(raw)
     store = random_store_for(cfg, seed=0, linear_std=0.02, norm_std=0.1)
     t0 = time.time()
@@ -231,7 +235,7 @@ def main() -> int:
     page = 64
     max_batch = 8 if (args.skip_points or args.only != "all") else 64
     max_batch = max(max_batch, args.batch)
-    num_pages = max_batch * (CONTEXT // page) + PREFILL_TOKENS // page + 8
+    num_pages = max_batch * (-(-CONTEXT // page)) + -(-PREFILL_TOKENS // page) + 8
     runner = ModelRunner(model, page_size=page, num_pages=num_pages, max_requests=max_batch + 1)
     g = torch.Generator(device=dev)
     g.manual_seed(1)
@@ -298,14 +302,14 @@ def main() -> int:
     step_bytes = wb + args.batch * mean_ctx * kvb
     achieved = step_bytes / sec / 1e9
     out = {
-        "metric": "decode tok/s at batch 8, Qwen3-8B bf16", "value": round(args.batch / sec, 2),
+        "metric": f"decode tok/s at batch {args.batch}, {model_name} bf16", "value": round(args.batch / sec, 2),
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic: seeded random weights, uniform random token ids, random cache contents",
         "config": {
-            "model": "Qwen3-8B layer sizes", "global_batch": args.batch, "seq_len": CONTEXT,
-            "parallelism": "single GPU", "layers": args.layers, "layers_of_model": FULL_LAYERS,
+            "model": f"{model_name} layer sizes", "global_batch": args.batch, "seq_len": CONTEXT,
+            "parallelism": "single GPU", "layers": args.layers, "layers_of_model": full_layers,
             "hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size,
             "num_attention_heads": cfg.num_attention_heads, "num_key_value_heads": cfg.num_key_value_heads,
             "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size, "rope_theta": cfg.rope_theta,

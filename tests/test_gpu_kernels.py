@@ -421,6 +421,31 @@ def test_linear_mid_gated(M, N, K):
             kernels.linear_mid_gated(x.to(DEV), w.to(DEV), torch.ones((M, 4), device=DEV), 1e-5)
 
 
+@pytest.mark.parametrize("M", [1, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K,features", [(17408, 256, None), (25600, 128, None), (300, 320, 100), (129, 64, 128), (4100, 512, 65)])
+def test_linear_mid_gated_wide_tile(M, N, K, features):
+    """The gated product with up to 128 features a workgroup (a tile of 256 rows of w): chosen by
+    itself from 17 to 64 rows where 64 features would make two rounds of workgroups (intermediate
+    sizes of 17,408 and 25,600: 68 and 100 features), and forced here at other widths: a last
+    workgroup of few features, waves without any, a single workgroup."""
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(14)
+    x = _rand((M, K), torch.bfloat16, g)
+    w = _rand((2 * N, K), torch.bfloat16, g, 0.05)
+    gate, up = x.double() @ w[:N].double().T, x.double() @ w[N:].double().T
+    ref = gate / (1 + torch.exp(-gate)) * up
+    if features is None:
+        chosen = int(kernels.lib().xi_linear_mid_gated_features(N, M))
+        assert chosen == ({17408: 68, 25600: 100}[N] if M > 16 else {17408: 34, 25600: 50}[N])
+    y = kernels.linear_mid_gated(x.to(DEV), w.to(DEV), features=features)
+    assert (y.cpu().double() - ref).abs().max() / ref.abs().max() < 2.0 ** -8
+    narrow = kernels.linear_mid_gated(x.to(DEV), w.to(DEV), features=32)
+    assert (y.float() - narrow.float()).abs().max() <= 2.0 ** -7 * ref.abs().max()      # the sums' order differs, no more
+    if features is not None:
+        with pytest.raises(kernels.KernelError, match="up to 64 rows"):
+            kernels.linear_mid_gated(_rand((65, K), torch.bfloat16, g).to(DEV), w.to(DEV), features=features)
+
+
 def test_linear_skinny_plan_fills_the_compute_units():
     """The shapes the streaming product chooses: grids that are multiples of the 256 compute
     units where the width allows (a workgroup may own a number of features that is no multiple

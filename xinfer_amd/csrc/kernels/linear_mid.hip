@@ -29,7 +29,10 @@
 // one pass over w at any M up to 128, where the streaming kernel's workgroups (16 to 50
 // features) re-read x from L2 more the more rows there are.  FOLD: x is the first half of a
 // folded RMSNorm (see linear_skinny.hip): the rows of the product are multiplied by
-// rsqrt(sum of the row's parts / K + eps) before the activation.
+// rsqrt(sum of the row's parts / K + eps) before the activation.  WR = 8: a tile of 256 rows of w,
+// R <= 128 features a workgroup (up to 64 rows of x): where 64 features make two rounds of
+// workgroups (intermediate sizes above 16,384) one round of twice the features reads x from L2
+// half as often; at 17 to 64 rows, where x is as many bytes as a workgroup's share of w.
 //
 // Reference call site: candle matmul in /root/reference/src/models/layers/linear.rs:76-124
 // (vendor BLAS).
@@ -47,6 +50,7 @@ constexpr int kMidLdsRow = kMidK + 8;  // elements of a row in LDS
 constexpr int kMidDepth = 2;           // tiles whose loads are in flight (the default; measured: more gain nothing)
 constexpr int kMidTile = 128 * kMidLdsRow;   // elements of one operand's tile in LDS
 constexpr size_t kMidLdsBytes = 2 * 2 * (size_t)kMidTile * sizeof(bf16) + 16 * sizeof(float);
+constexpr size_t kMidWideLdsBytes = 2 * 3 * (size_t)kMidTile * sizeof(bf16) + 16 * sizeof(float);   // WR = 8
 constexpr int kMidSsLoads = 32;        // 16 threads x 32 loads: up to 512 parts of a row's sum of squares
 
 struct MidFold {
@@ -59,19 +63,23 @@ struct MidFold {
 // D: tiles whose loads are in flight.  FULL: up to 128 rows of x, the four waves take a quarter
 // of the tile each (64 rows of w by 64 rows of x); else up to 16 * TJ <= 64 rows of x and a wave
 // takes a quarter of the rows of w (32) by all rows of x.  GATED, FOLD: see the head of the file.
-template <int D, int TJ, bool FULL, bool GATED, bool FOLD>
+template <int D, int TJ, bool FULL, bool GATED, bool FOLD, int WR = 4>
 __global__ __launch_bounds__(256, 1) void linear_mid_kernel(const bf16* __restrict__ x,
                                                             const bf16* __restrict__ w, void* __restrict__ yv,
                                                             int M, int N, int K, int ks, size_t slice_stride,
                                                             int R, int rotate, MidFold fold) {
   static_assert(!FULL || TJ == 4, "the full form multiplies 64 rows of x per wave");
   static_assert(!FOLD || (GATED && !FULL && TJ == 1), "a folded norm: the gated form, up to 16 rows");
+  static_assert(WR == 4 || (WR == 8 && GATED && !FULL && !FOLD), "the tile of 256 rows of w: the gated form, up to 64 rows of x");
+  constexpr int WROWS = 32 * WR;                      // rows of the w tile
+  constexpr int HALF = WROWS / 2;                     // GATED: so many gate rows, then as many up rows
+  constexpr int WT = WROWS * kMidLdsRow;              // elements of the w tile in LDS (the x tile: kMidTile)
   extern __shared__ __align__(16) unsigned char mid_smem[];
-  bf16* lds = reinterpret_cast<bf16*>(mid_smem);   // [buffer][w tile | x tile][128][kMidLdsRow]
-  float* inv_s = reinterpret_cast<float*>(mid_smem + 2 * 2 * (size_t)kMidTile * sizeof(bf16));   // [16]
+  bf16* lds = reinterpret_cast<bf16*>(mid_smem);   // [buffer][w tile [WROWS] | x tile [128]][kMidLdsRow]
+  float* inv_s = reinterpret_cast<float*>(mid_smem + 2 * (size_t)(WT + kMidTile) * sizeof(bf16));   // [16]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, j = lane >> 4;
-  constexpr int TI = FULL ? 4 : 2;                    // 16-row tiles of w a wave multiplies
+  constexpr int TI = FULL ? 4 : WR / 2;               // 16-row tiles of w a wave multiplies
   constexpr int TG = GATED ? TI / 2 : TI;             // of them gate tiles (the others: their up tiles)
   constexpr int XI = FULL ? 4 : (TJ == 4 ? 2 : 1);    // 32-row groups of x that are copied
   const int wf = FULL ? (wave & 1) : wave;            // which of the wave's shares of the features,
@@ -100,21 +108,21 @@ __global__ __launch_bounds__(256, 1) void linear_mid_kernel(const bf16* __restri
     }
   }
 
-  // ---- copying: a tile is 128 rows of 8 16-byte chunks; thread t moves chunk t % 8 of rows
+  // ---- copying: a tile is 128 rows (of w: WROWS) of 8 16-byte chunks; thread t moves chunk t % 8 of rows
   // t / 8 + 32 i.  Row q of the w tile is feature n0 + q (GATED: the gate row of feature
-  // n0 + q % 64 for q < 64, its up row for q >= 64); rows past the workgroup's last feature read
+  // n0 + q % HALF for q < HALF, its up row for q >= HALF); rows past the workgroup's last feature read
   // that feature's row again and rows of x past M row M - 1 (the same address many times in one
   // instruction costs one access); their results are dropped.  No load is conditional, so the
   // counter of loads in flight is exact and only the tile that is needed is waited for.
   const int srow = tid >> 3, skc = tid & 7;
-  const bf16* wsrc[4];
+  const bf16* wsrc[WR];
   const bf16* xsrc[XI];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < WR; ++i) {
     const int row = srow + 32 * i;
-    int n = n0 + (GATED ? (row & 63) : row);
+    int n = n0 + (GATED ? (row & (HALF - 1)) : row);
     n = n < n_last ? n : n_last;
-    if (GATED && row >= 64) n += N;
+    if (GATED && row >= HALF) n += N;
     wsrc[i] = w + (size_t)n * K + (size_t)kt0 * kMidK + 8 * skc;
   }
 #pragma unroll
@@ -123,7 +131,7 @@ __global__ __launch_bounds__(256, 1) void linear_mid_kernel(const bf16* __restri
     xsrc[i] = x + (size_t)(row < M ? row : M - 1) * K + (size_t)kt0 * kMidK + 8 * skc;
   }
   const int sdst = srow * kMidLdsRow + 8 * skc;
-  bf16x8 wr[D][4], xr[D][XI];
+  bf16x8 wr[D][WR], xr[D][XI];
 
   // a wave whose rows of x lie past M, or whose features past the workgroup's, has nothing to do
   const int wave_row0 = GATED ? 16 * TG * wf : 16 * TI * wf;     // its first feature within the workgroup
@@ -138,7 +146,7 @@ __global__ __launch_bounds__(256, 1) void linear_mid_kernel(const bf16* __restri
   do {                                                                                \
     int tt_ = (t) + start;                                                            \
     tt_ = tt_ >= nkt ? tt_ - nkt : tt_;                                               \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                     \
+    _Pragma("unroll") for (int i = 0; i < WR; ++i)                                    \
       wr[slot][i] = *reinterpret_cast<const bf16x8*>(wsrc[i] + (size_t)tt_ * kMidK);  \
     _Pragma("unroll") for (int i = 0; i < XI; ++i)                                    \
       xr[slot][i] = *reinterpret_cast<const bf16x8*>(xsrc[i] + (size_t)tt_ * kMidK);  \
@@ -155,14 +163,14 @@ __global__ __launch_bounds__(256, 1) void linear_mid_kernel(const bf16* __restri
   // products.  One barrier a tile is enough: whoever writes this buffer again, two tiles on, has
   // passed the next tile's barrier, which every thread reaches only after these products.
   // Row of the w tile of the wave's tile ti: its features' rows; GATED: gate tiles first, then
-  // the up tiles of the same features, 64 rows further.
+  // the up tiles of the same features, HALF rows further.
   int buf = 0;
-#define XI_MID_WROW(ti) (GATED ? (((ti) / TG) * 64 + wave_row0 + 16 * ((ti) % TG)) : (wave_row0 + 16 * (ti)))
+#define XI_MID_WROW(ti) (GATED ? (((ti) / TG) * HALF + wave_row0 + 16 * ((ti) % TG)) : (wave_row0 + 16 * (ti)))
 #define XI_MID_TILE(s, t)                                                                                 \
   do {                                                                                                    \
-    bf16* Ws = lds + buf * (2 * kMidTile);                                                                \
-    bf16* Xs = Ws + kMidTile;                                                                             \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                         \
+    bf16* Ws = lds + buf * (WT + kMidTile);                                                               \
+    bf16* Xs = Ws + WT;                                                                                   \
+    _Pragma("unroll") for (int i = 0; i < WR; ++i)                                                        \
       *reinterpret_cast<bf16x8*>(Ws + sdst + 32 * i * kMidLdsRow) = wr[s][i];                             \
     _Pragma("unroll") for (int i = 0; i < XI; ++i)                                                        \
       *reinterpret_cast<bf16x8*>(Xs + sdst + 32 * i * kMidLdsRow) = xr[s][i];                             \
@@ -261,22 +269,23 @@ static int mid_slices(int N, int K) {
   return ks < 1 ? 1 : ks;
 }
 
-// Features a workgroup of the gated form owns (at most 64): the fewest workgroups that are a
-// multiple of the 256 compute units, or failing that (N < 256 or so) of 64 features each.
-static int mid_gated_features(int N) {
+// Features a workgroup of the gated form owns (at most `most`: 64, or 128 for the tile of 256
+// rows of w): the fewest workgroups that are a multiple of the 256 compute units, or failing that
+// (N < 256 or so) of 64 features each.
+static int mid_gated_features(int N, int most = 64) {
   for (int waves = 1; waves <= 64; ++waves) {
     const int wgs = 256 * waves;
     const int rr = (N + wgs - 1) / wgs;
-    if (rr <= 64) return rr < 16 ? 16 : rr;     // a narrow output: whole 16-feature tiles
+    if (rr <= most) return rr < 16 ? 16 : rr;     // a narrow output: whole 16-feature tiles
   }
   return 64;
 }
 
 template <typename Kern>
-static int mid_lds(Kern kern, bool* done) {
+static int mid_lds(Kern kern, bool* done, size_t bytes = kMidLdsBytes) {
   if (*done) return 0;
-  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMidLdsBytes);
-  XI_CHECK(e == hipSuccess, "linear_mid: cannot get %zu bytes of LDS: %s", kMidLdsBytes, hipGetErrorString(e));
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  XI_CHECK(e == hipSuccess, "linear_mid: cannot get %zu bytes of LDS: %s", bytes, hipGetErrorString(e));
   *done = true;
   return 0;
 }
@@ -295,8 +304,17 @@ int xi_linear_mid_slices(int N, int K) {
   return mid_slices(N, K);
 }
 
-// Features per workgroup of the gated form for an output of N features (w is [2N, K]).
-int xi_linear_mid_gated_features(int N) { return N < 1 ? 0 : mid_gated_features(N); }
+// Features per workgroup of the gated form for an output of N features (w is [2N, K]) at M rows.
+// From 17 to 64 rows a workgroup takes up to 128 features where that saves a round of workgroups.
+int xi_linear_mid_gated_features(int N, int M) {
+  if (N < 1) return 0;
+  const int r = mid_gated_features(N);
+  if (M > 16 && M <= 64) {
+    const int wide = mid_gated_features(N, 128);
+    if (wide > 64 && (N + wide - 1) / wide < (N + r - 1) / r) return wide;
+  }
+  return r;
+}
 
 // y: float32 [slices, M, N] with slices = xi_linear_mid_slices(N, K).  Up to 256 rows: blocks of
 // 128 rows are launched one after the other (the second pass over w comes in part from the
@@ -352,10 +370,26 @@ int xi_linear_mid_gated(const void* x, const void* w, void* y, int M, int N, int
   XI_CHECK(rotate >= 0, "linear_mid_gated: rotate=%d", rotate);
   XI_CHECK(ss == nullptr || (M <= 16 && parts >= 1 && parts <= 16 * kMidSsLoads),
            "linear_mid_gated: a folded norm takes up to 16 rows and %d parts (M=%d, parts=%d)", 16 * kMidSsLoads, M, parts);
-  const int R = features > 0 ? features : mid_gated_features(N);     // features: an override, for measurements
+  const int R = features > 0 ? features : xi_linear_mid_gated_features(N, M);     // features: an override, for measurements
   const long long wgs = (N + R - 1) / R;
-  XI_CHECK(R >= 1 && R <= 64 && wgs < (1ll << 31), "linear_mid_gated: %d features per workgroup", R);
+  XI_CHECK(R >= 1 && R <= 128 && wgs < (1ll << 31), "linear_mid_gated: %d features per workgroup", R);
+  XI_CHECK(R <= 64 || (M <= 64 && ss == nullptr), "linear_mid_gated: %d features per workgroup are taken up to 64 rows, without a folded norm", R);
   const MidFold fold{ss, parts, eps, 1.f / (float)K};
+  if (R > 64) {
+#define XI_MIDW(TJ)                                                                                                     \
+  do {                                                                                                                  \
+    static bool lds_set = false;                                                                                        \
+    if (mid_lds(linear_mid_kernel<kMidDepth, TJ, false, true, false, 8>, &lds_set, kMidWideLdsBytes)) return 1;         \
+    linear_mid_kernel<kMidDepth, TJ, false, true, false, 8><<<(unsigned)wgs, 256, kMidWideLdsBytes, stream>>>(          \
+        (const bf16*)x, (const bf16*)w, y, M, N, K, 1, 0, R, rotate, fold);                                             \
+  } while (0)
+    if (M <= 16) XI_MIDW(1);
+    else if (M <= 32) XI_MIDW(2);
+    else XI_MIDW(4);
+#undef XI_MIDW
+    XI_LAUNCH_CHECK("linear_mid_gated");
+    return 0;
+  }
 #define XI_MIDG(TJ, FULL, FOLD)                                                                               \
   do {                                                                                                        \
     static bool lds_set = false;                                                                              \

@@ -599,11 +599,14 @@ def gated_uses_mid(M: int, w: torch.Tensor) -> bool:
     return (MID_GATED_FROM <= M <= MID_GATED_UP_TO) or (0 < M < MID_GATED_FROM and w.numel() * 2 >= MID_GATED_BIG)
 
 
-def linear_mid_gated(x: torch.Tensor, w: torch.Tensor, ss: Optional[torch.Tensor] = None, eps: float = 0.0) -> torch.Tensor:
+def linear_mid_gated(x: torch.Tensor, w: torch.Tensor, ss: Optional[torch.Tensor] = None, eps: float = 0.0,
+                     features: Optional[int] = None) -> torch.Tensor:
     """silu(x @ gate^T) * (x @ up^T) in bfloat16 for w = [gate; up] [2N, K] and up to MID_GATED_ROWS
     rows with the tiled kernel: one pass over w whatever the number of rows.  `ss` [M, parts]
     float32 (up to FOLD_ROWS rows): x is the first half of a folded RMSNorm (`linear_fold_out`)
-    and the rows of the products are multiplied by rsqrt(sum(ss[row]) / K + eps) first."""
+    and the rows of the products are multiplied by rsqrt(sum(ss[row]) / K + eps) first.
+    `features`: the features a workgroup owns (up to 64, up to 128 for up to 64 rows), for
+    measurements and tests; chosen from the sizes if not given."""
     _dev(x, w, ss)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError("linear_mid_gated: operands must be bfloat16")
@@ -622,7 +625,7 @@ def linear_mid_gated(x: torch.Tensor, w: torch.Tensor, ss: Optional[torch.Tensor
         parts = int(ss.shape[1])
     y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
     _ok(lib().xi_linear_mid_gated(_p(x), _p(w), _p(y), M, N, K, _p(ss), parts, ctypes.c_float(eps), int(MID_GATED_ROTATE),
-                                  int(MID_GATED_FEATURES), _stream()))
+                                  int(features if features is not None else MID_GATED_FEATURES), _stream()))
     return y
 
 
