@@ -6,7 +6,7 @@
 
 Names follow the reference's Python package (xinfer.pyi).
 """
-from .config.engine_config import (EngineConfig, GenerationConfig, GenerationOutput, Message,
+from .config.engine_config import (DType, EngineConfig, GenerationConfig, GenerationOutput, Message,
                                    SamplingParams, StreamItem)
 
 
@@ -18,5 +18,5 @@ def __getattr__(name):
     raise AttributeError(name)
 
 
-__all__ = ["Engine", "EngineConfig", "GenerationConfig", "GenerationOutput", "LLMEngine", "Message",
+__all__ = ["DType", "Engine", "EngineConfig", "GenerationConfig", "GenerationOutput", "LLMEngine", "Message",
            "SamplingParams", "StreamItem"]

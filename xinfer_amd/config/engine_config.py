@@ -9,7 +9,16 @@ prefix cache, server, speculative decoding) are absent rather than accepted and 
 from __future__ import annotations
 
 from dataclasses import dataclass, field
+from enum import Enum
 from typing import List, Optional, Tuple, Union
+
+
+class DType(Enum):
+    """The reference's names (xinfer.pyi:8-11).  Half precision (F16) is not built: the engine
+    refuses it when it is made."""
+    F16 = "f16"
+    BF16 = "bf16"
+    F32 = "f32"
 
 
 @dataclass
@@ -46,6 +55,7 @@ class SamplingParams:
 class Message:
     role: str
     content: str
+    num_images: int = 0         # the reference's field (xinfer.pyi:151-155); text only here, so it must stay 0
 
 
 @dataclass

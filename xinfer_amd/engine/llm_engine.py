@@ -137,6 +137,10 @@ class LLMEngine:
         by_use = self.econfig.max_num_seqs * (-(-self.max_model_len // page))
         return max(1, min(by_memory, by_use))
 
+    def get_num_cached_tokens(self) -> int:
+        """Tokens held by the prefix cache (xinfer.pyi:215-222): there is none here, so none."""
+        return 0
+
     def get_available_kv_tokens(self) -> int:
         return min(self.runner.cache.free_pages(g) for g in range(len(self.runner.cache.groups))) \
             * self.econfig.page_size
@@ -335,6 +339,7 @@ class LLMEngine:
         if isinstance(messages, str):
             ids = self.tokenizer.encode(messages)
         elif messages and isinstance(messages[0], Message):
+            _text_only(messages)
             ids = self.tokenizer.encode(self.tokenizer.apply_chat_template(list(messages)))
         else:
             ids = [int(t) for t in messages]
@@ -357,8 +362,15 @@ class LLMEngine:
                       message_list: Sequence[Sequence[Message]]) -> List[GenerationOutput]:
         """The reference's blocking chat entry point (xinfer.pyi:199-205): every message list
         is rendered with the chat template and completed."""
+        for m in message_list:
+            _text_only(m)
         prompts = [self.tokenizer.apply_chat_template(list(m)) for m in message_list]
         return self.generate(prompts, list(params))
+
+
+def _text_only(messages) -> None:
+    if any(getattr(m, "num_images", 0) for m in messages):
+        raise ValueError("a message brings images: this engine takes text only")
 
 
 def _completes_a_stop(stops: List[List[int]], generated: Sequence[int], token: int) -> bool:

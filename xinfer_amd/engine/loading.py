@@ -16,6 +16,8 @@ _DTYPES = {"bf16": torch.bfloat16, "bfloat16": torch.bfloat16, "f32": torch.floa
 def parse_dtype(name) -> torch.dtype:
     """The reference takes --dtype f16|bf16|f32 (/root/reference/src/utils/mod.rs:2479-2486);
     float16 is not built here."""
+    if hasattr(name, "value") and isinstance(getattr(name, "value"), str):      # the DType enum
+        name = name.value
     if isinstance(name, torch.dtype):
         if name not in (torch.bfloat16, torch.float32):
             raise ValueError(f"dtype {name} is not supported (bfloat16 or float32)")
