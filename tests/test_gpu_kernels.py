@@ -929,15 +929,27 @@ def test_attention_decode_many_splits(nq, nkv, d, page, window, seqs, kpw):
 
 
 def test_decode_keys_per_workgroup_grow_with_the_work():
-    """About 512 workgroups a launch: chunks of 128 keys for one short sequence, of 512 at most."""
+    """Sequences of about one length: the splits that make the fewest rounds of workgroups over the
+    256 compute units, one round of large chunks where there is one, whole sequences from 256
+    (sequence, kv head) pairs on, and no fewer workgroups than units where the keys allow.  Mixed
+    lengths: chunks of 128 to 512 keys, about 512 workgroups."""
     from xinfer_amd import kernels
-    assert kernels.decode_keys_per_workgroup(8, 4096, similar=True) == 128
-    assert kernels.decode_keys_per_workgroup(32, 4096, similar=True) == 256
-    assert kernels.decode_keys_per_workgroup(64, 4096, similar=True) == 512
-    assert kernels.decode_keys_per_workgroup(8, 131072, similar=True) == 512
-    assert kernels.decode_keys_per_workgroup(1024, 1 << 20, similar=True) > 1 << 20      # one split
-    assert kernels.decode_keys_per_workgroup(1100, 1 << 20, similar=True) == 512
-    assert kernels.decode_keys_per_workgroup(512, 2304, similar=False) == 512
+    plan = lambda pairs, span: kernels.decode_keys_per_workgroup(pairs, span, similar=True)
+    assert plan(8, 4096) == 128                  # 32 splits: 256 workgroups
+    assert plan(64, 4096) == 1024                # 4 splits: 256 workgroups
+    assert plan(128, 8704) == 4352               # 2 splits
+    assert plan(96, 4096) == 512                 # 8 splits, three rounds: two splits would leave 64 units idle
+    assert plan(8, 8704) == 128                  # 544 small workgroups rather than 184 larger ones
+    assert plan(256, 4096) > 4096 and plan(512, 4096) > 4096 and plan(1024, 1 << 20) > 1 << 20      # one split
+    assert plan(384, 4096) == 2048               # three rounds of halves, not two of whole sequences
+    assert plan(8, 131072) == 4096
+    for pairs, span in ((8, 4096), (24, 4096), (40, 3000), (100, 900), (8, 131072)):
+        k = plan(pairs, span)
+        assert k % 128 == 0 and pairs * -(-span // k) >= 256, (pairs, span, k)
+    assert plan(4, 1024) == 128                  # too few keys for 256 workgroups: as many as there are
+    mixed = lambda pairs, span: kernels.decode_keys_per_workgroup(pairs, span, similar=False)
+    assert mixed(8, 4096) == 128 and mixed(32, 4096) == 256 and mixed(64, 4096) == 512
+    assert mixed(512, 2304) == 512 and mixed(8, 131072) == 512
 
 
 @pytest.mark.parametrize("window", [0, 100])
@@ -950,7 +962,6 @@ def test_attention_decode_one_split_per_sequence(window):
     seqs = [(290 + (7 * b) % 30, 1) for b in range(32)]
     assert kernels.decode_keys_per_workgroup(32 * nkv, 320, similar=True) > 320
     assert kernels.decode_keys_per_workgroup(32 * nkv, 320, similar=False) == 128
-    assert kernels.decode_keys_per_workgroup(48 * nkv, 320, similar=True) == 128     # 384 pairs leave units idle
     case = _paged_case(g, torch.bfloat16, nq, nkv, d, page, seqs)
     scale = 1.0 / math.sqrt(d)
     ref = _attention_ref(case, seqs, window, scale)

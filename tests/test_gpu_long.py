@@ -78,8 +78,8 @@ def _one_long_request():
 def test_long_request_portions_and_decoding_across_4096(dtype, long_model):
     """One request of 6,200 tokens: portions of 2,048 and 2,000 (the second attends to 2,048 cached
     keys), 60 single tokens from 4,048 to 4,108 (recorded the third time a bucket is seen and replayed
-    from then on: the bucket of 4,096 keys, then the one of 8,192), a portion of 2,048 behind 4,108
-    cached keys, and single tokens to the end; every position's logits against the plain model."""
+    from then on: the bucket of 4,096 keys, then the one of 5,120), a portion of 2,048 behind 4,108
+    cached keys, and single tokens to the end (the bucket of 7,168); every position's logits against the plain model."""
     from xinfer_amd.engine import ModelRunner, load_model
     d, pm = long_model
     reqs = _one_long_request()
@@ -97,7 +97,7 @@ def test_long_request_portions_and_decoding_across_4096(dtype, long_model):
     runner = ModelRunner(model, page_size=page, num_pages=-(-len(toks) // page), max_requests=2, graph_after=3)
     got = harness.replay(runner, steps)
     assert len(got) == len(toks)
-    assert {k[1] for k in runner._graphs} == {4096, 8192} and runner.graph_replays >= 60
+    assert {k[1] for k in runner._graphs} == {4096, 5120, 7168} and runner.graph_replays >= 60
     rel = harness.compare(got, _ref(pm, reqs), harness.TOL[dtype], f"LONG/{dtype}/one request")
     print(f"LONG/{dtype}/one request: worst error {rel:.2e} of the largest logit")
 
@@ -133,7 +133,7 @@ def test_decode_batch_of_eight_unequal_lengths(dtype, long_model):
     model = load_model(d, dtype, DEV)
     runner = ModelRunner(model, page_size=page, num_pages=sum(-(-n // page) for n in lens), max_requests=8, graph_after=3)
     got = harness.replay(runner, steps)
-    assert runner.graph_replays == tail - 2 and list(runner._graphs) == [(8, 8192, False)]
+    assert runner.graph_replays == tail - 2 and list(runner._graphs) == [(8, 6144, False)]
     rel = harness.compare(got, _ref(pm, reqs), harness.TOL[dtype], f"LONG/{dtype}/batch of eight")
     print(f"LONG/{dtype}/batch of eight: worst error {rel:.2e} of the largest logit")
 
@@ -223,15 +223,17 @@ def test_reference_attention_probe_cases(prefix, append, hq, hkv, page_map):
         tiles = torch.tensor([(0, q0) for q0 in range(0, append, qb)], dtype=torch.int32, device=DEV)
         out = kernels.attention_prefill_bf16(q_dev, kc, vt, bt, tiles, cu, cl, scale, 0, small=small)
         check(out, slice(None), f"prefill small={small}")
+    from xinfer_amd.engine.runner import context_bucket
     n_last = min(4, append)
     lens = torch.arange(kv_len - n_last + 1, kv_len + 1, dtype=torch.int32, device=DEV)
-    bucket = 1 << (kv_len - 1).bit_length()          # a recorded step's grid is laid out for its bucket's longest context
+    bucket = max(context_bucket(kv_len), 2 * kv_len)     # a recorded step's grid is laid out for more keys than there are: here twice
     wide = torch.zeros((n_last, -(-bucket // page)), dtype=torch.int32, device=DEV)
     wide[:, :n_pages] = bt
-    for kpw, span, tables in ((None, kv_len, bt.expand(n_last, -1).contiguous()), (128, kv_len, wide), (None, bucket, wide)):
+    for kpw, span, tables, similar in ((None, kv_len, bt.expand(n_last, -1).contiguous(), False), (128, kv_len, wide, False),
+                                       (None, bucket, wide, False), (None, context_bucket(kv_len), wide, True)):
         out = kernels.attention_decode_bf16(q_dev[-n_last:].contiguous(), kc, vt, tables, lens, span, scale, 0,
-                                            keys_per_workgroup=kpw)
-        check(out, slice(append - n_last, append), f"decode kpw={kpw} span={span}")
+                                            keys_per_workgroup=kpw, similar=similar)
+        check(out, slice(append - n_last, append), f"decode kpw={kpw} span={span} similar={similar}")
     out = kernels.attention_generic(q_dev[-n_last:].contiguous(), kc, vt, bt, torch.zeros(n_last, dtype=torch.int32, device=DEV),
                                     positions[-n_last:].to(DEV), scale, 0, v_transposed=True)
     check(out, slice(append - n_last, append), "generic")

@@ -117,6 +117,19 @@ class _DecodeGraph:
         return sum(t.numel() * t.element_size() for t in (self.dev32, self.dev64, self.logits))
 
 
+def context_bucket(longest: int) -> int:
+    """The longest context a recorded decode step is laid out for, given the step's longest: the
+    next multiple of 1,024 up to 16,384, of an eighth of the power of two below beyond that (eight
+    buckets an octave).  Kernels whose grid depends on the longest context are recorded for the
+    bucket's upper bound; with buckets an eighth apart or closer what they plan for is near what
+    they get (powers of two planned the attention's workgroups for up to twice the keys)."""
+    longest = max(1, int(longest))
+    if longest <= 16384:
+        return -(-longest // 1024) * 1024
+    step = 1 << (longest.bit_length() - 1 - 3)
+    return -(-longest // step) * step
+
+
 GRAPHS_MOST = 48                    # recorded decode graphs kept at a time, and
 GRAPH_BYTES_MOST = 1 << 30          # the bytes they may hold together; the least recently used goes first
 
@@ -375,9 +388,7 @@ class ModelRunner:
                              -3: f"request {rid}: its tokens exceed the model's {spec.max_positions} positions",
                              -4: f"a token id is outside the vocabulary of {spec.vocab_size}"}.get(
                                  ex.kind, f"the step could not be prepared ({ex.kind})")) from None
-        bucket = 1024
-        while bucket < longest:
-            bucket *= 2
+        bucket = context_bucket(longest)
         g = self._graphs.get((B, bucket, similar))
         if g is None:
             return None
@@ -458,9 +469,7 @@ class ModelRunner:
         beyond a request's own length ends at once)."""
         B = a.num_seqs
         longest = int(a.ctx_lens.max())
-        bucket = 1024
-        while bucket < longest:
-            bucket *= 2
+        bucket = context_bucket(longest)
         key = (B, bucket, _similar(a.ctx_lens))     # what kernels choose their shapes from
         all_rows = np.zeros(B, dtype=np.int32)
         all_rows[:rows32.size] = rows32

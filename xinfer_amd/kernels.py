@@ -9,6 +9,7 @@ cannot be built or loaded, importing fails loudly.
 from __future__ import annotations
 
 import ctypes
+import functools
 import math
 from typing import Optional
 
@@ -286,30 +287,51 @@ def gemm_tn(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] =
     return out
 
 
-DECODE_WORKGROUPS = 512             # workgroups of the split-K decode kernel a launch aims at: two a compute unit
+DECODE_WORKGROUPS = 512             # workgroups of the split-K decode kernel a launch of mixed lengths aims at: two a compute unit
 DECODE_KEYS_LEAST = 128             # keys of a workgroup: from one 32-key step a wave
-DECODE_KEYS_MOST = 512              # to four
+DECODE_KEYS_MOST = 512              # to four, in batches of mixed lengths
+DECODE_WORKGROUP_KEYS = 32          # what a workgroup costs beyond its keys (start, page numbers, merge, partial results), in keys
+DECODE_SPLITS_MOST = 1024           # splits of a sequence that the search below tries
 
 
 def decode_keys_per_workgroup(pairs: int, span: int, similar: bool = False) -> int:
+    return _decode_keys_per_workgroup(int(pairs), int(span), bool(similar))
+
+
+@functools.lru_cache(maxsize=4096)
+def _decode_keys_per_workgroup(pairs: int, span: int, similar: bool) -> int:
     """Keys per workgroup of the split-K decode kernel for `pairs` (sequence, kv head) pairs of
-    up to `span` keys: 128, 256 or 512, whichever makes about DECODE_WORKGROUPS workgroups.  A
-    workgroup costs the chip about 5 ns beyond its keys (launch, page numbers, merge, partial
-    results), so thousands of small ones lose to a few hundred larger ones (8 sequences of 4,096
-    keys on 8 kv heads: 33.9 us at 256 keys, 30.9 at 512; one sequence of 4,096: 11.2 us at 128,
-    13.0 at 256, 16.3 at 512).  Chunks of 1,024 or 2,048 keys gain another 4 to 8% on long
-    sequences of one length, but where they leave two or three workgroups a compute unit the time
-    depends on where the workgroups land (16 sequences of 8,400 keys in chunks of 2,048: 91 us
-    with a grid laid out for 10,240 keys, 115 for 16,384), and in batches of mixed lengths they
-    lose (64 sequences of 256 to 2,304 keys: 75 us at 512, 81 at 1,024): not used.  `similar`: the
-    sequences are about equally long; then, if the pairs alone fill the compute units evenly, a
-    workgroup takes a whole sequence: long loops, no partial results, no second kernel (8 to 11%
-    less time at 256 to 1024 pairs, but a quarter more where the pairs leave compute units idle
-    at the end)."""
-    if similar and pairs >= COMPUTE_UNITS:
-        rounds = pairs / COMPUTE_UNITS
-        if math.ceil(rounds) / rounds <= 1.1:
+    up to `span` keys (a multiple of 128; more than `span`: a workgroup takes a whole sequence and
+    there is no second kernel).
+
+    `similar` (the sequences are about equally long): the number of splits s that makes the least
+    of rounds(s) * (keys of a split + DECODE_WORKGROUP_KEYS), rounds(s) = ceil(pairs * s /
+    compute units): the compute units take the workgroups in turn, so the launch lasts as long
+    as the unit with the most of them, and a workgroup costs about 32 keys' time beyond its keys.
+    One round of large chunks wins where it exists (8 sequences of 4,096 keys on 8 kv heads: 4
+    splits, 31.7 us against 32.2 at 8 and 33.8 at 16; 16 sequences of 8,500 keys, 64 query heads:
+    2 splits, 104 us against 121 at 17; one sequence of 4,096: 32 splits of 128 keys, 11.2 us
+    against 13.0 at 16), whole sequences from 256 pairs on.
+
+    Otherwise (mixed lengths): 128, 256 or 512 keys, whichever makes about DECODE_WORKGROUPS
+    workgroups: larger chunks lose there (64 sequences of 256 to 2,304 keys: 75 us at 512, 81 at
+    1,024), since the short sequences' workgroups end early and the long ones' run on."""
+    if similar:
+        chunks = max(1, -(-int(span) // 128))
+        plans = []
+        for s in range(1, min(chunks, DECODE_SPLITS_MOST) + 1):
+            kpw = -(-chunks // s) * 128
+            splits = -(-chunks * 128 // kpw)
+            cost = -(-pairs * splits // COMPUTE_UNITS) * (kpw + DECODE_WORKGROUP_KEYS)
+            plans.append((cost, kpw, splits))
+        # a workgroup alone on its compute unit does not draw the unit's share of the memory
+        # bandwidth: with fewer workgroups than units more, smaller ones are ahead (one sequence of
+        # 8,704 keys: 16.8 us in 544 workgroups of 128 keys, 18.9 in 184 of 384)
+        filling = [p for p in plans if pairs * p[2] >= COMPUTE_UNITS]
+        best = min(filling or [max(plans, key=lambda p: p[2])], key=lambda p: (p[0], -p[1]))
+        if best[2] == 1:
             return (span + 128) // 128 * 128          # more than span: one split
+        return best[1]
     kpw = DECODE_KEYS_LEAST
     while kpw < DECODE_KEYS_MOST and pairs * span >= 2 * kpw * DECODE_WORKGROUPS:
         kpw *= 2
