@@ -931,7 +931,7 @@ def test_attention_decode_many_splits(nq, nkv, d, page, window, seqs, kpw):
 def test_decode_keys_per_workgroup_grow_with_the_work():
     """Sequences of about one length: the splits that make the fewest rounds of workgroups over the
     256 compute units, one round of large chunks where there is one, whole sequences from 256
-    (sequence, kv head) pairs on, and no fewer workgroups than units where the keys allow.  Mixed
+    (sequence, kv head) pairs on, and workgroups for seven eighths of the units at least where the keys allow.  Mixed
     lengths: chunks of 128 to 512 keys, about 512 workgroups."""
     from xinfer_amd import kernels
     plan = lambda pairs, span: kernels.decode_keys_per_workgroup(pairs, span, similar=True)
@@ -945,7 +945,7 @@ def test_decode_keys_per_workgroup_grow_with_the_work():
     assert plan(8, 131072) == 4096
     for pairs, span in ((8, 4096), (24, 4096), (40, 3000), (100, 900), (8, 131072)):
         k = plan(pairs, span)
-        assert k % 128 == 0 and pairs * -(-span // k) >= 256, (pairs, span, k)
+        assert k % 128 == 0 and pairs * -(-span // k) >= 224, (pairs, span, k)
     assert plan(4, 1024) == 128                  # too few keys for 256 workgroups: as many as there are
     mixed = lambda pairs, span: kernels.decode_keys_per_workgroup(pairs, span, similar=False)
     assert mixed(8, 4096) == 128 and mixed(32, 4096) == 256 and mixed(64, 4096) == 512

@@ -325,9 +325,10 @@ def _decode_keys_per_workgroup(pairs: int, span: int, similar: bool) -> int:
             cost = -(-pairs * splits // COMPUTE_UNITS) * (kpw + DECODE_WORKGROUP_KEYS)
             plans.append((cost, kpw, splits))
         # a workgroup alone on its compute unit does not draw the unit's share of the memory
-        # bandwidth: with fewer workgroups than units more, smaller ones are ahead (one sequence of
-        # 8,704 keys: 16.8 us in 544 workgroups of 128 keys, 18.9 in 184 of 384)
-        filling = [p for p in plans if pairs * p[2] >= COMPUTE_UNITS]
+        # bandwidth: with workgroups for fewer than seven eighths of the units more, smaller ones are
+        # ahead (one sequence of 8,704 keys: 16.8 us in 544 workgroups of 128 keys, 18.9 in 184 of
+        # 384; three of them: 27.4 us in 240 workgroups of 896 keys, 30.5 in 408 of 512)
+        filling = [p for p in plans if pairs * p[2] >= COMPUTE_UNITS * 7 // 8]
         best = min(filling or [max(plans, key=lambda p: p[2])], key=lambda p: (p[0], -p[1]))
         if best[2] == 1:
             return (span + 128) // 128 * 128          # more than span: one split
