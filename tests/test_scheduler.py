@@ -186,3 +186,71 @@ def test_two_long_requests_share_a_small_window_pool():
         spans = [x for x in seen[rid] if x != "preempted"]
         assert spans[-1][0] + spans[-1][1] == p + n - 1
     assert cm.free_pages(0) == 60 and cm.free_pages(1) == 7
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_running_one_step_ahead_keeps_the_books(seed):
+    """The engine's way of running ahead, with made-up tokens: after a step is committed every
+    sampled request is told to grow by one (or, if that token is the last its length allows, let go
+    of at once), the next step is planned and committed, and only then does the loop learn which
+    requests of the step before ended on their token's value; those are finished late, after one more
+    token of theirs has run for nothing.  Under random sizes, few pages (requests are preempted with
+    a token still on its way) and a window group: plans stay consistent, every request runs all its
+    tokens, and every page and slot comes back."""
+    rng = random.Random(100 + seed)
+    cm, s = make(num_pages=rng.choice([10, 16, 40]), page=rng.choice([4, 8, 16]), max_seqs=rng.choice([2, 3, 4]),
+                 budget=rng.choice([16, 33, 64]), chunk=rng.choice([5, 16, 48]), window_pages=rng.choice([None, 40]))
+    cap = cm.groups[0].num_pages * cm.groups[0].page_size
+    reqs, ends_at = {}, {}
+    for rid in range(14):
+        p = rng.randrange(1, cap // 2)
+        n = rng.randrange(1, max(2, min(30, cap - p)))
+        reqs[rid] = (p, n)
+        ends_at[rid] = rng.randrange(1, n + 1) if rng.random() < 0.6 else None     # its k-th token is an end-of-sequence
+        s.add(rid, p, n)
+    total = {rid: p for rid, (p, _) in reqs.items()}        # tokens the scheduler knows of
+    sampled_n = {rid: 0 for rid in reqs}                     # tokens sampled for it (launched)
+    live, closed, preempted_n, wasted = set(reqs), set(), 0, 0
+    launched = None                                          # requests sampled by the step that is "on the GPU"
+    steps = 0
+    while not s.idle() or launched:
+        plan, pre = s.schedule()
+        preempted_n += len(pre)
+        if launched and not plan:
+            pass                                             # nothing to launch: only the earlier step is read
+        else:
+            assert plan, "nothing planned although requests remain"
+            assert sum(e.count for e in plan) <= s.max_batched_tokens
+            assert len({e.request for e in plan}) == len(plan) <= s.max_num_seqs
+            for e in plan:
+                assert e.request in live and e.request not in closed
+                assert e.start == s.computed(e.request) and e.sample == (e.start + e.count == total[e.request])
+            s.commit()
+            cm.check()
+        now = []
+        for e in plan:
+            if e.sample:
+                rid = e.request
+                sampled_n[rid] += 1
+                now.append((rid, sampled_n[rid]))
+                if sampled_n[rid] >= reqs[rid][1]:           # its last token by length: the scheduler lets go now
+                    s.finish(rid)
+                    closed.add(rid)
+                else:
+                    total[rid] += 1
+                    s.append_token(rid)
+        for rid, k in launched or []:                        # the step before is read now
+            if rid not in live:
+                wasted += 1                                  # it ended a step ago: this token ran for nothing
+                continue
+            if ends_at[rid] == k or k >= reqs[rid][1]:
+                if rid not in closed:
+                    s.finish(rid)
+                live.discard(rid)
+        launched = now
+        steps += 1
+        assert steps < 20000
+    assert not live and cm.live_requests() == 0
+    for g, grp in enumerate(cm.groups):
+        assert cm.free_pages(g) == grp.num_pages
+    assert wasted <= sum(1 for rid in reqs if ends_at[rid] is not None)
