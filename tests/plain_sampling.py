@@ -5,7 +5,7 @@ order, each token whose preceding cumulative mass is below p (:82-111); top-k th
 applies the cutoff to the renormalised top-k set (:143-200); penalties subtract
 count * frequency + [count > 0] * presence (:358-378).  Ties are ordered by token id.  The
 draw walks the kept tokens in token order with a given uniform number."""
-from typing import List, Optional, Sequence
+from typing import Sequence
 
 import torch
 

@@ -9,7 +9,7 @@ from configs import TINY
 from xinfer_amd.config import ConfigError, Qwen3Config
 from xinfer_amd.engine.model import CausalLM
 from xinfer_amd.models import config_from_dict, family_of, load_config, registered_architectures
-from xinfer_amd.weights import (RandomStore, SafetensorsStore, TensorDecl, WeightError, write_random_model,
+from xinfer_amd.weights import (RandomStore, SafetensorsStore, WeightError, write_random_model,
                                 write_safetensors)
 
 

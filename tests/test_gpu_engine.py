@@ -665,7 +665,6 @@ def test_trace_run_program(dtype, model_dirs, tmp_path):
 def test_parts_alone(dtype, model_dirs):
     """Norm, feed-forward and attention mixer of tiny W's layer 0 each against its plain function."""
     from xinfer_amd.engine import ModelRunner, StepEntry, load_model
-    from xinfer_amd.parts import StepContext
     name = "W"
     model = load_model(model_dirs[name], dtype, DEV)
     pm = plain.PlainModel(model_dirs[name])

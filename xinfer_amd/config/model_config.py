@@ -9,8 +9,8 @@ from __future__ import annotations
 
 import json
 import os
-from dataclasses import dataclass, field, fields
-from typing import Any, Dict, List, Optional, Tuple
+from dataclasses import dataclass, fields
+from typing import Any, Dict, Optional, Tuple
 
 
 class ConfigError(ValueError):

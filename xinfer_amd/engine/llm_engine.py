@@ -12,7 +12,7 @@ from __future__ import annotations
 import os
 import time
 from dataclasses import dataclass, field
-from typing import Dict, Iterable, List, Optional, Sequence, Union
+from typing import Dict, List, Optional, Sequence, Union
 
 import torch
 
@@ -24,7 +24,7 @@ from ..config.model_config import ConfigError
 from ..models import family_of
 from .loading import load_model, parse_dtype
 from .runner import ModelRunner, StepEntry
-from .scheduler import RequestTooLarge, Scheduler
+from .scheduler import Scheduler
 from .tokenizer import IncrementalText, load_tokenizer
 
 DEFAULT_MAX_TOKENS = 16384      # /root/reference/src/core/engine.rs:650-678

@@ -10,11 +10,11 @@ from __future__ import annotations
 
 import sys
 from dataclasses import dataclass
-from typing import Dict, List, Optional, Tuple
+from typing import Dict, List, Tuple
 
 import torch
 
-from ..config.spec import ModelSpec, ScheduleEntry
+from ..config.spec import ModelSpec
 from ..parts import (KVNeed, LayerCache, StateNeed, StepContext, Stream, block_class, embedding_class,
                      head_class, norm_class)
 from ..weights.store import TensorDecl, WeightStore

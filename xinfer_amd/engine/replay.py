@@ -22,7 +22,6 @@ import os
 import sys
 from typing import Dict
 
-import numpy as np
 
 
 def main(argv=None) -> int:

@@ -17,13 +17,13 @@ sequence; this one mixes them and leaves sampling to the caller.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Any, Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
 
-from ..cache import DecodeStepError, BatchArrays, CacheGroup, OutOfPages, PagedCacheManager
+from ..cache import DecodeStepError, BatchArrays, CacheGroup, PagedCacheManager
 from ..parts import PAGE, LayerCache, StepContext
 from .model import CausalLM
 

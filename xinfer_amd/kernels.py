@@ -10,7 +10,6 @@ from __future__ import annotations
 
 import ctypes
 import functools
-import math
 from typing import Optional
 
 import torch

@@ -13,7 +13,6 @@ more than 128 were sampled, never the prompt, and a penalty of exactly 1.0 count
 """
 from __future__ import annotations
 
-import ctypes
 from dataclasses import dataclass
 from typing import List, Optional, Sequence
 
