@@ -834,6 +834,40 @@ def test_attention_prefill_mfma(nq, nkv, d, page, window, seqs):
     assert err < _tol(torch.bfloat16, 2), err
 
 
+@pytest.mark.parametrize("d", list(range(16, 257, 16)))
+def test_attention_mfma_every_head_size(d):
+    """Head sizes in steps of 16 up to 256 through the matrix-core kernels: a portion behind a cached
+    prefix and a whole prompt (every workgroup shape), and single tokens (two chunk lengths), with a
+    window in one run; three query heads on each of two kv heads."""
+    from xinfer_amd import kernels
+    nq, nkv, page = 6, 2, 16
+    assert kernels.mfma_attention_supported(nq, nkv, d, page)
+    scale = 1.0 / math.sqrt(d)
+    g = torch.Generator().manual_seed(1000 + d)
+    for window in (0, 50):
+        seqs = [(230, 90), (70, 70), (1, 1)]
+        case = _paged_case(g, torch.bfloat16, nq, nkv, d, page, seqs)
+        ref = _attention_ref(case, seqs, window, scale)
+        q, kc, vt, bt = _mfma_inputs(case)
+        cu, ctx = _cu_ctx(seqs)
+        for small in ((0, 1, 2) if kernels.prefill_ring_supported(d) else (0, 1)):
+            qb = kernels.prefill_block(d, nq // nkv, small)
+            tiles = torch.tensor([(b, q0) for b, (_, n) in enumerate(seqs) for q0 in range(0, n, qb)], dtype=torch.int32)
+            out = kernels.attention_prefill_bf16(q, kc, vt, bt, tiles.to(DEV), cu.to(DEV), ctx.to(DEV), scale, window, small=small)
+            err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
+            assert err < _tol(torch.bfloat16, 2), ("prefill", window, small, err)
+        seqs = [(300, 1), (129, 1), (50, 1), (1, 1)]
+        case = _paged_case(g, torch.bfloat16, nq, nkv, d, page, seqs)
+        ref = _attention_ref(case, seqs, window, scale)
+        q, kc, vt, bt = _mfma_inputs(case)
+        _, ctx = _cu_ctx(seqs)
+        if kernels.decode_attention_takes(nq, nkv, d):
+            for kpw in (None, 128):
+                out = kernels.attention_decode_bf16(q, kc, vt, bt, ctx.to(DEV), 300, scale, window, keys_per_workgroup=kpw)
+                err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
+                assert err < _tol(torch.bfloat16, 2), ("decode", window, kpw, err)
+
+
 @pytest.mark.parametrize("nq,nkv,d,page,window", [(8, 2, 64, 16, 0), (5, 5, 48, 16, 24), (32, 8, 128, 64, 0), (10, 2, 128, 64, 0)])
 def test_attention_of_a_mixed_batch_splits_between_the_kernels(nq, nkv, d, page, window):
     """A step's attention as the engine asks for it: single tokens of decoding requests at the head of
