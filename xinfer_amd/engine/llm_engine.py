@@ -178,7 +178,9 @@ class LLMEngine:
 
     # ---- the loop ------------------------------------------------------------------------
     def step(self) -> List[int]:
-        """One iteration: plan, run the batch, sample, finish.  Returns the ids that finished."""
+        """One iteration: plan a step, launch it with its sampling, then read the tokens of the step
+        launched before it and apply the finishing rules to them (with `run_ahead` off: this step's
+        own).  Returns the ids that were found finished."""
         done: List[int] = []
         plan, preempted = self.scheduler.schedule()
         for rid in preempted:
