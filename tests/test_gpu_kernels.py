@@ -962,6 +962,111 @@ def test_attention_decode_many_splits(nq, nkv, d, page, window, seqs, kpw):
     assert (out.cpu().double() - ref).abs().max() / ref.abs().max() < _tol(torch.bfloat16, 2)
 
 
+PACKED_CASES = [
+    # nq, nkv, d, page, window, rot, interleaved, norm, bias, slices, kpw, contexts
+    (32, 8, 128, 64, 0, 128, False, True, False, 0, None, [4096, 1, 257, 256, 1025, 65]),
+    (32, 8, 128, 64, 0, 128, False, True, False, 3, 256, [513, 257, 256, 1024, 1]),     # the last position opens a chunk
+    (6, 2, 16, 8, 0, 16, False, True, True, 0, 128, [200, 130, 513, 129]),
+    (5, 5, 48, 16, 24, 32, False, True, False, 0, None, [100, 24, 25, 7]),              # a window, partial rotation
+    (8, 2, 128, 64, 300, 128, True, False, True, 2, 128, [2000, 299, 301, 600]),
+    (16, 1, 64, 8, 0, 64, True, True, False, 0, 128, [700, 9]),                         # a group of 16 for four waves
+    (2, 2, 256, 16, 0, 256, False, True, True, 5, None, [70, 300]),
+    (3, 1, 80, 8, 0, 0, False, False, False, 0, 128, [40, 13, 130]),                    # no rotation, no norm
+    (8, 2, 128, 64, 0, 64, False, True, False, 0, 128, [300, 129, 64]),                 # half of the head rotated
+    (4, 4, 64, 16, 0, 64, False, True, True, 2, 128, [200, 65, 128]),
+]
+
+
+@pytest.mark.parametrize("nq,nkv,d,page,window,rot,interleaved,norm,bias,slices,kpw,contexts", PACKED_CASES)
+def test_attention_decode_packed_gives_the_bits_of_the_two_kernels(nq, nkv, d, page, window, rot, interleaved, norm,
+                                                                   bias, slices, kpw, contexts):
+    """A decode step's attention from the packed projection (norm, rotation and cache write inside
+    the attention kernel) against the two kernels one after the other: the same output and the same
+    cache, bit for bit; a sequence with a negative slot stores nothing; and a new key made to win the
+    softmax brings back the new value, so the workgroup that wrote it has read it."""
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(31)
+    seqs = [(c, 1) for c in contexts]
+    B, heads = len(seqs), nq + 2 * nkv
+    case = _paged_case(g, torch.bfloat16, nq, nkv, d, page, seqs)
+    _, kc, vt, bt = _mfma_inputs(case)
+    _, ctx = _cu_ctx(seqs)
+    positions = (ctx - 1).to(torch.int32)
+    slots = torch.tensor([int(case["bt"][b, (c - 1) // page]) * page + (c - 1) % page for b, c in enumerate(contexts)],
+                         dtype=torch.int64)
+    slots[B - 1] = -1                     # the last sequence's token is another run's to store
+    packed = _rand((B, heads * d), torch.bfloat16, g)
+    if slices:
+        cut = torch.randn((slices, B, heads * d), generator=g) * 0.3
+        cut[0] += packed.float() - cut.sum(0)
+        packed = cut
+    cos, sin = plain.rope_tables(10000.0, rot, max(contexts) + 1) if rot else (torch.zeros(1, 0), torch.zeros(1, 0))
+    qw = (1 + 0.3 * torch.randn(d, generator=g)).to(DEV) if norm else None
+    kw = (1 + 0.3 * torch.randn(d, generator=g)).to(DEV) if norm else None
+    bs = (0.2 * torch.randn(heads * d, generator=g)).to(DEV) if bias else None
+    scale, eps, longest = 1.0 / math.sqrt(d), 1e-5, max(contexts)
+    cos, sin, positions, slots, ctx_d = cos.to(DEV), sin.to(DEV), positions.to(DEV), slots.to(DEV), ctx.to(DEV)
+
+    def both(packed):
+        k1, v1 = kc.clone(), vt.clone()
+        q = kernels.qk_norm_rope_kv(packed.to(DEV), qw, kw, eps, cos, sin, rot, interleaved, positions, slots, k1, v1,
+                                    nq, nkv, d, v_transposed=True, vector_min_tokens=1 << 30, bias=bs)
+        one = kernels.attention_decode_bf16(q, k1, v1, bt, ctx_d, longest, scale, window, keys_per_workgroup=kpw)
+        k2, v2 = kc.clone(), vt.clone()
+        two = kernels.attention_decode_packed_bf16(packed.to(DEV), qw, kw, eps, cos, sin, rot, interleaved, positions,
+                                                   slots, k2, v2, bt, ctx_d, longest, nq, scale, window, bias=bs,
+                                                   keys_per_workgroup=kpw)
+        assert torch.equal(k1, k2) and torch.equal(v1, v2)
+        assert not torch.equal(k1[:, :, :, :], kc) and not torch.equal(v1, vt)       # something was stored
+        assert torch.equal(one, two)
+        return two, k2, v2
+
+    out, k2, v2 = both(packed)
+    # the sequence with the negative slot: its place in the cache is as it was
+    c = contexts[B - 1]
+    pg, off = int(case["bt"][B - 1, (c - 1) // page]), (c - 1) % page
+    assert torch.equal(k2[pg, :, off], kc[pg, :, off]) and torch.equal(v2[pg, :, :, off], vt[pg, :, :, off])
+    if not norm and not rot and not slices:
+        # the new key of sequence 0 points along its first query head of every group, far longer than any other
+        x = packed.clone().reshape(B, heads, d)
+        gsz = nq // nkv
+        for kvh in range(nkv):
+            qv = x[0, kvh * gsz].float()
+            x[0, nq + kvh] = (qv / qv.norm() * 60 / scale / qv.norm()).to(torch.bfloat16)
+        out, _, _ = both(x.reshape(B, heads * d))
+        new_v = x[0, nq + nkv:].float()
+        for kvh in range(nkv):
+            assert (out[0].reshape(nq, d)[kvh * gsz].float().cpu() - new_v[kvh]).abs().max() < 0.05, kvh
+
+
+def test_attention_decode_packed_refuses():
+    from xinfer_amd import kernels
+    nq, nkv, d, page = 4, 2, 32, 16
+    kc = torch.zeros((4, nkv, page, d), dtype=torch.bfloat16, device=DEV)
+    vt = torch.zeros((4, nkv, d, page), dtype=torch.bfloat16, device=DEV)
+    bt = torch.zeros((2, 2), dtype=torch.int32, device=DEV)
+    ctx = torch.tensor([3, 5], dtype=torch.int32, device=DEV)
+    pos = (ctx - 1).to(torch.int32)
+    slots = torch.tensor([2, 4], dtype=torch.int64, device=DEV)
+    cos = torch.ones((8, d // 2), device=DEV)
+    good = torch.zeros((2, (nq + 2 * nkv) * d), dtype=torch.bfloat16, device=DEV)
+
+    def call(qkv=good, cos=cos, slots=slots, rot=d, qw=None, kw=None):
+        return kernels.attention_decode_packed_bf16(qkv, qw, kw, 1e-6, cos, cos, rot, False, pos, slots, kc, vt, bt, ctx,
+                                                    5, nq, 1.0)
+    call()
+    with pytest.raises(kernels.KernelError, match="is not contiguous"):
+        call(qkv=good[:, :-d])
+    with pytest.raises(kernels.KernelError, match="bfloat16"):
+        call(qkv=good.float())
+    with pytest.raises(kernels.KernelError, match="cos/sin"):
+        call(rot=d - 2)
+    with pytest.raises(kernels.KernelError, match="one block table row"):
+        call(slots=slots[:1])
+    with pytest.raises(kernels.KernelError, match="both"):
+        call(qw=torch.ones(d, device=DEV))
+
+
 def test_decode_keys_per_workgroup_grow_with_the_work():
     """Sequences of about one length: the splits that make the fewest rounds of workgroups over the
     256 compute units, one round of large chunks where there is one, whole sequences from 256

@@ -73,6 +73,37 @@ def test_tail_one_by_one(name, dtype, model_dirs):
     _run(name, dtype, model_dirs, harness.trace_tail_one_by_one(_requests(name)), "tail")
 
 
+@pytest.mark.parametrize("name", list(TINY))
+def test_decode_steps_with_the_attention_kernel_doing_the_steps_own_work(name, model_dirs):
+    """Steps of single tokens in bfloat16 let the attention kernel norm and rotate its heads and
+    store the new keys and values; with that switched off (the kernel of its own before the
+    attention, as in steps that bring portions) the logits are the same bit for bit."""
+    from xinfer_amd.engine import load_model
+    from xinfer_amd import kernels
+    together = dict([(k, v) for k, v in _requests(name).items() if len(v) > 8][:4])
+    steps = harness.trace_tail_one_by_one(_requests(name)) + harness.trace_batch_decode(together, tail=6)
+    _run(name, "bfloat16", model_dirs, steps, "tail")                 # warms the cached model too
+    model = _runner_cache[(name, "bfloat16")]
+    mixers = [b.mixer for b in model.blocks]
+    assert all(m.decode_packed for m in mixers)
+    calls = []
+    inner = kernels.attention_decode_packed_bf16
+    kernels.attention_decode_packed_bf16 = lambda *a, **k: (calls.append(1), inner(*a, **k))[1]
+    try:
+        got = _run(name, "bfloat16", model_dirs, steps, "tail, packed")
+        assert calls
+        for m in mixers:
+            m.decode_packed = False
+        n = len(calls)
+        again = _run(name, "bfloat16", model_dirs, steps, "tail, two kernels")
+        assert len(calls) == n
+    finally:
+        kernels.attention_decode_packed_bf16 = inner
+        for m in mixers:
+            m.decode_packed = True
+    assert got.keys() == again.keys() and all(torch.equal(got[k], again[k]) for k in got)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", list(TINY))
 def test_portions(name, dtype, model_dirs):

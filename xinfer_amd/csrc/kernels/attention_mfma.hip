@@ -27,6 +27,7 @@
 // /root/reference/src/utils/kvcache_allocator.rs:662-673); golden formula
 // /root/reference/tests/probes/compare_flashinfer_probe.py:51-73.
 #include "common.h"
+#include "qk_row.h"
 
 namespace xi {
 
@@ -36,6 +37,11 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ __forceinline__ bf16x8 load8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
+// A barrier for what went through LDS only: reads of global memory that are under way stay
+// under way (__syncthreads waits for them all, which leaves the memory pipeline empty once).
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+__device__ __forceinline__ void wait_global() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 __device__ __forceinline__ bf16x8 zero8() {
   bf16x8 z;
 #pragma unroll
@@ -53,13 +59,38 @@ __device__ __forceinline__ bf16x8 zero8() {
 // (sums scaled by 2^-m, with m and l) go to a workspace, combined by the second kernel in
 // split order; with one split for every sequence the kernel writes the result itself.
 // =====================================================================================
-template <int KC, int DT>
+//
+// PACKED: the step's own part of the work is done here too, which saves the kernel that otherwise
+// runs before this one.  `q` is then the packed projection [sequences, (nq + 2 nkv) d] (1: bfloat16
+// rows; 2: float32 partial sums of a product cut along K): every workgroup norms and rotates its own
+// query heads into LDS, and the workgroup whose chunk holds the sequence's last position first does
+// the same for the new key, copies the new value, and writes both into the cache, from where it
+// reads them back with the rest of its chunk (a workgroup sees its own writes after a barrier; no
+// other workgroup of the launch reads that position).  The caches are therefore not `__restrict__`
+// nor read-only in this form.
+struct PackedStep {
+  int slices;                  // PACKED == 2: partial sums, `slice_stride` elements apart
+  size_t slice_stride;
+  const float* bias;           // of the packed row (float32), or null
+  const float* qw;             // per-head norm weights [d], or null (both)
+  const float* kw;
+  float eps;
+  const float* cos_t;          // [positions, rot / 2]
+  const float* sin_t;
+  int rot, interleaved;
+  const int* positions;        // [sequences]
+  const long long* slots;      // [sequences]; negative: the sequence's key and value are not stored
+};
+
+template <int KC, int DT, int PACKED>
 __global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
-    const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ vt_cache,
+    const void* q_v, bf16* k_cache_w, bf16* vt_cache_w,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ ctx_lens,
     float* __restrict__ part_o, float* __restrict__ part_ml, bf16* __restrict__ out, int max_splits, float scale_log2,
-    int window, int page, int nq, int nkv, int d, int keys_per_wg) {
+    int window, int page, int nq, int nkv, int d, int keys_per_wg, PackedStep ps) {
   extern __shared__ float lds[];  // [4 waves][g][d] + [4][g][2] + page numbers of the chunk
+  const bf16* k_cache = k_cache_w;
+  const bf16* vt_cache = vt_cache_w;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, j = lane >> 4;
   // the kv head runs fastest: workgroups go to the chip's eight dies in turn, and with eight kv
@@ -75,6 +106,9 @@ __global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
   const int kvh = blockIdx.x, seq = blockIdx.y, split = blockIdx.z;
   const int g = nq / nkv;
   const int ctx = ctx_lens[seq];
+  // asked for together with the length, not after the test below that needs it
+  const int tok_pos = PACKED ? ps.positions[seq] : 0;
+  const long long slot = PACKED ? ps.slots[seq] : -1;
   const int pos = ctx - 1;
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int k_begin = (lo & ~31) + split * keys_per_wg;
@@ -89,19 +123,6 @@ __global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
   const int n_pages = ((k_end - 1) >> page_shift) - first_page + 1;
   const int* bt = block_tables + (size_t)seq * max_pages;
   for (int i = threadIdx.x; i < n_pages; i += 256) pages[i] = bt[first_page + i];
-
-  // this lane's query column: head kvh*g + r of the sequence, or none
-  const bool col = r < g;
-  bf16x8 qb[KC];
-  {
-    const bf16* qrow = q + ((size_t)seq * nq + kvh * g + (col ? r : 0)) * d;
-#pragma unroll
-    for (int c = 0; c < KC; ++c) {
-      const int off = 32 * c + 8 * j;
-      qb[c] = (col && off < d) ? load8(qrow + off) : zero8();
-    }
-  }
-  __syncthreads();
 
   // the four waves take alternate steps: the two halves of a 128-byte line of V^T (64 keys) are
   // then asked for at about the same time
@@ -138,14 +159,105 @@ __global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
     for (int dt = 0; dt < DT; ++dt) va[dt] = (16 * dt < d) ? load8(vp + (size_t)16 * dt * page) : zero8();
   };
 
+  // this lane's query column: head kvh*g + r of the sequence, or none
+  const bool col = r < g;
+  bf16x8 qb[KC];
+  if constexpr (PACKED == 0) {
+    const bf16* qrow = reinterpret_cast<const bf16*>(q_v) + ((size_t)seq * nq + kvh * g + (col ? r : 0)) * d;
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+      const int off = 32 * c + 8 * j;
+      qb[c] = (col && off < d) ? load8(qrow + off) : zero8();
+    }
+    __syncthreads();
+    if (kb0 < kb1) {
+      load_k(kb0);
+      load_v(kb0);
+    }
+  } else {
+    // The waves share out the heads: in the workgroup that holds the last position the new key
+    // and value first, then the group's query heads, which go to LDS (in the space of the merge).
+    // Everything the first two heads of a wave need is asked for before the barrier that the page
+    // numbers need anyway, so that the kernel has one more dependent read than without this work
+    // only where a wave has more than two heads (groups of more than six query heads).  The
+    // barriers wait for LDS alone: reads of the cache that are under way stay under way.
+    // (Measured at 8 sequences of 4,096 keys, 32 query and 8 kv heads of 128: 30.9 us against 27.8
+    // for the kernel that is given q, and the kernel of 4.9 us before it is gone.  Every lane
+    // making its own part of the heads in registers, without LDS, took 32.2: each wave then reads
+    // the norm's weights and the tables' rows again for all 64 lanes.)
+    constexpr bool PARTS = PACKED == 2;
+    bf16* qs = reinterpret_cast<bf16*>(lds_o);   // [g][d]
+    const int heads = nq + 2 * nkv;
+    const bool owner = pos < k_begin + keys_per_wg && slot >= 0;
+    const int first_q = owner ? 2 : 0;           // rows: [new key, new value,] query heads
+    const int n_rows = g + first_q;
+    auto head_of = [&](int row) { return row >= first_q ? kvh * g + row - first_q : row == 0 ? nq + kvh : nq + nkv + kvh; };
+    auto packed_head = [&](int h) {
+      return PackedHead<bf16, PARTS>{q_v, ((size_t)seq * heads + h) * d, ps.slices, ps.slice_stride,
+                                     ps.bias ? ps.bias + (size_t)h * d : nullptr};
+    };
+    const long long spage = slot >> page_shift;
+    const int soff = (int)(slot & (page - 1));
+    bf16* k_new = k_cache_w + (((size_t)spage * nkv + kvh) * page + soff) * d;
+    bf16* v_new = vt_cache_w + ((size_t)spage * nkv + kvh) * d * page + soff;
+    HeadRegs<bf16, PARTS> hr[2];
+    float vr[4];
+#pragma unroll
+    for (int rd = 0; rd < 2; ++rd) {
+      const int row = wave + 4 * rd;
+      if (row >= n_rows) continue;
+      const auto x = packed_head(head_of(row));
+      if (row >= first_q || row == 0) {
+        hr[rd].load(x, row >= first_q ? ps.qw : ps.kw, ps.cos_t, ps.sin_t, ps.rot, ps.interleaved, tok_pos, d, lane);
+      } else {
+#pragma unroll
+        for (int p = 0; p < 4; ++p) vr[p] = lane + kWave * p < d ? x.at(lane + kWave * p) : 0.f;
+      }
+    }
+    lds_barrier();     // the page numbers are in LDS
+    // The first keys and values are asked for before the heads are worked on, except in a chunk so
+    // short that a wave's first step holds the new key: that waits until the key is written.
+    const bool late = owner && k_end - k_begin <= 128;
+    if (!late && kb0 < kb1) {
+      load_k(kb0);
+      load_v(kb0);
+    }
+#pragma unroll
+    for (int rd = 0; rd < 2; ++rd) {
+      const int row = wave + 4 * rd;
+      if (row >= n_rows) continue;
+      if (row >= first_q) {
+        hr[rd].finish(ps.qw != nullptr, ps.eps, ps.rot, ps.interleaved, d, lane, qs + (size_t)(row - first_q) * d);
+      } else if (row == 0) {
+        hr[rd].finish(ps.kw != nullptr, ps.eps, ps.rot, ps.interleaved, d, lane, k_new);
+      } else {
+#pragma unroll
+        for (int p = 0; p < 4; ++p)
+          if (lane + kWave * p < d) v_new[(size_t)(lane + kWave * p) * page] = __float2bfloat16(vr[p]);
+      }
+    }
+    for (int row = wave + 8; row < n_rows; row += 4)
+      norm_rope_head<bf16, PARTS>(packed_head(head_of(row)), ps.qw, ps.eps, ps.cos_t, ps.sin_t, ps.rot, ps.interleaved,
+                                  tok_pos, d, lane, qs + (size_t)(row - first_q) * d);
+    if (owner && wave < 2) wait_global();   // the new key and value are written (what the other waves read comes after the barrier)
+    lds_barrier();     // the heads are in LDS
+    const bf16* qrow = qs + (size_t)(col ? r : 0) * d;
+#pragma unroll
+    for (int c = 0; c < KC; ++c) {
+      const int off = 32 * c + 8 * j;
+      qb[c] = (col && off < d) ? load8(qrow + off) : zero8();
+    }
+    lds_barrier();     // before the merge's space is written
+    if (late && kb0 < kb1) {
+      load_k(kb0);
+      load_v(kb0);
+    }
+  }
+
   f32x4 acc[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;   // running max (log2 domain) and this lane's part of the sum
-  if (kb0 < kb1) {
-    load_k(kb0);
-    load_v(kb0);
-  }
   for (int kb = kb0; kb < kb1; kb += 128) {
     const bool more = kb + 128 < kb1;
     f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
@@ -388,10 +500,11 @@ int xi_attention_mfma_supported(int nq, int nkv, int d, int page) {
   return (d % 16 == 0 && d >= 16 && d <= 256 && page >= 8 && (page & (page - 1)) == 0 && nq % nkv == 0) ? 1 : 0;
 }
 
-int xi_attention_decode_bf16(const void* q, const void* k_cache, const void* vt_cache, const int* block_tables,
-                             int max_pages, const int* ctx_lens, void* out, float* part_o, float* part_ml,
-                             int max_splits, int keys_per_wg, float scale, int window, int page, int n_seq,
-                             int nq, int nkv, int d, hipStream_t stream) {
+// The decode launch: `packed` 0 takes q [sequences, nq, d]; 1 and 2 the packed projection, see PackedStep.
+static int launch_decode(int packed, const void* q, const PackedStep& ps, void* k_cache, void* vt_cache,
+                         const int* block_tables, int max_pages, const int* ctx_lens, void* out, float* part_o,
+                         float* part_ml, int max_splits, int keys_per_wg, float scale, int window, int page, int n_seq,
+                         int nq, int nkv, int d, hipStream_t stream) {
   XI_CHECK(xi_attention_mfma_supported(nq, nkv, d, page), "attention_decode: unsupported sizes nq=%d nkv=%d d=%d page=%d",
            nq, nkv, d, page);
   const int g = nq / nkv;
@@ -404,13 +517,20 @@ int xi_attention_decode_bf16(const void* q, const void* k_cache, const void* vt_
   if (n_seq == 0) return 0;
   dim3 grid(nkv, n_seq, max_splits);
   const float sl = scale * kLog2e;
-#define XI_DC(KC, DT)                                                                              \
-  attn_decode_split_kernel<KC, DT><<<grid, 256, lds, stream>>>(                                    \
-      (const bf16*)q, (const bf16*)k_cache, (const bf16*)vt_cache, block_tables, max_pages, ctx_lens, \
-      part_o, part_ml, (bf16*)out, max_splits, sl, window, page, nq, nkv, d, keys_per_wg)
-  if (d <= 64) XI_DC(2, 4);
-  else if (d <= 128) XI_DC(4, 8);
-  else XI_DC(8, 16);
+#define XI_DC(KC, DT, PACKED)                                                                      \
+  attn_decode_split_kernel<KC, DT, PACKED><<<grid, 256, lds, stream>>>(                            \
+      q, (bf16*)k_cache, (bf16*)vt_cache, block_tables, max_pages, ctx_lens,                       \
+      part_o, part_ml, (bf16*)out, max_splits, sl, window, page, nq, nkv, d, keys_per_wg, ps)
+#define XI_DCP(KC, DT)             \
+  do {                             \
+    if (packed == 0) XI_DC(KC, DT, 0); \
+    else if (packed == 1) XI_DC(KC, DT, 1); \
+    else XI_DC(KC, DT, 2);         \
+  } while (0)
+  if (d <= 64) XI_DCP(2, 4);
+  else if (d <= 128) XI_DCP(4, 8);
+  else XI_DCP(8, 16);
+#undef XI_DCP
 #undef XI_DC
   XI_LAUNCH_CHECK("attention_decode_split");
   if (max_splits == 1) return 0;   // the split kernel has written the result
@@ -425,6 +545,46 @@ int xi_attention_decode_bf16(const void* q, const void* k_cache, const void* vt_
   }
   XI_LAUNCH_CHECK("attention_decode_combine");
   return 0;
+}
+
+int xi_attention_decode_bf16(const void* q, const void* k_cache, const void* vt_cache, const int* block_tables,
+                             int max_pages, const int* ctx_lens, void* out, float* part_o, float* part_ml,
+                             int max_splits, int keys_per_wg, float scale, int window, int page, int n_seq,
+                             int nq, int nkv, int d, hipStream_t stream) {
+  return launch_decode(0, q, PackedStep{}, const_cast<void*>(k_cache), const_cast<void*>(vt_cache), block_tables,
+                       max_pages, ctx_lens, out, part_o, part_ml, max_splits, keys_per_wg, scale, window, page, n_seq,
+                       nq, nkv, d, stream);
+}
+
+// A decode step's attention from the packed projection: per-head norm and rotation of q and k,
+// the new keys and values into the cache at `slots`, and the attention over the cache, in one
+// launch (plus the combine).  `qkv` is [n_seq, (nq + 2 nkv) d] bfloat16 (`slices` 0) or `slices`
+// float32 partial sums of that shape, added in slice order.  The other operands are those of
+// xi_qk_norm_rope_kv and xi_attention_decode_bf16, and the results have the same bits as theirs.
+int xi_attention_decode_packed_bf16(const void* qkv, int slices, const float* bias, const float* qw, const float* kw,
+                                    float eps, const float* cos_t, const float* sin_t, int rot, int interleaved,
+                                    const int* positions, const long long* slots, void* k_cache, void* vt_cache,
+                                    const int* block_tables, int max_pages, const int* ctx_lens, void* out,
+                                    float* part_o, float* part_ml, int max_splits, int keys_per_wg, float scale,
+                                    int window, int page, int n_seq, int nq, int nkv, int d, hipStream_t stream) {
+  XI_CHECK(rot >= 0 && rot <= d && rot % 2 == 0, "attention_decode_packed: rotary_dim %d must be even and <= head_dim %d", rot, d);
+  XI_CHECK((qw == nullptr) == (kw == nullptr), "attention_decode_packed: q and k norm weights must both be given or both absent");
+  XI_CHECK(slices >= 0 && slices <= 64, "attention_decode_packed: %d slices", slices);
+  PackedStep ps;
+  ps.slices = slices;
+  ps.slice_stride = (size_t)n_seq * (nq + 2 * nkv) * d;
+  ps.bias = bias;
+  ps.qw = qw;
+  ps.kw = kw;
+  ps.eps = eps;
+  ps.cos_t = cos_t;
+  ps.sin_t = sin_t;
+  ps.rot = rot;
+  ps.interleaved = interleaved;
+  ps.positions = positions;
+  ps.slots = slots;
+  return launch_decode(slices ? 2 : 1, qkv, ps, k_cache, vt_cache, block_tables, max_pages, ctx_lens, out, part_o,
+                       part_ml, max_splits, keys_per_wg, scale, window, page, n_seq, nq, nkv, d, stream);
 }
 
 }  // extern "C"

@@ -3,6 +3,7 @@
 // All reductions are float32 in an order fixed by the row alone, so a row's
 // result does not depend on what else is in the batch.
 #include "common.h"
+#include "qk_row.h"
 
 #include <algorithm>
 #include <stdarg.h>
@@ -274,110 +275,26 @@ __global__ void qk_norm_rope_kv_kernel(const void* __restrict__ qkv_v, int slice
   if (wid >= (long long)n_tok * heads) return;
   const int t = (int)(wid / heads);
   const int h = (int)(wid - (long long)t * heads);
-  const size_t row0 = (size_t)t * heads * d + (size_t)h * d;
-  const float* bs = bias ? bias + (size_t)h * d : nullptr;
-  // element i of this head's row, without the bias
-  auto ld = [&](int i) -> float {
-    if constexpr (PARTS) {
-      const float* p = reinterpret_cast<const float*>(qkv_v) + row0 + i;
-      float a = 0.f;
-#pragma unroll 4
-      for (int sl = 0; sl < slices; ++sl) a += p[(size_t)sl * slice_stride];
-      return a;
-    } else {
-      return to_float(reinterpret_cast<const T*>(qkv_v)[row0 + i]);
-    }
-  };
-
-  T* dst;
-  const float* w = nullptr;
-  bool rotate = true;
+  const PackedHead<T, PARTS> x{qkv_v, (size_t)t * heads * d + (size_t)h * d, slices, slice_stride,
+                               bias ? bias + (size_t)h * d : nullptr};
   if (h < nq) {
-    dst = q_out + ((size_t)t * nq + h) * d;
-    w = qw;
-  } else {
-    const long long slot = slots[t];
-    if (slot < 0) return;
-    const long long page = slot / page_size;
-    const int off = (int)(slot - page * page_size);
-    const bool is_k = h < nq + nkv;
-    const int kvh = is_k ? h - nq : h - nq - nkv;
-    if (!is_k && v_transposed) {  // V kept as [page, kv_head, d, offset]
-      T* vt = v_cache + ((size_t)page * nkv + kvh) * d * page_size + off;
-      for (int i = lane; i < d; i += kWave)
-        vt[(size_t)i * page_size] = from_float<T>(bs ? ld(i) + bs[i] : ld(i));
-      return;
-    }
-    T* cache = is_k ? k_cache : v_cache;
-    dst = cache + (((size_t)page * nkv + kvh) * page_size + off) * d;
-    w = is_k ? kw : nullptr;
-    rotate = is_k;
-  }
-  if (!rotate) {  // v: plain copy
-    for (int i = lane; i < d; i += kWave) dst[i] = from_float<T>(bs ? ld(i) + bs[i] : ld(i));
+    norm_rope_head<T, PARTS>(x, qw, eps, cos_t, sin_t, rot, interleaved, positions[t], d, lane,
+                             q_out + ((size_t)t * nq + h) * d);
     return;
   }
-  // The kernel lives on latency: everything that can be asked for at once is.  A lane holds
-  // pairs lane and lane + 64 of the rotated part and up to 4 elements of the rest (head_dim <=
-  // 256); the position's row of the tables is asked for as soon as the position is there,
-  // while the sum of squares is still being taken.
-  const int half = rot / 2;
-  const int pos = positions[t];
-  float xa[2], xb[2], wa[2], wb[2], xt[4], wt[4];
-#pragma unroll
-  for (int p = 0; p < 2; ++p) {
-    const int i = lane + kWave * p;
-    const bool ok = i < half;
-    const int ia = interleaved ? 2 * i : i;
-    const int ib = interleaved ? 2 * i + 1 : i + half;
-    xa[p] = ok ? ld(ia) + (bs ? bs[ia] : 0.f) : 0.f;
-    xb[p] = ok ? ld(ib) + (bs ? bs[ib] : 0.f) : 0.f;
-    wa[p] = (ok && w) ? w[ia] : 1.f;
-    wb[p] = (ok && w) ? w[ib] : 1.f;
-  }
-#pragma unroll
-  for (int p = 0; p < 4; ++p) {
-    const int i = rot + lane + kWave * p;
-    const bool ok = i < d;
-    xt[p] = ok ? ld(i) + (bs ? bs[i] : 0.f) : 0.f;
-    wt[p] = (ok && w) ? w[i] : 1.f;
-  }
-  const float* c = cos_t + (size_t)pos * half;
-  const float* sn_row = sin_t + (size_t)pos * half;
-  float cs[2], sn[2];
-#pragma unroll
-  for (int p = 0; p < 2; ++p) {
-    const int i = lane + kWave * p;
-    cs[p] = i < half ? c[i] : 1.f;
-    sn[p] = i < half ? sn_row[i] : 0.f;
-  }
-  float inv = 1.f;
-  if (w) {
-    float ss = 0.f;
-#pragma unroll
-    for (int p = 0; p < 2; ++p) ss += xa[p] * xa[p] + xb[p] * xb[p];
-#pragma unroll
-    for (int p = 0; p < 4; ++p) ss += xt[p] * xt[p];
-    ss = wave_sum(ss);
-    inv = rsqrtf(ss / (float)d + eps);
-  }
-#pragma unroll
-  for (int p = 0; p < 2; ++p) {
-    const int i = lane + kWave * p;
-    if (i < half) {
-      // the reference rounds the normed value to the activation type before rotating
-      // (two kernels); here it stays in float32 until the single final rounding.
-      const float a = xa[p] * inv * wa[p];
-      const float b = xb[p] * inv * wb[p];
-      dst[interleaved ? 2 * i : i] = from_float<T>(a * cs[p] - b * sn[p]);
-      dst[interleaved ? 2 * i + 1 : i + half] = from_float<T>(a * sn[p] + b * cs[p]);
-    }
-  }
-#pragma unroll
-  for (int p = 0; p < 4; ++p) {  // dims beyond the rotary part
-    const int i = rot + lane + kWave * p;
-    if (i < d) dst[i] = from_float<T>(xt[p] * inv * wt[p]);
-  }
+  const long long slot = slots[t];
+  if (slot < 0) return;
+  const long long page = slot / page_size;
+  const int off = (int)(slot - page * page_size);
+  const bool is_k = h < nq + nkv;
+  const int kvh = is_k ? h - nq : h - nq - nkv;
+  if (is_k)
+    norm_rope_head<T, PARTS>(x, kw, eps, cos_t, sin_t, rot, interleaved, positions[t], d, lane,
+                             k_cache + (((size_t)page * nkv + kvh) * page_size + off) * d);
+  else if (v_transposed)   // V kept as [page, kv_head, d, offset]
+    copy_head<T, PARTS>(x, d, lane, v_cache + ((size_t)page * nkv + kvh) * d * page_size + off, (size_t)page_size);
+  else
+    copy_head<T, PARTS>(x, d, lane, v_cache + (((size_t)page * nkv + kvh) * page_size + off) * d, 1);
 }
 
 // The same for bfloat16 with the transposed V pool, 16 bytes per lane and one pass: a

@@ -465,6 +465,63 @@ def attention_decode_bf16(q, k_cache, vt_cache, block_tables, ctx_lens, max_ctx_
     return out
 
 
+def attention_decode_packed_bf16(qkv, q_weight, k_weight, eps, cos, sin, rotary_dim, interleaved, positions, slots,
+                                 k_cache, vt_cache, block_tables, ctx_lens, max_ctx_len, num_heads, scale, window=0,
+                                 bias=None, out=None, keys_per_workgroup=None, similar=False):
+    """What `qk_norm_rope_kv` and `attention_decode_bf16` do one after the other for a batch in which
+    every sequence has one token, in one launch less: `qkv` is the packed projection
+    [B, (nq + 2 nkv) d] in bfloat16, or a stack [slices, B, width] of float32 partial sums; the new
+    keys and values go into the cache at `slots` on the way (the same bits as the other kernel's)."""
+    _dev(qkv, q_weight, k_weight, cos, sin, positions, slots, k_cache, vt_cache, block_tables, ctx_lens, out, bias)
+    nq, nkv, page, d = int(num_heads), k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
+    slices = 0
+    if qkv.dim() == 3:
+        _want(qkv, torch.float32, "attention_decode_packed: partial sums")
+        slices = int(qkv.shape[0])
+        if not (0 < slices <= 64):
+            raise KernelError(f"attention_decode_packed: {slices} slices of partial sums, at most 64")
+    else:
+        _want(qkv, torch.bfloat16, "attention_decode_packed: qkv")
+    if qkv.dim() not in (2, 3) or qkv.shape[-1] != (nq + 2 * nkv) * d:
+        raise KernelError(f"attention_decode_packed: qkv {tuple(qkv.shape)} is not [B, {(nq + 2 * nkv) * d}]")
+    B = int(qkv.shape[-2])
+    _check_cache(k_cache, vt_cache, nkv, d, torch.bfloat16, True, "attention_decode_packed")
+    _want(block_tables, torch.int32, "attention_decode_packed: block_tables")
+    _want(ctx_lens, torch.int32, "attention_decode_packed: ctx_lens")
+    _want(positions, torch.int32, "attention_decode_packed: positions")
+    _want(slots, torch.int64, "attention_decode_packed: slots")
+    _want(cos, torch.float32, "attention_decode_packed: cos")
+    _want(sin, torch.float32, "attention_decode_packed: sin")
+    if block_tables.shape[0] != B or ctx_lens.shape != (B,) or positions.shape != (B,) or slots.shape != (B,):
+        raise KernelError("attention_decode_packed: one block table row, context length, position and slot per sequence")
+    if cos.dim() != 2 or cos.shape[1] != rotary_dim // 2 or sin.shape != cos.shape:
+        raise KernelError(f"attention_decode_packed: cos/sin {tuple(cos.shape)} are not [positions, {rotary_dim // 2}]")
+    for w in (q_weight, k_weight):
+        if w is not None:
+            _want(w, torch.float32, "attention_decode_packed: norm weight")
+            if w.shape != (d,):
+                raise KernelError("attention_decode_packed: norm weight must be [head_dim]")
+    if bias is not None:
+        _want(bias, torch.float32, "attention_decode_packed: bias")
+        if bias.shape != (qkv.shape[-1],):
+            raise KernelError(f"attention_decode_packed: bias {tuple(bias.shape)} is not [{qkv.shape[-1]}]")
+    span = min(int(max_ctx_len), int(window) + 31) if window > 0 else int(max_ctx_len)
+    kpw = int(keys_per_workgroup or decode_keys_per_workgroup(B * nkv, span, similar))
+    max_splits = span // kpw + 1
+    part_o = torch.empty((B, nq, max_splits, d), dtype=torch.float32, device=qkv.device)
+    part_ml = torch.empty((B, nq, max_splits, 2), dtype=torch.float32, device=qkv.device)
+    if out is None:
+        out = torch.empty((B, nq * d), dtype=torch.bfloat16, device=qkv.device)
+    elif out.shape != (B, nq * d) or out.dtype != torch.bfloat16 or not out.is_contiguous():
+        raise KernelError("attention_decode_packed: out has the wrong shape or dtype")
+    _ok(lib().xi_attention_decode_packed_bf16(
+        _p(qkv), slices, _p(bias), _p(q_weight), _p(k_weight), ctypes.c_float(eps), _p(cos), _p(sin), int(rotary_dim),
+        int(bool(interleaved)), _p(positions), _p(slots), _p(k_cache), _p(vt_cache), _p(block_tables),
+        int(block_tables.shape[1]), _p(ctx_lens), _p(out), _p(part_o), _p(part_ml), max_splits, kpw,
+        ctypes.c_float(scale), int(window), int(page), B, nq, nkv, d, _stream()))
+    return out
+
+
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx, group: int,
               scale: float, window: int = 0, v_transposed: bool = False) -> torch.Tensor:
     """Attention of one step's tokens over the paged cache of `group`; chooses the kernel

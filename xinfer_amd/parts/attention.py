@@ -24,6 +24,7 @@ from .linear import Linear
 @register_mixer("attention")
 class PagedAttention(Mixer):
     VECTOR_MIN_DECODE = 512      # decoded tokens lie in a page each: the form with one wave per head stays ahead up to here
+    DECODE_PACKED = True         # steps of single tokens: norm, rotation and cache write inside the attention kernel
 
     def __init__(self, spec: PartSpec, dtype: torch.dtype):
         super().__init__(spec, dtype)
@@ -42,6 +43,8 @@ class PagedAttention(Mixer):
         # generic kernel serves it; sizes that only the prefill kernel takes (more than 16 query heads
         # per kv head) need the step's lengths on the host to lay out its tiles.
         self.graph_safe = dtype != torch.bfloat16 or kernels.decode_attention_takes(self.nq, self.nkv, self.d)
+        self.decode_packed = (self.DECODE_PACKED and dtype == torch.bfloat16
+                              and kernels.decode_attention_takes(self.nq, self.nkv, self.d))
         pos = spec.get("position")
         self.position = position_encoding_class(pos.kind)(pos, dtype) if pos is not None else None
         self.qkv: Optional[Linear] = None
@@ -102,6 +105,20 @@ class PagedAttention(Mixer):
         pos = self.position
         slots = ctx.slots[cache.group] if cache.write else ctx.no_slots
         vt = self.dtype == torch.bfloat16
+        if (vt and ctx.max_q_len == 1 and self.decode_packed
+                and kernels.mfma_attention_supported(self.nq, self.nkv, self.d, cache.k.shape[2])):
+            # a step of single tokens: the attention kernel norms and rotates its own heads and
+            # stores the new keys and values, one launch less in every layer
+            a = kernels.attention_decode_packed_bf16(
+                qkv, self.q_norm_w, self.k_norm_w, self.qk_norm_eps,
+                pos.cos if pos is not None else ctx.empty_f32,
+                pos.sin if pos is not None else ctx.empty_f32,
+                pos.rotary_dim if pos is not None else 0,
+                pos.interleaved if pos is not None else False,
+                ctx.positions, slots, cache.k, cache.v, ctx.block_tables[cache.group], ctx.ctx_lens, ctx.max_ctx_len,
+                self.nq, self.scale, self.window, bias=self.qkv_bias,
+                similar=getattr(ctx, "similar_lengths", False))
+            return self.o(a, out_dtype=self.dtype, allow_split=True, sink=sink)
         q = kernels.qk_norm_rope_kv(
             qkv, self.q_norm_w, self.k_norm_w, self.qk_norm_eps,
             pos.cos if pos is not None else ctx.empty_f32,
