@@ -446,6 +446,48 @@ def test_linear_mid_gated_wide_tile(M, N, K, features):
             kernels.linear_mid_gated(_rand((65, K), torch.bfloat16, g).to(DEV), w.to(DEV), features=features)
 
 
+@pytest.mark.parametrize("M,N,K,slices", [(129, 4096, 4096, 4), (256, 4096, 12288, 8), (200, 1024, 3072, 2), (512, 4096, 12288, 8),
+                                          (1000, 5120, 17408, 2), (256, 7168, 5120, 4), (300, 4096, 4096, 1), (128, 4096, 12288, 1),
+                                          (256, 4096, 1024, 1), (1025, 4096, 12288, 1), (200, 1000, 2056, 1)])
+def test_library_split_slices_and_their_sum(M, N, K, slices):
+    """Narrow products of 129 to 1,024 rows go to the library as one batched product over slices of
+    K: the chosen number of slices, the dispatch (`linear_bf16` with `allow_split`), and the sum of
+    the partial sums against a float64 product."""
+    from xinfer_amd import kernels
+    assert kernels.library_split_slices(M, N, K) == slices
+    g = torch.Generator().manual_seed(41)
+    x = _rand((M, K), torch.bfloat16, g)
+    w = _rand((N, K), torch.bfloat16, g, scale=0.05)
+    ref = x.double() @ w.double().T
+    y = kernels.linear_bf16(x.to(DEV), w.to(DEV), torch.bfloat16, allow_split=True)
+    if slices > 1:
+        assert y.shape == (slices, M, N) and y.dtype == torch.float32
+        # each slice is the product over its own part of K
+        k0 = K // slices
+        part = x[:, k0:2 * k0].double() @ w[:, k0:2 * k0].double().T
+        assert (y[1].cpu().double() - part).abs().max() / part.abs().max() < 1e-5
+        total = y.cpu().double().sum(0)
+        assert (total - ref).abs().max() / ref.abs().max() < 1e-5
+        # the norm adds them in order: the same as adding them here
+        resid = torch.zeros((M, N), device=DEV)
+        ones = torch.ones(N, device=DEV)
+        kernels.add_rmsnorm(resid, y, ones, 1e-6, torch.float32)
+        acc = torch.zeros((M, N), device=DEV)
+        for sl in range(slices):
+            acc += y[sl]
+        assert torch.equal(resid, acc)
+    elif y.dim() == 2:
+        assert y.shape == (M, N) and y.dtype == torch.bfloat16
+        assert (y.cpu().double() - ref).abs().max() / ref.abs().max() < _tol(torch.bfloat16)
+    else:       # the tiled kernel's own slices
+        assert (y.cpu().double().sum(0) - ref).abs().max() / ref.abs().max() < 1e-5
+    with pytest.raises(kernels.KernelError, match="slices"):
+        kernels.linear_library_split(x.to(DEV), w.to(DEV), 3 if K % 24 else 7)
+    if M > kernels.LIBRARY_SPLIT_MOST_ROWS:
+        with pytest.raises(kernels.KernelError, match="rows, at most"):
+            kernels.linear_library_split(x.to(DEV), w.to(DEV), 2)
+
+
 def test_linear_skinny_plan_fills_the_compute_units():
     """The shapes the streaming product chooses: grids that are multiples of the 256 compute
     units where the width allows (a workgroup may own a number of features that is no multiple

@@ -165,12 +165,12 @@ def test_real_layer_sizes(name, real_model_dirs):
 
 
 @pytest.mark.parametrize("name,live", [("8B", 12), ("8B", 40), ("14B", 8), ("14B", 48), ("32B", 16), ("32B", 70), ("0.6B", 9), ("0.6B", 33),
-                                       ("4B", 16), ("4B", 64)])
+                                       ("4B", 16), ("4B", 64), ("8B", 150), ("14B", 200), ("0.6B", 256), ("32B", 129)])
 def test_real_layer_sizes_wide_decode_batches(name, live, real_model_dirs):
     """Decode steps of many requests at real layer sizes, in bfloat16: the kernels that serve 6 to
     16 rows (thin products with the folded norm, the gated tiled product), 17 to 64 (tiled
-    products with partial sums) and more (the library beside them), inside the model against
-    the plain implementation; the steps are launched one by one and, the third time on, replayed
+    products with partial sums), more (the library beside them) and 129 to 256 (the library's
+    batched product over slices of K), inside the model against the plain implementation; the steps are launched one by one and, the third time on, replayed
     from a graph."""
     from xinfer_amd.engine import ModelRunner, load_model
     t = REAL[name]

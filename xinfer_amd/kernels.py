@@ -663,6 +663,55 @@ def linear_mid(x: torch.Tensor, w: torch.Tensor, depth: int = 0) -> torch.Tensor
     return y
 
 
+LIBRARY_SPLIT_ROWS = 1024     # most rows of a product that is cut along K into one batched library product
+LIBRARY_SPLIT_K = 1024        # least K of a slice up to 512 rows; twice that beyond
+LIBRARY_SPLIT_MOST_ROWS = 1024    # what `linear_library_split` takes at all
+
+
+def library_split_slices(M: int, N: int, K: int) -> int:
+    """Slices of K into which x [M, K] @ w [N, K]^T is cut for the library, 1 = not at all.  A
+    narrow output gives the library too few tiles for the chip's 256 compute units (256 rows by
+    4096 columns: 16 tiles of 256 x 256), and its own choice of kernel does not split K: slices
+    as one batched product, with float32 partial sums [slices, M, N] for the caller to add in
+    order, put more of the chip to work.  As many slices (a power of two) as keep the tiles x
+    slices within the compute units and a slice's K long enough to pay for its start.  Beyond
+    256 rows only for K >= 2 N (the down projection): the reader of the partial sums then reads
+    `slices` float32 values for every one it would read in bfloat16, which a smaller gain does
+    not pay for.  Measured on MI355X at Qwen3-8B sizes (qkv / o / down, us): 256 rows 36 / 19 / 49
+    in one library product and 36 / 27 / 55 in the tiled kernel against 22 / 18 / 35 so; down at
+    512 and 1,024 rows 80 -> 54 and 119 -> 87; at Qwen3-14B sizes and 256 rows 48 / 44 / 227
+    (tiled: 46 / 37 / 97) -> 29 / 23 / 54.  Up to 128 rows the tiled kernel is level or ahead."""
+    if not (MID_BLOCK < M <= min(LIBRARY_SPLIT_ROWS, LIBRARY_SPLIT_MOST_ROWS)) or (M > MID_ROWS and K < 2 * N):
+        return 1
+    tiles = -(-M // 256) * -(-N // 256)
+    most = min(COMPUTE_UNITS // tiles, K // (LIBRARY_SPLIT_K if M <= 512 else 2 * LIBRARY_SPLIT_K))
+    slices = 1
+    while slices * 2 <= most and K % (slices * 2 * 64) == 0:
+        slices *= 2
+    return slices
+
+
+def linear_library_split(x: torch.Tensor, w: torch.Tensor, slices: int) -> torch.Tensor:
+    """bfloat16 x [M, K] @ w [N, K]^T as float32 partial sums [slices, M, N] over `slices` equal
+    parts of K, one batched library product over views of x and w (nothing is copied)."""
+    _dev(x, w)
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError("linear_library_split: operands must be bfloat16")
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
+        raise KernelError(f"linear_library_split: x {tuple(x.shape)} and w {tuple(w.shape)} do not match")
+    M, K = x.shape
+    N = w.shape[0]
+    if slices < 1 or K % (slices * 8):
+        raise KernelError(f"linear_library_split: K={K} is not {slices} slices of a multiple of 8")
+    if not (0 < M <= LIBRARY_SPLIT_MOST_ROWS):
+        # (a batched bfloat16 product of 2 x [2048, 6144] by [6144, 4096] ended in a GPU memory fault inside
+        # the library on this image; the float32 form is used for the sizes it has been run at)
+        raise KernelError(f"linear_library_split: {M} rows, at most {LIBRARY_SPLIT_MOST_ROWS}")
+    xs = x.view(M, slices, K // slices).transpose(0, 1)            # [slices, M, K / slices]
+    ws = w.view(N, slices, K // slices).permute(1, 2, 0)            # [slices, K / slices, N]
+    return torch.bmm(xs, ws, out_dtype=torch.float32)
+
+
 MID_GATED_ROWS = 128      # most rows of the gated form of the tiled product
 MID_GATED_FEATURES = 0    # features a workgroup of it owns; 0: chosen from N (the fewest workgroups that are a multiple of 256)
 MID_GATED_UP_TO = 64      # it is used up to this many rows (more: its reads of x from L2 outweigh the library's
@@ -859,6 +908,10 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtyp
     if out_dtype == torch.float32 and MID_WIDE_FROM <= x.shape[0] <= MID_GATED_ROWS \
             and linear_mid_slices(w.shape[0], w.shape[1]) == 1:
         return linear_mid(x, w)[0]           # a wide output in float32 (the head): one slice is the result
+    if allow_split and MID_BLOCK < x.shape[0] <= LIBRARY_SPLIT_ROWS:
+        slices = library_split_slices(x.shape[0], w.shape[0], w.shape[1])
+        if slices > 1:
+            return linear_library_split(x, w, slices)
     if allow_split and MID_FROM <= x.shape[0] <= MID_ROWS and linear_mid_slices(w.shape[0], w.shape[1]) > 0 \
             and w.shape[0] <= MID_WIDEST and (x.shape[0] <= MID_BLOCK or w.numel() * 2 >= MID_TWO_BLOCKS):
         return linear_mid(x, w)

@@ -4,8 +4,10 @@ The reference routes every dense projection through candle's matmul, i.e. the ve
 BLAS (/root/reference/src/models/layers/linear.rs:76-124).  Here:
   float32  : the hand-written fixed-order kernel (`kernels.gemm_tn`) - true 32-bit, and
              an output element does not depend on the batch it was computed in;
-  bfloat16 : the hand-written skinny kernel for few rows (decode), the vendor library
-             (hipBLASLt through torch) for many rows, as the reference uses a library.
+  bfloat16 : the hand-written kernels for few rows (decode), the vendor library
+             (hipBLASLt through torch) for many rows, as the reference uses a library;
+             narrow outputs at 129 to 1,024 rows as one batched library product over slices
+             of K where the caller takes partial sums (`kernels.library_split_slices`).
 A weight that the checkpoint stores in 32 bits stays in 32 bits; activations are then
 widened for this product.
 """
