@@ -1016,6 +1016,10 @@ PACKED_CASES = [
     (3, 1, 80, 8, 0, 0, False, False, False, 0, 128, [40, 13, 130]),                    # no rotation, no norm
     (8, 2, 128, 64, 0, 64, False, True, False, 0, 128, [300, 129, 64]),                 # half of the head rotated
     (4, 4, 64, 16, 0, 64, False, True, True, 2, 128, [200, 65, 128]),
+    # a window makes chunks start at any multiple of 32: every offset of the last position in its chunk and in
+    # its 128-byte line of V^T, among them lines of which the chunk's first reads have already taken a part
+    (8, 2, 128, 64, 300, 128, False, True, False, 0, 256, list(range(600, 664))),
+    (4, 1, 64, 64, 140, 64, False, True, False, 0, 256, list(range(450, 514))),     # one chunk of 140 to 171 keys
 ]
 
 
