@@ -37,8 +37,9 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 constexpr float kLog2e = 1.4426950408889634f;
 
 __device__ __forceinline__ bf16x8 load8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
-// A barrier for what went through LDS only: reads of global memory that are under way stay
-// under way (__syncthreads waits for them all, which leaves the memory pipeline empty once).
+// A barrier for what went through LDS, written out: this wave's LDS operations are waited for,
+// reads of global memory that are under way are not.  `wait_global` is the other half, for a
+// wave whose writes to global memory others are about to read.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 __device__ __forceinline__ void wait_global() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
@@ -179,8 +180,8 @@ __global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
     // and value first, then the group's query heads, which go to LDS (in the space of the merge).
     // Everything the first two heads of a wave need is asked for before the barrier that the page
     // numbers need anyway, so that the kernel has one more dependent read than without this work
-    // only where a wave has more than two heads (groups of more than six query heads).  The
-    // barriers wait for LDS alone: reads of the cache that are under way stay under way.
+    // only where a wave has more than two heads (groups of more than six query heads), and the
+    // first keys and values are asked for before the heads are worked on.
     // (Measured at 8 sequences of 4,096 keys, 32 query and 8 kv heads of 128: 30.9 us against 27.8
     // for the kernel that is given q, and the kernel of 4.9 us before it is gone.  Every lane
     // making its own part of the heads in registers, without LDS, took 32.2: each wave then reads
