@@ -178,10 +178,8 @@ __global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
   } else {
     // The waves share out the heads: in the workgroup that holds the last position the new key
     // and value first, then the group's query heads, which go to LDS (in the space of the merge).
-    // Everything the first two heads of a wave need is asked for before the barrier that the page
-    // numbers need anyway, so that the kernel has one more dependent read than without this work
-    // only where a wave has more than two heads (groups of more than six query heads), and the
-    // first keys and values are asked for before the heads are worked on.
+    // The first keys and values are asked for before the heads are worked on, so that what the
+    // heads need travels beside them.
     // (Measured at 8 sequences of 4,096 keys, 32 query and 8 kv heads of 128: 30.9 us against 27.8
     // for the kernel that is given q, and the kernel of 4.9 us before it is gone.  Every lane
     // making its own part of the heads in registers, without LDS, took 32.2: each wave then reads
@@ -201,20 +199,6 @@ __global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
     const int soff = (int)(slot & (page - 1));
     bf16* k_new = k_cache_w + (((size_t)spage * nkv + kvh) * page + soff) * d;
     bf16* v_new = vt_cache_w + ((size_t)spage * nkv + kvh) * d * page + soff;
-    HeadRegs<bf16, PARTS> hr[2];
-    float vr[4];
-#pragma unroll
-    for (int rd = 0; rd < 2; ++rd) {
-      const int row = wave + 4 * rd;
-      if (row >= n_rows) continue;
-      const auto x = packed_head(head_of(row));
-      if (row >= first_q || row == 0) {
-        hr[rd].load(x, row >= first_q ? ps.qw : ps.kw, ps.cos_t, ps.sin_t, ps.rot, ps.interleaved, tok_pos, d, lane);
-      } else {
-#pragma unroll
-        for (int p = 0; p < 4; ++p) vr[p] = lane + kWave * p < d ? x.at(lane + kWave * p) : 0.f;
-      }
-    }
     lds_barrier();     // the page numbers are in LDS
     // The first keys and values are asked for before the heads are worked on, except in a chunk so
     // short that a wave's first step holds the new key: that waits until the key is written.
@@ -223,23 +207,14 @@ __global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
       load_k(kb0);
       load_v(kb0);
     }
-#pragma unroll
-    for (int rd = 0; rd < 2; ++rd) {
-      const int row = wave + 4 * rd;
-      if (row >= n_rows) continue;
-      if (row >= first_q) {
-        hr[rd].finish(ps.qw != nullptr, ps.eps, ps.rot, ps.interleaved, d, lane, qs + (size_t)(row - first_q) * d);
-      } else if (row == 0) {
-        hr[rd].finish(ps.kw != nullptr, ps.eps, ps.rot, ps.interleaved, d, lane, k_new);
-      } else {
-#pragma unroll
-        for (int p = 0; p < 4; ++p)
-          if (lane + kWave * p < d) v_new[(size_t)(lane + kWave * p) * page] = __float2bfloat16(vr[p]);
-      }
+    for (int row = wave; row < n_rows; row += 4) {
+      const auto x = packed_head(head_of(row));
+      if (row == 1 && owner)
+        copy_head<bf16, PARTS>(x, d, lane, v_new, (size_t)page);
+      else      // a query head into LDS, or the new key into the cache
+        norm_rope_head<bf16, PARTS>(x, row >= first_q ? ps.qw : ps.kw, ps.eps, ps.cos_t, ps.sin_t, ps.rot, ps.interleaved,
+                                    tok_pos, d, lane, row >= first_q ? qs + (size_t)(row - first_q) * d : k_new);
     }
-    for (int row = wave + 8; row < n_rows; row += 4)
-      norm_rope_head<bf16, PARTS>(packed_head(head_of(row)), ps.qw, ps.eps, ps.cos_t, ps.sin_t, ps.rot, ps.interleaved,
-                                  tok_pos, d, lane, qs + (size_t)(row - first_q) * d);
     if (owner && wave < 2) wait_global();   // the new key and value are written (what the other waves read comes after the barrier)
     lds_barrier();     // the heads are in LDS
     const bf16* qrow = qs + (size_t)(col ? r : 0) * d;

@@ -55,8 +55,17 @@ struct HeadRegs {
                                        int interleaved, int pos, int d, int lane) {
     const int half = rot / 2;
     const float* bs = x.bias;
+    // (a group of 64 lanes none of which holds anything is skipped as a whole: the tests on p are
+    // the same for every lane)
+    const float* c = cos_t + (size_t)pos * half;
+    const float* sn_row = sin_t + (size_t)pos * half;
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
+      xa[p] = xb[p] = 0.f;
+      wa[p] = wb[p] = 1.f;
+      cs[p] = 1.f;
+      sn[p] = 0.f;
+      if (kWave * p >= half) continue;
       const int i = lane + kWave * p;
       const bool ok = i < half;
       const int ia = interleaved ? 2 * i : i;
@@ -65,21 +74,18 @@ struct HeadRegs {
       xb[p] = ok ? x.raw(ib) + (bs ? bs[ib] : 0.f) : 0.f;
       wa[p] = (ok && w) ? w[ia] : 1.f;
       wb[p] = (ok && w) ? w[ib] : 1.f;
+      cs[p] = ok ? c[i] : 1.f;
+      sn[p] = ok ? sn_row[i] : 0.f;
     }
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
+      xt[p] = 0.f;
+      wt[p] = 1.f;
+      if (rot + kWave * p >= d) continue;
       const int i = rot + lane + kWave * p;
       const bool ok = i < d;
       xt[p] = ok ? x.raw(i) + (bs ? bs[i] : 0.f) : 0.f;
       wt[p] = (ok && w) ? w[i] : 1.f;
-    }
-    const float* c = cos_t + (size_t)pos * half;
-    const float* sn_row = sin_t + (size_t)pos * half;
-#pragma unroll
-    for (int p = 0; p < 2; ++p) {
-      const int i = lane + kWave * p;
-      cs[p] = i < half ? c[i] : 1.f;
-      sn[p] = i < half ? sn_row[i] : 0.f;
     }
   }
 
@@ -100,6 +106,7 @@ struct HeadRegs {
     }
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
+      if (kWave * p >= half) continue;
       const int i = lane + kWave * p;
       if (i < half) {
         // the reference rounds the normed value to the activation type before rotating
@@ -112,6 +119,7 @@ struct HeadRegs {
     }
 #pragma unroll
     for (int p = 0; p < 4; ++p) {  // dims beyond the rotary part
+      if (rot + kWave * p >= d) continue;
       const int i = rot + lane + kWave * p;
       if (i < d) dst[i] = from_float<T>(xt[p] * inv * wt[p]);
     }
