@@ -23,6 +23,24 @@ def _rand(shape, dtype, gen, scale=1.0):
     return (torch.randn(shape, generator=gen) * scale).to(dtype)
 
 
+def test_lanes_exchange_across_powers_of_two():
+    """The exchange between lanes that the reductions are built from (lane swaps and data-parallel
+    moves instead of a trip through LDS): lane l gets lane l ^ 1, 2, 4, 8, 16, 32's value; the
+    wave's sum is the sum in the order of the butterfly from 32 down to 1, the same bits in every lane."""
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(3)
+    v = torch.randn(64, generator=g) * torch.logspace(-3, 3, 64)
+    out = kernels.lane_xor_probe(v.to(DEV)).cpu()
+    lanes = torch.arange(64)
+    for i in range(6):
+        assert torch.equal(out[i], v[lanes ^ (1 << i)]), i
+    s = v.clone()
+    for off in (32, 16, 8, 4, 2, 1):
+        s = s + s[lanes ^ off]
+    assert torch.equal(out[6], s) and len(set(out[6].tolist())) == 1
+    assert torch.equal(out[7], torch.full((64,), float(v.max())))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("V,H,T", [(301, 72, 37), (1000, 4096, 5)])
 def test_embed(dtype, V, H, T):

@@ -260,8 +260,8 @@ __global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
     float mx = sc[0];
 #pragma unroll
     for (int v = 1; v < 8; ++v) mx = fmaxf(mx, sc[v]);
-    mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    mx = fmaxf(mx, lane_xor<16>(mx));
+    mx = fmaxf(mx, lane_xor<32>(mx));
     const float m_new = fmaxf(m_run, mx);
     const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
     const float corr = __builtin_amdgcn_exp2f(m_run - m_safe);
@@ -286,8 +286,8 @@ __global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
     if (more) load_v(kb + 128);
   }
   // the column's sum over the four lane groups
-  float lt = l_run + __shfl_xor(l_run, 16, kWave);
-  lt += __shfl_xor(lt, 32, kWave);
+  float lt = l_run + lane_xor<16>(l_run);
+  lt += lane_xor<32>(lt);
   if (col) {
     if (j == 0) {
       lds_ml[(wave * g + r) * 2] = m_run;

@@ -244,8 +244,8 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_prefill_lds_kernel(
 #pragma unroll
         for (int ct = 0; ct < NQT; ++ct) {
           float mc = mx[ct];
-          mc = fmaxf(mc, __shfl_xor(mc, 16, kWave));
-          mc = fmaxf(mc, __shfl_xor(mc, 32, kWave));
+          mc = fmaxf(mc, lane_xor<16>(mc));
+          mc = fmaxf(mc, lane_xor<32>(mc));
           const float m_new = fmaxf(m_run[ct], mc);
           const float corr = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_run[ct] - m_new);
           l_run[ct] *= corr;
@@ -294,8 +294,8 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_prefill_lds_kernel(
   if (!active) return;
 #pragma unroll
   for (int ct = 0; ct < NQT; ++ct) {
-    float lt = l_run[ct] + __shfl_xor(l_run[ct], 16, kWave);
-    lt += __shfl_xor(lt, 32, kWave);
+    float lt = l_run[ct] + lane_xor<16>(l_run[ct]);
+    lt += lane_xor<32>(lt);
     const int tile = wave * NQT + ct;
     const int pb = tile / GH, hh = tile - pb * GH;
     const int qi = q0_blk + 16 * pb + r;

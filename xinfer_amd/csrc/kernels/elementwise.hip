@@ -441,6 +441,20 @@ __global__ __launch_bounds__(1024) void qk_norm_rope_kvt_bf16_kernel(
   }
 }
 
+// out[i][l] = in[l ^ (1 << i)] for i = 0 .. 5, by `lane_xor` (for its test)
+__global__ void lane_xor_probe_kernel(const float* __restrict__ in, float* __restrict__ out) {
+  const int l = threadIdx.x;
+  const float v = in[l];
+  out[0 * kWave + l] = lane_xor<1>(v);
+  out[1 * kWave + l] = lane_xor<2>(v);
+  out[2 * kWave + l] = lane_xor<4>(v);
+  out[3 * kWave + l] = lane_xor<8>(v);
+  out[4 * kWave + l] = lane_xor<16>(v);
+  out[5 * kWave + l] = lane_xor<32>(v);
+  out[6 * kWave + l] = wave_sum(v);
+  out[7 * kWave + l] = wave_max(v);
+}
+
 }  // namespace xi
 
 using namespace xi;
@@ -448,6 +462,13 @@ using namespace xi;
 extern "C" {
 
 const char* xi_last_error() { return g_error; }
+
+// in [64] float32 -> out [8][64]: lanes exchanged across 1, 2, 4, 8, 16, 32, the wave's sum and maximum
+int xi_lane_xor_probe(const float* in, float* out, hipStream_t stream) {
+  lane_xor_probe_kernel<<<1, kWave, 0, stream>>>(in, out);
+  XI_LAUNCH_CHECK("lane_xor_probe");
+  return 0;
+}
 
 int xi_embed(const void* table, int dtype, const int* ids, float* out, int n_tok, int H, float scale,
              hipStream_t stream) {

@@ -214,8 +214,11 @@ __global__ __launch_bounds__(NW * 64) void linear_skinny_kernel(const bf16* __re
     float t = 0.f;
 #pragma unroll
     for (int i = 0; i < kSsLoads; ++i) t += ss_mine[i];
-#pragma unroll
-    for (int o = 16; o; o >>= 1) t += __shfl_xor(t, o, kWave);
+    t += lane_xor<16>(t);
+    t += lane_xor<8>(t);
+    t += lane_xor<4>(t);
+    t += lane_xor<2>(t);
+    t += lane_xor<1>(t);
     if ((threadIdx.x & 31) == 0) fold_lds[threadIdx.x >> 5] = rsqrtf(t * fold.inv_h + fold.eps);
   }
 #pragma unroll

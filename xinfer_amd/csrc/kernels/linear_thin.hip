@@ -171,8 +171,10 @@ __global__ __launch_bounds__(256) void linear_thin_kernel(const bf16* __restrict
     float t = 0.f;
 #pragma unroll
     for (int i = 0; i < kThinSsLoads; ++i) t += ss_mine[i];
-#pragma unroll
-    for (int o = 8; o; o >>= 1) t += __shfl_xor(t, o, kWave);
+    t += lane_xor<8>(t);
+    t += lane_xor<4>(t);
+    t += lane_xor<2>(t);
+    t += lane_xor<1>(t);
     if ((tid & 15) == 0) side[tid >> 4] = rsqrtf(t * fold.inv_h + fold.eps);
   }
   __syncthreads();

@@ -31,6 +31,22 @@ constexpr int kSampleWaves = kSampleThreads / kWave;
 
 __device__ __forceinline__ float block_sum_f(float v, float* s) { return block_sum<kSampleWaves>(v, s); }
 
+// The wave's largest value and, among equal ones, the lowest index, in every lane.
+template <int OFF>
+__device__ __forceinline__ void argmax_with(float& best, int& idx) {
+  const float ob = lane_xor<OFF>(best);
+  const int oi = lane_xor<OFF>(idx);
+  if (ob > best || (ob == best && oi < idx)) { best = ob; idx = oi; }
+}
+__device__ __forceinline__ void wave_argmax(float& best, int& idx) {
+  argmax_with<32>(best, idx);
+  argmax_with<16>(best, idx);
+  argmax_with<8>(best, idx);
+  argmax_with<4>(best, idx);
+  argmax_with<2>(best, idx);
+  argmax_with<1>(best, idx);
+}
+
 __device__ __forceinline__ int block_sum_i(int v, int* s) {
 #pragma unroll
   for (int off = kWave / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
@@ -64,12 +80,7 @@ __device__ int block_argmax(const float* row, int V, float* sf, int* si) {
     const float v = row[i];
     if (v > best || (v == best && i < idx)) { best = v; idx = i; }
   }
-#pragma unroll
-  for (int off = kWave / 2; off > 0; off >>= 1) {
-    const float ob = __shfl_xor(best, off, kWave);
-    const int oi = __shfl_xor(idx, off, kWave);
-    if (ob > best || (ob == best && oi < idx)) { best = ob; idx = oi; }
-  }
+  wave_argmax(best, idx);
   __syncthreads();
   if ((threadIdx.x & (kWave - 1)) == 0) { sf[threadIdx.x / kWave] = best; si[threadIdx.x / kWave] = idx; }
   __syncthreads();
@@ -105,12 +116,7 @@ __global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __rest
     const float v = r[i];
     if (v > best || (v == best && i < idx)) { best = v; idx = i; }
   }
-#pragma unroll
-  for (int off = kWave / 2; off > 0; off >>= 1) {
-    const float ob = __shfl_xor(best, off, kWave);
-    const int oi = __shfl_xor(idx, off, kWave);
-    if (ob > best || (ob == best && oi < idx)) { best = ob; idx = oi; }
-  }
+  wave_argmax(best, idx);
   if ((threadIdx.x & (kWave - 1)) == 0) { sf[threadIdx.x / kWave] = best; si[threadIdx.x / kWave] = idx; }
   __syncthreads();
   if (threadIdx.x == 0) {
@@ -131,12 +137,7 @@ __global__ __launch_bounds__(64) void argmax_merge_kernel(const float* __restric
     const int i = pidx[(size_t)row * n_chunks + c];
     if (v > best || (v == best && i < idx)) { best = v; idx = i; }
   }
-#pragma unroll
-  for (int off = kWave / 2; off > 0; off >>= 1) {
-    const float ob = __shfl_xor(best, off, kWave);
-    const int oi = __shfl_xor(idx, off, kWave);
-    if (ob > best || (ob == best && oi < idx)) { best = ob; idx = oi; }
-  }
+  wave_argmax(best, idx);
   if (threadIdx.x == 0) out[row] = idx;
 }
 

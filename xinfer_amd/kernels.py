@@ -108,6 +108,18 @@ def stream_read(t: torch.Tensor, workgroups: int = 2048, chunk_bytes: int = 1 <<
                              ctypes.c_int64(chunk_bytes), _stream()))
 
 
+def lane_xor_probe(values: torch.Tensor) -> torch.Tensor:
+    """values [64] float32 -> [8, 64]: row i < 6 holds values[l ^ (1 << i)] as the kernels' exchange
+    between lanes gives it, row 6 the wave's sum and row 7 its maximum in every lane (for tests)."""
+    _dev(values)
+    _want(values, torch.float32, "lane_xor_probe: values")
+    if values.shape != (64,):
+        raise KernelError("lane_xor_probe: 64 values, one a lane")
+    out = torch.empty((8, 64), dtype=torch.float32, device=values.device)
+    _ok(lib().xi_lane_xor_probe(_p(values), _p(out), _stream()))
+    return out
+
+
 def softcap_(logits: torch.Tensor, cap: float) -> torch.Tensor:
     """logits = cap * tanh(logits / cap), in place, float32."""
     _dev(logits)
