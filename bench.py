@@ -21,7 +21,8 @@ larger configurations through the whole engine (scheduler, chunked prefill, cont
 batching, greedy sampling) and print their own JSON line: total generated tokens per second.
 `--workload many06b` is the one run the reference publishes a figure for (Qwen3-0.6B, 256
 concurrent requests, 1,024 new tokens each); its line carries the ratio to that figure, which
-was measured on other hardware.
+was measured on other hardware.  `--workload many8b` is 192 concurrent requests (prompts of 64
+to 512 tokens, 256 new tokens each) at Qwen3-8B sizes: decode steps of 129 to 256 rows.
 """
 from __future__ import annotations
 
@@ -53,6 +54,8 @@ WORKLOADS = {
                     chunk=2048, max_model_len=1088, reference_tok_s=10944.62),
     "serve14b": dict(model=QWEN3_14B, name="Qwen3-14B layer sizes", requests=64, prompt=(128, 2048), new_tokens=256,
                      chunk=2048, max_model_len=2304),
+    "many8b": dict(model=QWEN3_8B, name="Qwen3-8B layer sizes", requests=192, prompt=(64, 512), new_tokens=256,
+                   chunk=2048, max_model_len=768),
     "long32b": dict(model=QWEN3_32B, name="Qwen3-32B layer sizes", requests=16, prompt=(8192, 8192), new_tokens=512,
                     chunk=2048, max_model_len=8704),
 }
