@@ -7,7 +7,9 @@ Prints ONE JSON line.  `value` is decoded tokens per second at batch 8 and the c
 length the configuration names (the last timed step ends at that length); a "step" is one
 decode step through the engine's own step function (mixed-batch path, paged cache,
 kernels) followed by greedy sampling on the GPU.  Beside it: the prefill of one
-2,048-token prompt, the decode step's bandwidth roofline, and decode at batch 1 and 64.
+2,048-token prompt, the decode step's bandwidth roofline, decode at batch 1 and 64 (`points`,
+and each one's own roofline in `points_roofline`), and decode at batch 8 with four times the
+context (`further`).
 
 `--peaks` adds what this card itself reaches (a read-only stream, one large square product) and
 the fractions of those, beside the fractions of the published peaks that the line always has.
@@ -251,11 +253,11 @@ def main() -> int:
     def sync():
         torch.cuda.synchronize()
 
-    def decode_run(batch, steps, warmup):
-        """`batch` requests whose caches already hold CONTEXT - steps - warmup tokens decode
-        steps + warmup tokens, so that the last timed step ends at CONTEXT."""
+    def decode_run(batch, steps, warmup, context=None):
+        """`batch` requests whose caches already hold context - steps - warmup tokens decode
+        steps + warmup tokens, so that the last timed step ends at `context` (CONTEXT unless given)."""
         prep = runner.graph_after          # steps before the warm-up in which the decode graph is recorded
-        start = CONTEXT - steps - warmup - prep
+        start = (context or CONTEXT) - steps - warmup - prep
         rids = list(range(100, 100 + batch))
         for rid in rids:
             runner.add_request(rid)
@@ -300,10 +302,13 @@ def main() -> int:
         return 0
     sec = decode_run(args.batch, args.steps, args.warmup)
     wb, kvb = weight_bytes(cfg), kv_bytes_per_token(cfg)
-    # mean cache length over the timed steps (it grows by one each step, ending at CONTEXT)
-    mean_ctx = CONTEXT - (args.steps - 1) / 2.0
-    step_bytes = wb + args.batch * mean_ctx * kvb
-    achieved = step_bytes / sec / 1e9
+
+    def stream_rate(batch, steps, seconds, context):
+        """GB/s of a decode step: every weight once and the cache of its requests, over its time.  The
+        cache length is the mean over the timed steps (it grows by one a step and ends at `context`)."""
+        return (wb + batch * (context - (steps - 1) / 2.0) * kvb) / seconds / 1e9
+
+    achieved = stream_rate(args.batch, args.steps, sec, CONTEXT)
     out = {
         "metric": f"decode tok/s at batch {args.batch}, {model_name} bf16", "value": round(args.batch / sec, 2),
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -341,12 +346,25 @@ def main() -> int:
         out["prefill"]["frac_of_measured"] = round(flops / psec / (peaks[1] * 1e12), 4)
     print(f"[bench] prefill {PREFILL_TOKENS}: {psec * 1e3:.2f} ms", file=sys.stderr, flush=True)
     if not args.skip_points:
-        points = {}
+        points, roofs = {}, {}
+        k, w = max(8, args.steps // 2), max(2, args.warmup // 2)
         for b in (1, 64):
-            s = decode_run(b, max(8, args.steps // 2), max(2, args.warmup // 2))
+            s = decode_run(b, k, w)
             points[f"decode_b{b}"] = round(b / s, 2)
+            rate = stream_rate(b, k, s, CONTEXT)
+            roofs[f"decode_b{b}"] = {"ms_per_step": round(s * 1e3, 4), "achieved": round(rate, 1),
+                                     "frac": round(rate / HBM_GBPS, 4)}
             print(f"[bench] decode b{b}: {s * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
         out["points"] = points
+        out["points_roofline"] = roofs          # GB/s of each point's step and its fraction of the 8 TB/s peak
+        # one point at a longer context: batch 8 with 16,384 tokens in every request's cache
+        far = 4 * CONTEXT
+        if max_batch * (-(-CONTEXT // page)) >= 8 * (-(-far // page)) and far <= cfg.max_position_embeddings:
+            s = decode_run(8, k, w, context=far)
+            rate = stream_rate(8, k, s, far)
+            out["further"] = {"decode_b8_ctx": far, "value": round(8 / s, 2), "ms_per_step": round(s * 1e3, 4),
+                              "achieved": round(rate, 1), "frac": round(rate / HBM_GBPS, 4)}
+            print(f"[bench] decode b8 at context {far}: {s * 1e3:.3f} ms/step", file=sys.stderr, flush=True)
     print(json.dumps(out), flush=True)
     return 0
 

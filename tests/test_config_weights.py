@@ -133,6 +133,27 @@ def test_random_folder_round_trip(tmp_path):
         assert torch.equal(f.get_tensor("model.layers.2.mlp.down_proj.weight"), w)
 
 
+def test_counter_normal_values_depend_on_key_and_index_alone():
+    """The CPU half of the random weights: a value is a function of (key, index), whatever the
+    piece it is made in; the values are normal (moments, tails, a Kolmogorov-Smirnov distance)
+    and two keys share nothing."""
+    import numpy as np
+    from xinfer_amd.weights.counter_normal import counter_normal
+    x = counter_normal(0x1234_5678_9ABC_DEF0, 0, 300_000)
+    assert x.dtype == np.float32 and np.isfinite(x).all()
+    assert np.array_equal(counter_normal(0x1234_5678_9ABC_DEF0, 65_530, 70_001), x[65_530:135_531])
+    assert abs(float(x.mean())) < 0.01 and abs(float(x.std()) - 1.0) < 0.01
+    assert abs(float((np.abs(x) < 0.6745).mean()) - 0.5) < 0.005 and abs(float((x > 2).mean()) - 0.02275) < 0.002
+    grid = np.sort(x.astype(np.float64))
+    from math import erf, sqrt
+    cdf = np.array([0.5 * (1 + erf(v / sqrt(2))) for v in grid[::100]])
+    assert float(np.abs(cdf - np.arange(0, grid.size, 100) / grid.size).max()) < 0.005
+    y = counter_normal(0x1234_5678_9ABC_DEF1, 0, 300_000)
+    assert abs(float(np.corrcoef(x, y)[0, 1])) < 0.01 and abs(float(np.corrcoef(x[:-1], x[1:])[0, 1])) < 0.01
+    z = counter_normal(7, 5, 1000, scale=0.02, shift=1.0)
+    assert np.array_equal(z, counter_normal(7, 5, 1000) * np.float32(0.02) + np.float32(1.0))
+
+
 def test_one_error_lists_everything_wrong(tmp_path):
     d = write_random_model(str(tmp_path / "m"), TINY["A"]["config"], seed=0)
     st = SafetensorsStore(d)

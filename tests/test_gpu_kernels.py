@@ -1203,3 +1203,28 @@ def test_attention_mfma_far_key_and_page_edges():
         for small in (0, 1, 2):
             out = kernels.attention_prefill_bf16(q, kc, vt, bt, tiles.to(DEV), cu.to(DEV), ctx.to(DEV), scale, 0, small=small)
             assert (out.cpu().double() - ref).abs().max() / ref.abs().max() < _tol(torch.bfloat16, 2), (far, small)
+
+
+# ---- random weights are the same on the CPU and on the GPU ------------------------------------------------
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_random_weights_do_not_depend_on_the_device(dtype):
+    """A linear tensor of [1000, 4096] and a norm tensor, made on the CPU (numpy) and on the GPU
+    (the kernel) from the same seed: equal bit for bit, in pieces too."""
+    import numpy as np
+    from xinfer_amd import kernels
+    from xinfer_amd.weights import RandomStore, TensorDecl
+    from xinfer_amd.weights.counter_normal import counter_normal
+    decls = [TensorDecl("model.layers.3.mlp.down_proj.weight", (1000, 4096)),
+             TensorDecl("model.norm.weight", (4096,), "norm"), TensorDecl("b", (77,), "zeros")]
+    rs = RandomStore(decls, 11, 0.02, 0.1, dtype)
+    for d in decls:
+        cpu, gpu = rs.get(d.name, None, "cpu"), rs.get(d.name, None, "cuda:0")
+        assert cpu.dtype == gpu.dtype == dtype and cpu.shape == tuple(d.shape)
+        assert torch.equal(cpu, gpu.cpu()), d.name
+    w = rs.get(decls[0].name, torch.float32, "cuda:0")
+    assert abs(float(w.std()) - 0.02) < 2e-4 and abs(float(rs.get("model.norm.weight", torch.float32, "cuda:0").mean()) - 1) < 0.01
+    # any piece of the stream, any key
+    for key, first, n in [(0, 0, 5000), (2 ** 64 - 1, 123_456_789_012, 4099), (0x9E3779B97F4A7C15, 2 ** 33 + 5, 70_000)]:
+        out = torch.empty(n, dtype=torch.float32, device="cuda:0")
+        kernels.counter_normal_(out, key, 1.0, 0.0, first=first)
+        assert np.array_equal(out.cpu().numpy(), counter_normal(key, first, n)), (key, first, n)

@@ -133,9 +133,134 @@ def test_decode_batch_of_eight_unequal_lengths(dtype, long_model):
     model = load_model(d, dtype, DEV)
     runner = ModelRunner(model, page_size=page, num_pages=sum(-(-n // page) for n in lens), max_requests=8, graph_after=3)
     got = harness.replay(runner, steps)
-    assert runner.graph_replays == tail - 2 and list(runner._graphs) == [(8, 6144, False)]
+    assert runner.graph_replays == tail - 3 and list(runner._graphs) == [(8, 6144, False)]
     rel = harness.compare(got, _ref(pm, reqs), harness.TOL[dtype], f"LONG/{dtype}/batch of eight")
     print(f"LONG/{dtype}/batch of eight: worst error {rel:.2e} of the largest logit")
+
+
+# ---- the matrix-core attention kernels against the generic kernel, inside the model ---------------------------
+_long_dirs = {}
+
+
+def _long_dir(tmp_path_factory, sharpen):
+    """The LONG model folder with its q_norm weights multiplied by `sharpen`."""
+    from safetensors.torch import load_file, save_file
+    from xinfer_amd.weights import write_random_model
+    if sharpen not in _long_dirs:
+        d = str(tmp_path_factory.mktemp(f"long_model_{sharpen}"))
+        write_random_model(d, LONG["config"], LONG["seed"], LONG["linear_std"], LONG["norm_std"])
+        tensors = load_file(d + "/model.safetensors")
+        for name in tensors:
+            if name.endswith("q_norm.weight"):
+                tensors[name] = (tensors[name].float() * sharpen).to(tensors[name].dtype)
+        save_file(tensors, d + "/model.safetensors")
+        _long_dirs[sharpen] = d
+    return _long_dirs[sharpen]
+
+
+def _long_steps():
+    """The long request's steps (portions behind 0, 2,048 and 4,108 cached keys, single tokens across
+    4,096 and to the end) and eight requests of unequal lengths whose last six tokens come together."""
+    toks = _one_long_request()["long"]
+    cuts = [2048, 2000] + [1] * 60 + [2048] + [1] * (6200 - 4108 - 2048)
+    steps, p = [], 0
+    for n in cuts:
+        steps.append({"step": len(steps), "entries": [{"id": "long", "tokens": toks[p:p + n], "want": list(range(max(0, n - 4), n))}],
+                      "end": ["long"] if p + n == len(toks) else []})
+        p += n
+    rng = random.Random(47)
+    reqs = {f"r{i}": harness.random_prompt(rng, n, LONG["config"]["vocab_size"]) for i, n in enumerate([900, 1500, 2100, 2600, 3300, 4090, 4700, 5800])}
+    tail, pos = 6, {r: 0 for r in reqs}
+    while any(pos[r] < len(reqs[r]) - tail for r in reqs):
+        entries, left = [], 2048
+        for r in reqs:
+            n = min(left, len(reqs[r]) - tail - pos[r])
+            if n > 0:
+                entries.append({"id": r, "tokens": reqs[r][pos[r]:pos[r] + n], "want": list(range(max(0, n - 2), n))})
+                pos[r] += n
+                left -= n
+        steps.append({"step": len(steps), "entries": entries, "end": []})
+    for k in range(tail):
+        steps.append({"step": len(steps), "end": list(reqs) if k == tail - 1 else [], "entries": [
+            {"id": r, "tokens": [reqs[r][len(reqs[r]) - tail + k]], "want": [0]} for r in reqs]})
+    return steps
+
+
+@pytest.mark.parametrize("sharpen", [1.5, 3.0])
+def test_matrix_core_attention_agrees_with_the_generic_kernel_inside_the_model(sharpen, tmp_path_factory):
+    """The same bfloat16 steps twice: as the engine runs them (the ring prefill kernel, the split-K
+    decode kernel that norms, rotates and stores its own heads, graphs), and with every attention
+    call sent to the generic kernel (one thread a score, float32 softmax, no matrix cores), which
+    the float32 tests hold against the plain model.  Both runs see the same bfloat16 weights and
+    the same rounding of activations between kernels, so what is left between them is the
+    attention kernels alone: the matrix-core kernels round the softmax weights to bfloat16
+    before the second product and sum in other orders.  A key that one of them dropped or
+    misplaced would move a row by far more than that, at any sharpness of the scores."""
+    from xinfer_amd import kernels
+    from xinfer_amd.engine import ModelRunner, load_model
+    d = _long_dir(tmp_path_factory, sharpen)
+    page = LONG["page_size"]
+    steps = _long_steps()
+    pages = harness.tokens_needed(steps, page) // page
+    model = load_model(d, "bfloat16", DEV)
+    runner = ModelRunner(model, page_size=page, num_pages=pages, max_requests=8, graph_after=3)
+    got = harness.replay(runner, steps)
+    assert runner.graph_replays > 60
+    del runner
+
+    def generic(q, k_cache, v_cache, ctx, group, scale, window=0, v_transposed=False):
+        return kernels.attention_generic(q, k_cache, v_cache, ctx.block_tables[group], ctx.tok_seq, ctx.positions, scale,
+                                         window, v_transposed=v_transposed)
+
+    mixers = [b.mixer for b in model.blocks]
+    inner = kernels.attention
+    kernels.attention = generic
+    for m in mixers:
+        m.decode_packed = False
+    try:
+        plain_kernel = harness.replay(ModelRunner(model, page_size=page, num_pages=pages, max_requests=8, graph_after=3), steps)
+    finally:
+        kernels.attention = inner
+        for m in mixers:
+            m.decode_packed = True
+    assert got.keys() == plain_kernel.keys()
+    scale = max(float(v.abs().max()) for v in plain_kernel.values())
+    worst = max((float((got[k] - plain_kernel[k]).abs().max()), k) for k in got)
+    print(f"LONG/bfloat16/sharpen {sharpen}: the matrix-core kernels differ from the generic one by at most "
+          f"{worst[0] / scale:.2e} of the largest logit (request {worst[1][0]}, position {worst[1][1]})")
+    assert worst[0] < 2.0 ** -7 * scale, worst
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_decode_batch_of_eight_equal_lengths_at_4096(dtype, long_model):
+    """Eight requests of 4,082 to 4,096 tokens decode their last twelve tokens together: sequences
+    about equally long, recorded at the third step for the bucket of 4,096 keys (four splits of
+    1,024 keys a sequence) and replayed nine times; against the plain model."""
+    from xinfer_amd.engine import ModelRunner, load_model
+    d, pm = long_model
+    rng = random.Random(53)
+    base = [_one_long_request()["long"], harness.random_prompt(rng, 4096, LONG["config"]["vocab_size"])]
+    reqs = {f"e{i}": base[i % 2][:4096 - 2 * i] for i in range(8)}
+    tail, budget = 12, 2048
+    steps, pos = [], {r: 0 for r in reqs}
+    while any(pos[r] < len(reqs[r]) - tail for r in reqs):
+        entries, left = [], budget
+        for r in reqs:
+            n = min(left, len(reqs[r]) - tail - pos[r])
+            if n > 0:
+                entries.append({"id": r, "tokens": reqs[r][pos[r]:pos[r] + n], "want": [n - 1]})
+                pos[r] += n
+                left -= n
+        steps.append({"step": len(steps), "entries": entries, "end": []})
+    for k in range(tail):
+        steps.append({"step": len(steps), "end": list(reqs) if k == tail - 1 else [], "entries": [
+            {"id": r, "tokens": [reqs[r][len(reqs[r]) - tail + k]], "want": [0]} for r in reqs]})
+    page = LONG["page_size"]
+    runner = ModelRunner(load_model(d, dtype, DEV), page_size=page, num_pages=8 * (4096 // page), max_requests=8, graph_after=3)
+    got = harness.replay(runner, steps)
+    assert list(runner._graphs) == [(8, 4096, True)] and runner.graph_replays == tail - 3
+    rel = harness.compare(got, _ref(pm, reqs), harness.TOL[dtype], f"LONG/{dtype}/eight of equal length")
+    print(f"LONG/{dtype}/eight of equal length: worst error {rel:.2e} of the largest logit")
 
 
 # ---- the reference's attention probe cases --------------------------------------------------------

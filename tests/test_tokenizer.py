@@ -38,6 +38,20 @@ def test_stream_text_waits_for_whole_characters(tmp_path):
     assert "�" in "".join(tok.decode([i]) for i in ids)
 
 
+def test_stream_text_held_back_is_flushed_at_the_end(tmp_path):
+    """A request cut inside a character that spans several tokens (by max_tokens, say): the pieces
+    and what `finish` hands on are together the text of all tokens, as one decode gives it."""
+    tok = FileTokenizer(_byte_level_folder(tmp_path))
+    for text, cut in (("a ✓", 1), ("wörld", 4), ("ok", 0), ("é", 1)):
+        ids = tok.encode(text)
+        ids = ids[:len(ids) - cut]
+        inc = IncrementalText(tok)
+        pieces = [inc.add(ids[:n]) for n in range(1, len(ids) + 1)]
+        rest = inc.finish(ids)
+        assert "".join(pieces) + rest == tok.decode(ids), (text, cut)
+        assert (rest != "") == (cut > 0) and inc.finish(ids) == ""
+
+
 def test_chat_template_of_the_folder_is_rendered(tmp_path):
     """tokenizer_config.json's chat_template is rendered with the reference's variables
     (/root/reference/src/utils/chat_template.rs:459-472)."""

@@ -81,3 +81,31 @@ def test_static_argmax_refuses_sizes_beyond_its_scratch():
     assert rc == 0, lib.xi_last_error().decode()
     torch.cuda.synchronize()
     assert out[:most].tolist() == [16000] * most
+
+
+def test_static_argmax_recorded_in_a_graph():
+    """After `xi_argmax_static_init` (outside the capture) the two-stage form is recorded into a HIP
+    graph, which holds two kernels and no memset, and replayed with other logits in place, with
+    eager work between the replays; every replay against `xi_argmax`."""
+    lib = _library()
+    dev = torch.device("cuda:0")
+    assert lib.xi_argmax_static_init() == 0, lib.xi_last_error().decode()
+    gen = torch.Generator(device="cpu").manual_seed(12)
+    rows, V = 9, 151936
+    logits = torch.randn((rows, V), generator=gen, dtype=torch.float32).to(dev)
+    out = torch.full((rows,), -1, dtype=torch.int32, device=dev)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):                 # (the capture runs on a stream of its own)
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        rc = lib.xi_argmax_static(logits.data_ptr(), rows, V, out.data_ptr(), stream)
+    assert rc == 0, lib.xi_last_error().decode()
+    for k in range(3):
+        fresh = torch.randn((rows, V), generator=gen, dtype=torch.float32)
+        fresh[k, V - 1 - k] = 40.0
+        logits.copy_(fresh.to(dev))
+        out.fill_(-1)
+        graph.replay()
+        torch.cuda.synchronize()
+        _, want = _both(lib, logits)              # eager calls of both entry points between the replays
+        assert torch.equal(out.cpu(), want) and int(out[k]) == V - 1 - k, k

@@ -75,7 +75,9 @@ class GenerationOutput:
 class StreamItem:
     """An item of an `EngineStream` (xinfer.pyi:160-180).  datatype / data:
     "TOKEN" / the token's text; "TOKEN_ID" / its id; "DONE" / (prompt_start_time,
-    decode_start_time, decode_finish_time, decoded_length); "ERROR" / a message."""
+    decode_start_time, decode_finish_time, decoded_length); "COMPLETION" / (prompt_start_time,
+    decode_start_time, decode_finish_time, token ids), the one item of a request that is not
+    streamed; "ERROR" / a message."""
     datatype: str
     data: object
 

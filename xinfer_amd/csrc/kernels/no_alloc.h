@@ -13,6 +13,12 @@ extern "C" {
 // xi_argmax_static_max_rows() * 32 chunks * (4 + 4) bytes = 64 KiB per GPU until the process ends.
 int xi_argmax_static_max_rows();
 
+// Resolves the array's address on the current device (one runtime call, which is no stream
+// operation and may load the code object); later calls on that device make no such call.  A caller
+// that records `xi_argmax_static` into a HIP graph calls this, or the entry point itself once,
+// before the capture begins.  Returns 0 or non-zero as below.
+int xi_argmax_static_init();
+
 // out[r] = index of the largest of logits[r, 0..V) (the lowest index among equals), for
 // rows <= xi_argmax_static_max_rows().  `logits` float32 [rows, V] and `out` int32 [rows] are
 // device memory of the current device; the kernels run on `stream`.  Calls no hipMalloc, hipFree

@@ -14,6 +14,7 @@
 #include "common.h"
 #include "no_alloc.h"
 
+#include <atomic>
 #include <mutex>
 
 // Scratch of `xi_argmax_static`: per row and chunk the winner's value (float) and index (int).
@@ -442,25 +443,35 @@ int xi_argmax(const float* logits, int rows, int V, int* out, float* pval, int* 
 // Each GPU holds its own copy of `scratch` at its own address; the address is asked for once
 // per device, with that device current, and kept.
 constexpr int kStaticMaxDevices = 64;
-static void* g_static_scratch[kStaticMaxDevices];
+static std::atomic<void*> g_static_scratch[kStaticMaxDevices];
 static std::mutex g_static_mutex;
 
+// The array's address on the current device.  The first call on a device asks the runtime for it
+// (under the mutex, once); later calls read what was kept and make no runtime call but hipGetDevice.
 static int static_scratch(unsigned char** ptr) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   XI_CHECK(e == hipSuccess, "argmax_static: hipGetDevice failed: %s", hipGetErrorString(e));
   XI_CHECK(dev >= 0 && dev < kStaticMaxDevices, "argmax_static: device %d is beyond the %d this library keeps", dev,
            kStaticMaxDevices);
-  std::lock_guard<std::mutex> lock(g_static_mutex);
-  if (g_static_scratch[dev] == nullptr) {
-    void* p = nullptr;
-    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-    XI_CHECK(e == hipSuccess && p != nullptr, "argmax_static: hipGetSymbolAddress failed on device %d: %s", dev,
-             hipGetErrorString(e));
-    g_static_scratch[dev] = p;
+  void* p = g_static_scratch[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    p = g_static_scratch[dev].load(std::memory_order_relaxed);
+    if (p == nullptr) {
+      e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      XI_CHECK(e == hipSuccess && p != nullptr, "argmax_static: hipGetSymbolAddress failed on device %d: %s", dev,
+               hipGetErrorString(e));
+      g_static_scratch[dev].store(p, std::memory_order_release);
+    }
   }
-  *ptr = static_cast<unsigned char*>(g_static_scratch[dev]);
+  *ptr = static_cast<unsigned char*>(p);
   return 0;
+}
+
+int xi_argmax_static_init() {
+  unsigned char* base = nullptr;
+  return static_scratch(&base);
 }
 
 int xi_argmax_static_max_rows() { return kStaticArgmaxRows; }

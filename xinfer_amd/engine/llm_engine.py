@@ -334,10 +334,11 @@ class LLMEngine:
         return [self._output(self._finished.pop(rid)) for rid in rids]
 
     def generate_stream(self, params: SamplingParams,
-                        messages: Union[Sequence[Message], str, Sequence[int]]):
+                        messages: Union[Sequence[Message], str, Sequence[int]], completion: bool = False):
         """The reference's streaming entry point (xinfer.pyi:206-216): returns (seq_id,
         prompt_length, stream).  `messages` is a chat (rendered with the chat template), or a
-        prompt as text or token ids."""
+        prompt as text or token ids.  `completion`: the stream yields one COMPLETION item when
+        the request has ended instead of an item per token."""
         if isinstance(messages, str):
             ids = self.tokenizer.encode(messages)
         elif messages and isinstance(messages[0], Message):
@@ -346,7 +347,7 @@ class LLMEngine:
         else:
             ids = [int(t) for t in messages]
         rid = self.add_request(ids, params)
-        return rid, len(ids), EngineStream(self, rid, len(ids))
+        return rid, len(ids), EngineStream(self, rid, len(ids), completion)
 
     def cancel(self, rid: int) -> None:
         """Ends a request now and gives back what it holds (reference: Scheduler::cancel,
@@ -393,11 +394,16 @@ class EngineStream:
     xinfer.pyi:182-189).  Iterating drives the engine: every step also advances whatever other
     requests are live.  Each token comes as a TOKEN_ID item followed by a TOKEN item with the text
     it adds (empty while a character that spans several tokens is incomplete: the text is
-    decoded from all tokens so far and handed on up to where it is final); the last item is
-    DONE.  A stream that is dropped unread takes its request's record with it."""
+    decoded from all tokens so far and handed on up to where it is final); text still held back
+    when the request ends comes as one more TOKEN item, so that the pieces joined are the text of
+    all tokens; the last item is DONE.  With `completion` nothing comes until the request has
+    ended, and then one COMPLETION item with its times and all its token ids (the reference's
+    item for requests that are not streamed, /root/reference/src/core/engine.rs:64-70,1486-1492).
+    A stream that is dropped unread takes its request's record with it."""
 
-    def __init__(self, engine: "LLMEngine", rid: int, prompt_length: int):
+    def __init__(self, engine: "LLMEngine", rid: int, prompt_length: int, completion: bool = False):
         self._engine = engine
+        self._completion = bool(completion)
         self.seq_id = rid
         self.prompt_length = prompt_length
         self.finished = False
@@ -430,6 +436,13 @@ class EngineStream:
                 self.finished = True
                 return StreamItem("ERROR", f"request {self.seq_id} is gone")
             gen = r.generated
+            if self._completion:
+                if self.seq_id in eng._finished:
+                    eng._finished.pop(self.seq_id)
+                    self.finished = True
+                    return StreamItem("COMPLETION", (r.prompt_start, r.decode_start, r.decode_finish, list(gen)))
+                eng.step()
+                continue
             if self._sent < len(gen):
                 tok = gen[self._sent]
                 self._sent += 1
@@ -438,7 +451,12 @@ class EngineStream:
             if self.seq_id in eng._finished:
                 eng._finished.pop(self.seq_id)
                 self.finished = True
-                return StreamItem("DONE", (r.prompt_start, r.decode_start, r.decode_finish, len(gen)))
+                done = StreamItem("DONE", (r.prompt_start, r.decode_start, r.decode_finish, len(gen)))
+                rest = self._text.finish(gen)
+                if rest:
+                    self._pending = [done]
+                    return StreamItem("TOKEN", rest)
+                return done
             eng.step()
         return self._pending.pop(0)
 

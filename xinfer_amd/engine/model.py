@@ -112,7 +112,7 @@ class CausalLM:
                 want_rows: torch.Tensor) -> torch.Tensor:
         """ids int32 [T]; caches: layer index -> the cache that layer owns; want_rows int32
         [R].  Returns float32 logits [R, vocab]."""
-        stream = Stream(self.embedding.forward(ids), None)
+        stream = Stream(self.embedding.forward(ids, ctx), None)
         schedule = self.spec.schedule
         for i, e in enumerate(schedule):
             owner = e.layer if e.cache_of is None else e.cache_of

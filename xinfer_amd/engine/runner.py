@@ -142,8 +142,9 @@ class ModelRunner:
         `use_graphs`: record decode steps of up to `graph_max_batch` requests as HIP graphs; a
         (batch size, context bucket) is recorded the `graph_after`-th time it is seen, so that
         batch sizes that merely pass by (requests finishing one after the other) do not pay
-        for a recording.  A recording costs three passes of the host over the model and the
-        graph's instantiation (12 to 25 ms at 8B to 32B sizes on an MI355X); a replay saves what
+        for a recording.  The step that records runs its tokens once, launch by launch, and then
+        captures the same launches without running them: a recording costs two passes of the host
+        over the model and the graph's instantiation (12 to 25 ms at 8B to 32B sizes on an MI355X); a replay saves what
         the host's launches of a step take beyond the kernels' own time: everything for a small
         model, 0.1 to 0.2 ms a step for a large one, whose kernels outlast the launches.  Left to
         the runner, the count is 3 for a model whose step is bound by the host and 12 otherwise,
@@ -486,18 +487,25 @@ class ModelRunner:
             cur = torch.cuda.current_stream(self.device)
             side = torch.cuda.Stream(self.device)
             side.wait_stream(cur)
-            with torch.cuda.stream(side):       # a first run outside the graph warms every kernel up
-                self.model.forward(ids, ctx, self.layer_caches, every_row)
+            with torch.cuda.stream(side):       # this step's own run; it also warms every kernel up
+                logits = self.model.forward(ids, ctx, self.layer_caches, every_row)
             cur.wait_stream(side)
+            logits.record_stream(cur)           # allocated on the side stream, read on this one from here on
             torch.cuda.synchronize(self.device)
             if self._graph_pool is None:
                 self._graph_pool = torch.cuda.graph_pool_handle()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, pool=self._graph_pool):
-                logits = self.model.forward(ids, ctx, self.layer_caches, every_row)
-            g = _DecodeGraph(graph, d32, d64, logits, want, keep=(every_row, ctx, ids))
+                recorded = self.model.forward(ids, ctx, self.layer_caches, every_row)
+            g = _DecodeGraph(graph, d32, d64, recorded, want, keep=(every_row, ctx, ids))
             self._graphs[key] = g
             self._drop_least_used(keep=key)
+            # the step has run once, above; the capture ran nothing and the graph is first replayed
+            # by the next step of this key.  A part that updates per-request state in place is
+            # thus advanced once a step, also in the step that records.
+            if rows32.size == B and np.array_equal(rows32, np.arange(B)):
+                return logits
+            return logits.index_select(0, want[:rows32.size])
         else:
             self._used(g, key)
             self._upload(a, ids32, all_rows, g.dev32, g.dev64)

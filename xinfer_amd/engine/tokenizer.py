@@ -54,6 +54,15 @@ class IncrementalText:
         self._prefix, self._read = self._read, len(tokens)
         return now[len(before):]
 
+    def finish(self, tokens: Sequence[int]) -> str:
+        """The text that `add` still holds back when the request ends: whatever the tokens since
+        the last piece add, final or not (a request cut inside a character that spans several
+        tokens ends in U+FFFD, as the text of all its tokens does)."""
+        before = self._tok.decode(list(tokens[self._prefix:self._read]))
+        now = self._tok.decode(list(tokens[self._prefix:]))
+        self._prefix, self._read = self._read, len(tokens)
+        return now[len(before):] if len(now) > len(before) else ""
+
 
 class ByteTokenizer:
     """token = byte value modulo the vocabulary; decoding prints the ids."""

@@ -99,6 +99,18 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = 
     return out
 
 
+def counter_normal_(out: torch.Tensor, key: int, scale: float = 1.0, shift: float = 0.0, first: int = 0) -> torch.Tensor:
+    """out.flat[i] = normal(key, first + i) * scale + shift, rounded once to out's type (float32 or
+    bfloat16): seeded normal values that depend on (key, index) alone, bit for bit those of
+    `weights.counter_normal.counter_normal` on the CPU."""
+    _dev(out)
+    if not (0 <= key < 1 << 64) or first < 0:
+        raise KernelError("counter_normal: the key is a 64-bit number and the first index is not negative")
+    _ok(lib().xi_counter_normal(_p(out), ctypes.c_uint64(out.numel()), ctypes.c_uint64(first), ctypes.c_uint64(key),
+                                ctypes.c_float(scale), ctypes.c_float(shift), _code(out, "counter_normal"), _stream()))
+    return out
+
+
 def stream_read(t: torch.Tensor, workgroups: int = 2048, chunk_bytes: int = 1 << 18) -> None:
     """Reads all of a tensor's memory and keeps nothing: the plain read-only stream that the
     weight-streaming kernels are measured against.  A workgroup reads whole chunks of
@@ -716,8 +728,8 @@ def linear_library_split(x: torch.Tensor, w: torch.Tensor, slices: int) -> torch
     if slices < 1 or K % (slices * 8):
         raise KernelError(f"linear_library_split: K={K} is not {slices} slices of a multiple of 8")
     if not (0 < M <= LIBRARY_SPLIT_MOST_ROWS):
-        # (a batched bfloat16 product of 2 x [2048, 6144] by [6144, 4096] ended in a GPU memory fault inside
-        # the library on this image; the float32 form is used for the sizes it has been run at)
+        # (torch.bmm of bfloat16 [2, 2048, 6144] by [2, 6144, 4096] with a bfloat16 result ended in a GPU memory
+        # fault inside the library; only the form with a float32 result is used, at the sizes it has been run at)
         raise KernelError(f"linear_library_split: {M} rows, at most {LIBRARY_SPLIT_MOST_ROWS}")
     xs = x.view(M, slices, K // slices).transpose(0, 1)            # [slices, M, K / slices]
     ws = w.view(N, slices, K // slices).permute(1, 2, 0)            # [slices, K / slices, N]

@@ -17,8 +17,9 @@ runs on the tokens of one step.  A part never learns which model it is in.
   PositionEncoding data for the mixer's fused kernel (for "rope": cos/sin tables)
   Block            forward(stream, ctx, cache) -> stream, the arrangement of the above
                    around the residual stream.
-  TokenEmbedding   forward(ids) -> float32 [T, hidden], the start of the residual stream;
-                   `table` is what a tied head shares
+  TokenEmbedding   forward(ids, ctx) -> float32 [T, hidden], the start of the residual stream
+                   (`ctx` for kinds that need positions or the request; the built-in one
+                   ignores it); `table` is what a tied head shares
   Head             forward(h) -> float32 logits [R, vocab]; load(..., shared=) takes the
                    embedding's table when the spec says `tied`
 
@@ -217,7 +218,7 @@ class PositionEncoding(Part):
 class TokenEmbedding(Part):
     table: Optional[torch.Tensor] = None
 
-    def forward(self, ids: torch.Tensor) -> torch.Tensor:
+    def forward(self, ids: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         raise NotImplementedError
 
 

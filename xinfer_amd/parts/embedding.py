@@ -14,7 +14,7 @@ import torch
 from .. import kernels
 from ..config.spec import PartSpec
 from ..weights.store import TensorDecl, WeightStore
-from .base import Head, TokenEmbedding, register_embedding, register_head
+from .base import Head, StepContext, TokenEmbedding, register_embedding, register_head
 from .linear import Linear
 
 
@@ -39,7 +39,7 @@ class Embedding(TokenEmbedding):
             t = t.to(self.dtype)
         self.table = t.contiguous()
 
-    def forward(self, ids: torch.Tensor) -> torch.Tensor:
+    def forward(self, ids: torch.Tensor, ctx: Optional[StepContext] = None) -> torch.Tensor:
         return kernels.embed(self.table, ids, scale=self.scale)
 
 

@@ -38,6 +38,8 @@ def write_random_model(model_dir: str, config: Union[Dict[str, Any], Any], seed:
     os.makedirs(model_dir, exist_ok=True)
     with open(os.path.join(model_dir, "config.json"), "w", encoding="utf-8") as f:
         json.dump(config.to_dict(), f, indent=1)
+    # the values are the same wherever they are made; the GPU, if there is one, makes large tables faster
+    device = "cuda" if torch.cuda.is_available() else "cpu"
     write_safetensors(os.path.join(model_dir, "model.safetensors"),
-                      ((name, store.get(name)) for name in store.names()))
+                      ((name, store.get(name, None, device).cpu()) for name in store.names()))
     return model_dir

@@ -155,9 +155,11 @@ class SafetensorsStore(WeightStore):
 
 
 class RandomStore(WeightStore):
-    """Seeded random weights: each tensor has its own generator, keyed by the seed and the
-    tensor's name, so a tensor's values do not depend on which others exist or on order.
-    Values are rounded to `dtype` (bfloat16 unless told otherwise), as a checkpoint's are."""
+    """Seeded random weights: element i of a tensor is a normal value made from (seed, the
+    tensor's name, i) alone (`counter_normal`), so a tensor's values do not depend on which
+    others exist, on order, or on the device they are made on: the GPU's kernel and the CPU's
+    numpy twin give the same bits.  Values are rounded to `dtype` (bfloat16 unless told
+    otherwise), as a checkpoint's are."""
 
     def __init__(self, decls: Iterable[TensorDecl], seed: int, linear_std: float = 0.02,
                  norm_std: float = 0.1, dtype: torch.dtype = torch.bfloat16):
@@ -179,31 +181,49 @@ class RandomStore(WeightStore):
     def shape(self, name: str) -> Tuple[int, ...]:
         return tuple(self._decls[name].shape)
 
-    def _tensor_seed(self, name: str) -> int:
+    def _tensor_key(self, name: str) -> int:
         h = hashlib.sha256(f"{self.seed}:{name}".encode("utf-8")).digest()
-        return int.from_bytes(h[:8], "little") & ((1 << 63) - 1)
+        return int.from_bytes(h[:8], "little")
 
     def _raw(self, name: str, device) -> torch.Tensor:
         d = self._decls[name]
         dev = torch.device(device)
-        g = torch.Generator(device=dev)
-        g.manual_seed(self._tensor_seed(name))
         if d.init == "zeros":
-            t = torch.zeros(d.shape, dtype=torch.float32, device=dev)
+            return torch.zeros(d.shape, dtype=self.dtype, device=dev)
+        if d.init == "norm":
+            scale, shift = self.norm_std, 1.0
+        elif d.init == "linear":
+            scale, shift = self.linear_std, 0.0
         else:
-            # generated in pieces so that a [151936, 4096] table needs no float32 twin
-            t = torch.empty(d.shape, dtype=self.dtype, device=dev)
-            flat = t.view(-1)
-            step = 1 << 26
-            for b in range(0, flat.numel(), step):
-                n = min(step, flat.numel() - b)
-                r = torch.randn(n, generator=g, dtype=torch.float32, device=dev)
-                if d.init == "norm":
-                    r.mul_(self.norm_std).add_(1.0)
-                elif d.init == "linear":
-                    r.mul_(self.linear_std)
-                else:
-                    raise ValueError(f"tensor {name!r}: unknown init {d.init!r}")
-                flat[b:b + n] = r.to(self.dtype)
+            raise ValueError(f"tensor {name!r}: unknown init {d.init!r}")
+        key = self._tensor_key(name)
+        t = torch.empty(d.shape, dtype=self.dtype, device=dev)
+        flat = t.view(-1)
+        n = flat.numel()
+        if dev.type == "cuda":
+            from .. import kernels
+            with torch.cuda.device(dev):
+                if self.dtype in (torch.float32, torch.bfloat16):
+                    kernels.counter_normal_(flat, key, scale, shift)
+                else:                # in pieces, so that a large table needs no float32 twin
+                    step = 1 << 26
+                    for b in range(0, n, step):
+                        piece = torch.empty((min(step, n - b),), dtype=torch.float32, device=dev)
+                        flat[b:b + piece.numel()] = kernels.counter_normal_(piece, key, scale, shift, first=b).to(self.dtype)
             return t
-        return t.to(self.dtype)
+        from .counter_normal import counter_normal
+        step = 1 << 20
+
+        def piece(b: int) -> None:
+            m = min(step, n - b)
+            flat[b:b + m] = torch.from_numpy(counter_normal(key, b, m, scale, shift)).to(self.dtype)
+
+        starts = range(0, n, step)
+        if len(starts) > 1:          # numpy works outside the interpreter's lock
+            from concurrent.futures import ThreadPoolExecutor
+            with ThreadPoolExecutor(min(8, len(starts))) as ex:
+                list(ex.map(piece, starts))
+        else:
+            for b in starts:
+                piece(b)
+        return t
