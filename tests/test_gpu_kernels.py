@@ -464,15 +464,17 @@ def test_linear_mid_gated_wide_tile(M, N, K, features):
             kernels.linear_mid_gated(_rand((65, K), torch.bfloat16, g).to(DEV), w.to(DEV), features=features)
 
 
-@pytest.mark.parametrize("M,N,K,slices", [(129, 4096, 4096, 4), (256, 4096, 12288, 8), (200, 1024, 3072, 2), (512, 4096, 12288, 8),
-                                          (1000, 5120, 17408, 2), (256, 7168, 5120, 4), (300, 4096, 4096, 1), (128, 4096, 12288, 1),
-                                          (256, 4096, 1024, 1), (1025, 4096, 12288, 1), (200, 1000, 2056, 1)])
-def test_library_split_slices_and_their_sum(M, N, K, slices):
-    """Narrow products of 129 to 1,024 rows go to the library as one batched product over slices of
-    K: the chosen number of slices, the dispatch (`linear_bf16` with `allow_split`), and the sum of
-    the partial sums against a float64 product."""
+@pytest.mark.parametrize("M,N,K,slices", [(129, 4096, 4096, 8), (256, 4096, 12288, 8), (200, 1024, 3072, 4), (512, 4096, 12288, 4),
+                                          (1000, 5120, 17408, 1), (256, 7168, 5120, 4), (300, 4096, 4096, 1), (128, 4096, 12288, 1),
+                                          (256, 4096, 1024, 2), (1025, 4096, 12288, 1), (200, 1000, 2056, 1), (130, 6144, 2560, 4),
+                                          (512, 2560, 9728, 4), (1024, 5120, 25600, 1), (256, 5120, 8192, 4), (256, 10240, 5120, 2)])
+def test_tile_split_plan_and_the_sum_of_its_slices(M, N, K, slices):
+    """Narrow products of 129 to 1,024 rows go to the many-row tiled kernel with K cut into slices:
+    the chosen number of slices, the dispatch (`linear_bf16` with `allow_split`), every slice
+    against a float64 product of its part of K, and the sum of the partial sums as the norm adds
+    them."""
     from xinfer_amd import kernels
-    assert kernels.library_split_slices(M, N, K) == slices
+    assert kernels.tile_split_plan(M, N, K)[0] == slices
     g = torch.Generator().manual_seed(41)
     x = _rand((M, K), torch.bfloat16, g)
     w = _rand((N, K), torch.bfloat16, g, scale=0.05)
@@ -480,10 +482,10 @@ def test_library_split_slices_and_their_sum(M, N, K, slices):
     y = kernels.linear_bf16(x.to(DEV), w.to(DEV), torch.bfloat16, allow_split=True)
     if slices > 1:
         assert y.shape == (slices, M, N) and y.dtype == torch.float32
-        # each slice is the product over its own part of K
         k0 = K // slices
-        part = x[:, k0:2 * k0].double() @ w[:, k0:2 * k0].double().T
-        assert (y[1].cpu().double() - part).abs().max() / part.abs().max() < 1e-5
+        for sl in range(slices):
+            part = x[:, sl * k0:(sl + 1) * k0].double() @ w[:, sl * k0:(sl + 1) * k0].double().T
+            assert (y[sl].cpu().double() - part).abs().max() / part.abs().max() < 1e-5, sl
         total = y.cpu().double().sum(0)
         assert (total - ref).abs().max() / ref.abs().max() < 1e-5
         # the norm adds them in order: the same as adding them here
@@ -497,13 +499,48 @@ def test_library_split_slices_and_their_sum(M, N, K, slices):
     elif y.dim() == 2:
         assert y.shape == (M, N) and y.dtype == torch.bfloat16
         assert (y.cpu().double() - ref).abs().max() / ref.abs().max() < _tol(torch.bfloat16)
-    else:       # the tiled kernel's own slices
+    else:       # the tiled kernel of few rows and its own slices
         assert (y.cpu().double().sum(0) - ref).abs().max() / ref.abs().max() < 1e-5
-    with pytest.raises(kernels.KernelError, match="slices"):
-        kernels.linear_library_split(x.to(DEV), w.to(DEV), 3 if K % 24 else 7)
-    if M > kernels.LIBRARY_SPLIT_MOST_ROWS:
-        with pytest.raises(kernels.KernelError, match="rows, at most"):
-            kernels.linear_library_split(x.to(DEV), w.to(DEV), 2)
+
+
+@pytest.mark.parametrize("shape", [0, 1, 2])
+@pytest.mark.parametrize("M,N,K,slices", [(2048, 4096, 4096, 1), (129, 1000, 192, 1), (130, 264, 128, 2), (300, 516, 640, 5),
+                                          (1, 4, 64, 1), (257, 260, 3072, 3), (1111, 2560, 9728, 2), (640, 5120, 1024, 4)])
+def test_linear_tile_every_shape(M, N, K, slices, shape):
+    """The many-row tiled product alone, in its three tile shapes: rows and features that are no
+    multiple of a tile (what a tile holds past the end is read from the last row and never
+    stored), one slice rounded to bfloat16, several as float32 partial sums; against float64.
+    A slice's sum does not depend on the tile shape: the shapes give the same bits."""
+    from xinfer_amd import kernels
+    g = torch.Generator().manual_seed(43)
+    x = _rand((M, K), torch.bfloat16, g)
+    w = _rand((N, K), torch.bfloat16, g, scale=0.05)
+    ref = x.double() @ w.double().T
+    y = kernels.linear_tile(x.to(DEV), w.to(DEV), slices, partial=True, shape=shape)
+    assert y.shape == (slices, M, N) and y.dtype == torch.float32
+    assert (y.cpu().double().sum(0) - ref).abs().max() / ref.abs().max() < 1e-5
+    assert torch.equal(y, kernels.linear_tile(x.to(DEV), w.to(DEV), slices, partial=True, shape=(shape + 1) % 3))
+    if slices == 1:
+        yb = kernels.linear_tile(x.to(DEV), w.to(DEV), shape=shape)
+        assert yb.shape == (M, N) and yb.dtype == torch.bfloat16
+        assert torch.equal(yb, y[0].to(torch.bfloat16))          # one rounding of the same float32 sum
+
+
+def test_linear_tile_refuses():
+    from xinfer_amd import kernels
+    x = torch.zeros((130, 192), dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros((64, 192), dtype=torch.bfloat16, device=DEV)
+    assert kernels.linear_tile_takes(130, 64, 192, 3) and not kernels.linear_tile_takes(130, 64, 192, 2)
+    with pytest.raises(kernels.KernelError, match="not taken"):
+        kernels.linear_tile(x, w, 2, partial=True)                               # slices of 96
+    with pytest.raises(kernels.KernelError, match="not taken"):
+        kernels.linear_tile(x, torch.zeros((66, 192), dtype=torch.bfloat16, device=DEV))      # N no multiple of 4
+    with pytest.raises(kernels.KernelError, match="not taken"):
+        kernels.linear_tile(x[:, :100].contiguous(), w[:, :100].contiguous())      # K no multiple of 64
+    with pytest.raises(kernels.KernelError, match="bfloat16"):
+        kernels.linear_tile(x.float(), w.float())
+    with pytest.raises(kernels.KernelError, match="shape"):
+        kernels.linear_tile(x, w, shape=3)
 
 
 def test_linear_skinny_plan_fills_the_compute_units():

@@ -687,53 +687,64 @@ def linear_mid(x: torch.Tensor, w: torch.Tensor, depth: int = 0) -> torch.Tensor
     return y
 
 
-LIBRARY_SPLIT_ROWS = 1024     # most rows of a product that is cut along K into one batched library product
-LIBRARY_SPLIT_K = 1024        # least K of a slice up to 512 rows; twice that beyond
-LIBRARY_SPLIT_MOST_ROWS = 1024    # what `linear_library_split` takes at all
+TILE_SPLIT_ROWS = 1024        # most rows of a product that the many-row tiled kernel takes with K cut into slices
+TILE_SPLIT_K = 512            # least K of a slice
 
 
-def library_split_slices(M: int, N: int, K: int) -> int:
-    """Slices of K into which x [M, K] @ w [N, K]^T is cut for the library, 1 = not at all.  A
-    narrow output gives the library too few tiles for the chip's 256 compute units (256 rows by
-    4096 columns: 16 tiles of 256 x 256), and its own choice of kernel does not split K: slices
-    as one batched product, with float32 partial sums [slices, M, N] for the caller to add in
-    order, put more of the chip to work.  As many slices (a power of two) as keep the tiles x
-    slices within the compute units and a slice's K long enough to pay for its start.  Beyond
-    256 rows only for K >= 2 N (the down projection): the reader of the partial sums then reads
-    `slices` float32 values for every one it would read in bfloat16, which a smaller gain does
-    not pay for.  Measured on MI355X at Qwen3-8B sizes (qkv / o / down, us): 256 rows 36 / 19 / 49
-    in one library product and 36 / 27 / 55 in the tiled kernel against 22 / 18 / 35 so; down at
-    512 and 1,024 rows 80 -> 54 and 119 -> 87; at Qwen3-14B sizes and 256 rows 48 / 44 / 227
-    (tiled: 46 / 37 / 97) -> 29 / 23 / 54.  Up to 128 rows the tiled kernel is level or ahead."""
-    if not (MID_BLOCK < M <= min(LIBRARY_SPLIT_ROWS, LIBRARY_SPLIT_MOST_ROWS)) or (M > MID_ROWS and K < 2 * N):
-        return 1
-    tiles = -(-M // 256) * -(-N // 256)
-    most = min(COMPUTE_UNITS // tiles, K // (LIBRARY_SPLIT_K if M <= 512 else 2 * LIBRARY_SPLIT_K))
+def tile_split_plan(M: int, N: int, K: int):
+    """(slices, tile shape) of x [M, K] @ w [N, K]^T in the many-row tiled kernel (`linear_tile`) for a
+    narrow output at 129 to 1,024 rows, slices 1 = it is not used.  A narrow output gives too few
+    tiles for the chip's 256 compute units (256 rows by 4,096 features: 32 tiles of 256 x 128), so K
+    is cut into slices, each a workgroup's own, with float32 partial sums [slices, M, N] for the
+    caller to add in order: as many slices (a power of two) as keep tiles x slices within the
+    compute units and a slice at least 512 long.  The tile shape is the one that makes fewer
+    tiles: 256 rows by 128 features up to 256 rows (every row of w is read by one workgroup),
+    128 by 256 beyond.  Beyond 256 rows only for K >= 2 N (the down projection): the reader of the
+    partial sums reads `slices` float32 values for every bfloat16 one, which a smaller gain does
+    not pay for.  Measured on MI355X at Qwen3-8B sizes (qkv / o / down, us): 256 rows 36 / 20 / 44
+    in one library product against 23 / 17 / 31 so; down at 512 rows 70 -> 52; at 1,024 rows level
+    (103 -> 100).  Up to 128 rows the tiled kernel of few rows (`linear_mid`) is level or ahead."""
+    if not (MID_BLOCK < M <= TILE_SPLIT_ROWS) or (M > MID_ROWS and K < 2 * N) or N % 4 or K % 64:
+        return 1, 0
+    tall, wide = -(-M // 256) * -(-N // 128), -(-M // 128) * -(-N // 256)
+    shape = 1 if (tall < wide or (tall == wide and M <= 256)) else 0
+    tiles = tall if shape == 1 else wide
+    most = min(COMPUTE_UNITS // tiles, K // TILE_SPLIT_K)
     slices = 1
     while slices * 2 <= most and K % (slices * 2 * 64) == 0:
         slices *= 2
-    return slices
+    return slices, shape
 
 
-def linear_library_split(x: torch.Tensor, w: torch.Tensor, slices: int) -> torch.Tensor:
-    """bfloat16 x [M, K] @ w [N, K]^T as float32 partial sums [slices, M, N] over `slices` equal
-    parts of K, one batched library product over views of x and w (nothing is copied)."""
+def linear_tile_takes(M: int, N: int, K: int, slices: int = 1) -> bool:
+    """Whether the many-row tiled product takes a shape: K in whole tiles of 64 a slice, N in fours."""
+    return bool(lib().xi_linear_tile_takes(int(M), int(N), int(K), int(slices)))
+
+
+def linear_tile(x: torch.Tensor, w: torch.Tensor, slices: int = 1, partial: bool = False,
+                shape: Optional[int] = None) -> torch.Tensor:
+    """bfloat16 x [M, K] @ w [N, K]^T on the matrix cores for many rows: bfloat16 [M, N], or with
+    `partial` (needed for more than one slice) float32 partial sums [slices, M, N] over equal
+    slices of K.  `shape` 0: workgroup tiles of 128 rows by 256 features, 1: 256 by 128; None: the
+    one that makes fewer tiles (128 by 256 at equal numbers)."""
     _dev(x, w)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
-        raise KernelError("linear_library_split: operands must be bfloat16")
+        raise KernelError("linear_tile: operands must be bfloat16")
     if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
-        raise KernelError(f"linear_library_split: x {tuple(x.shape)} and w {tuple(w.shape)} do not match")
+        raise KernelError(f"linear_tile: x {tuple(x.shape)} and w {tuple(w.shape)} do not match")
     M, K = x.shape
     N = w.shape[0]
-    if slices < 1 or K % (slices * 8):
-        raise KernelError(f"linear_library_split: K={K} is not {slices} slices of a multiple of 8")
-    if not (0 < M <= LIBRARY_SPLIT_MOST_ROWS):
-        # (torch.bmm of bfloat16 [2, 2048, 6144] by [2, 6144, 4096] with a bfloat16 result ended in a GPU memory
-        # fault inside the library; only the form with a float32 result is used, at the sizes it has been run at)
-        raise KernelError(f"linear_library_split: {M} rows, at most {LIBRARY_SPLIT_MOST_ROWS}")
-    xs = x.view(M, slices, K // slices).transpose(0, 1)            # [slices, M, K / slices]
-    ws = w.view(N, slices, K // slices).permute(1, 2, 0)            # [slices, K / slices, N]
-    return torch.bmm(xs, ws, out_dtype=torch.float32)
+    partial = bool(partial) or slices > 1
+    if not linear_tile_takes(M, N, K, slices):
+        raise KernelError(f"linear_tile: M={M} N={N} K={K} in {slices} slices is not taken")
+    if shape is None:
+        shape = 1 if -(-M // 256) * -(-N // 128) < -(-M // 128) * -(-N // 256) else 0
+    if partial:
+        y = torch.empty((slices, M, N), dtype=torch.float32, device=x.device)
+    else:
+        y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+    _ok(lib().xi_linear_tile(_p(x), _p(w), _p(y), M, N, K, int(slices), int(partial), int(shape), _stream()))
+    return y
 
 
 MID_GATED_ROWS = 128      # most rows of the gated form of the tiled product
@@ -932,10 +943,10 @@ def linear_bf16(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtyp
     if out_dtype == torch.float32 and MID_WIDE_FROM <= x.shape[0] <= MID_GATED_ROWS \
             and linear_mid_slices(w.shape[0], w.shape[1]) == 1:
         return linear_mid(x, w)[0]           # a wide output in float32 (the head): one slice is the result
-    if allow_split and MID_BLOCK < x.shape[0] <= LIBRARY_SPLIT_ROWS:
-        slices = library_split_slices(x.shape[0], w.shape[0], w.shape[1])
+    if allow_split and MID_BLOCK < x.shape[0] <= TILE_SPLIT_ROWS:
+        slices, shape = tile_split_plan(x.shape[0], w.shape[0], w.shape[1])
         if slices > 1:
-            return linear_library_split(x, w, slices)
+            return linear_tile(x, w, slices, partial=True, shape=shape)
     if allow_split and MID_FROM <= x.shape[0] <= MID_ROWS and linear_mid_slices(w.shape[0], w.shape[1]) > 0 \
             and w.shape[0] <= MID_WIDEST and (x.shape[0] <= MID_BLOCK or w.numel() * 2 >= MID_TWO_BLOCKS):
         return linear_mid(x, w)

@@ -6,8 +6,8 @@ BLAS (/root/reference/src/models/layers/linear.rs:76-124).  Here:
              an output element does not depend on the batch it was computed in;
   bfloat16 : the hand-written kernels for few rows (decode), the vendor library
              (hipBLASLt through torch) for many rows, as the reference uses a library;
-             narrow outputs at 129 to 1,024 rows as one batched library product over slices
-             of K where the caller takes partial sums (`kernels.library_split_slices`).
+             narrow outputs at 129 to 1,024 rows in the hand-written many-row tiled kernel over
+             slices of K where the caller takes partial sums (`kernels.tile_split_plan`).
 A weight that the checkpoint stores in 32 bits stays in 32 bits; activations are then
 widened for this product.
 """
