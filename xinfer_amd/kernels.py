@@ -689,6 +689,10 @@ def linear_mid(x: torch.Tensor, w: torch.Tensor, depth: int = 0) -> torch.Tensor
 
 TILE_SPLIT_ROWS = 1024        # most rows of a product that the many-row tiled kernel takes with K cut into slices
 TILE_SPLIT_K = 512            # least K of a slice
+TILE_SPLIT_BYTES = 8 << 20    # a weight up to this size is left to the library (level there, measured at Qwen3-0.6B sizes)
+TILE_SHAPES = ((128, 256), (256, 128), (256, 256))     # rows of x by rows of w a workgroup, by `shape` of `linear_tile`
+TILE_FILL_RATE = 58e9         # bytes a second that one compute unit's loads bring into its LDS
+TILE_STREAM_RATE = 5e12       # bytes a second that the chip streams from memory
 
 
 def tile_split_plan(M: int, N: int, K: int):
@@ -696,24 +700,33 @@ def tile_split_plan(M: int, N: int, K: int):
     narrow output at 129 to 1,024 rows, slices 1 = it is not used.  A narrow output gives too few
     tiles for the chip's 256 compute units (256 rows by 4,096 features: 32 tiles of 256 x 128), so K
     is cut into slices, each a workgroup's own, with float32 partial sums [slices, M, N] for the
-    caller to add in order: as many slices (a power of two) as keep tiles x slices within the
-    compute units and a slice at least 512 long.  The tile shape is the one that makes fewer
-    tiles: 256 rows by 128 features up to 256 rows (every row of w is read by one workgroup),
-    128 by 256 beyond.  Beyond 256 rows only for K >= 2 N (the down projection): the reader of the
-    partial sums reads `slices` float32 values for every bfloat16 one, which a smaller gain does
-    not pay for.  Measured on MI355X at Qwen3-8B sizes (qkv / o / down, us): 256 rows 36 / 20 / 44
-    in one library product against 23 / 17 / 31 so; down at 512 rows 70 -> 52; at 1,024 rows level
-    (103 -> 100).  Up to 128 rows the tiled kernel of few rows (`linear_mid`) is level or ahead."""
-    if not (MID_BLOCK < M <= TILE_SPLIT_ROWS) or (M > MID_ROWS and K < 2 * N) or N % 4 or K % 64:
+    caller to add in order.  Slices (a power of two, a slice at least 512 long) and tile shape are
+    those with the least cost in a model of two terms that fits what was measured on MI355X within a
+    tenth: a workgroup brings (rows of x + rows of w of its tile) x its slice of K into LDS at 58 GB/s
+    (that, not the matrix cores, bounds these shapes: x is fetched again by every workgroup, so
+    tiles with as many rows of w as of x are ahead where x is a whole tile's rows), rounds of 256
+    workgroups one after the other, never faster than the weight streams from memory; and the
+    partial sums are written and read again, 8 bytes an element and slice.  256 rows of N = 5120,
+    K = 17408: 4 slices of 256 x 128 tiles 71 us, 8 slices of 256 x 256 tiles 55.  Beyond 256 rows
+    only for K >= 2 N (the down projection): the reader of the partial sums reads `slices` float32
+    values for every bfloat16 one, which a smaller gain does not pay for.  Up to 128 rows the tiled
+    kernel of few rows (`linear_mid`) is level or ahead."""
+    if not (MID_BLOCK < M <= TILE_SPLIT_ROWS) or (M > MID_ROWS and K < 2 * N) or N % 4 or K % 64 \
+            or N * K * 2 <= TILE_SPLIT_BYTES:
         return 1, 0
-    tall, wide = -(-M // 256) * -(-N // 128), -(-M // 128) * -(-N // 256)
-    shape = 1 if (tall < wide or (tall == wide and M <= 256)) else 0
-    tiles = tall if shape == 1 else wide
-    most = min(COMPUTE_UNITS // tiles, K // TILE_SPLIT_K)
-    slices = 1
-    while slices * 2 <= most and K % (slices * 2 * 64) == 0:
-        slices *= 2
-    return slices, shape
+    best = None
+    for shape in ((1, 0, 2) if M <= 256 else (0, 1, 2)):      # (among equals: every row of w in one workgroup)
+        bm, bn = TILE_SHAPES[shape]
+        tiles = -(-M // bm) * -(-N // bn)
+        slices = 2
+        while slices <= 16 and K % (slices * 64) == 0 and K // slices >= TILE_SPLIT_K:
+            rounds = -(-tiles * slices // COMPUTE_UNITS)
+            fill = rounds * (bm + bn) * (K // slices) * 2 / TILE_FILL_RATE
+            cost = max(fill, N * K * 2 / TILE_STREAM_RATE) + slices * M * N * 8 / TILE_STREAM_RATE
+            if best is None or cost < best[0] - 1e-9:
+                best = (cost, slices, shape)
+            slices *= 2
+    return (best[1], best[2]) if best is not None else (1, 0)
 
 
 def linear_tile_takes(M: int, N: int, K: int, slices: int = 1) -> bool:
@@ -726,7 +739,7 @@ def linear_tile(x: torch.Tensor, w: torch.Tensor, slices: int = 1, partial: bool
     """bfloat16 x [M, K] @ w [N, K]^T on the matrix cores for many rows: bfloat16 [M, N], or with
     `partial` (needed for more than one slice) float32 partial sums [slices, M, N] over equal
     slices of K.  `shape` 0: workgroup tiles of 128 rows by 256 features, 1: 256 by 128; None: the
-    one that makes fewer tiles (128 by 256 at equal numbers)."""
+    one that makes fewer tiles (128 by 256 at equal numbers); 2: 256 by 256."""
     _dev(x, w)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError("linear_tile: operands must be bfloat16")
