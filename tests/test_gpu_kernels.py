@@ -464,10 +464,7 @@ def test_linear_mid_gated_wide_tile(M, N, K, features):
             kernels.linear_mid_gated(_rand((65, K), torch.bfloat16, g).to(DEV), w.to(DEV), features=features)
 
 
-@pytest.mark.parametrize("M,N,K,slices", [(129, 4096, 4096, 8), (256, 4096, 12288, 8), (200, 1024, 3072, 1), (512, 4096, 12288, 8),
-                                          (1000, 5120, 17408, 2), (256, 7168, 5120, 4), (300, 4096, 4096, 1), (128, 4096, 12288, 1),
-                                          (256, 4096, 1024, 1), (1025, 4096, 12288, 1), (200, 1000, 2056, 1), (130, 6144, 2560, 4),
-                                          (512, 2560, 9728, 8), (1024, 5120, 25600, 8), (256, 5120, 8192, 8), (256, 10240, 5120, 4)])
+@pytest.mark.parametrize("M,N,K,slices", [(129, 4096, 4096, 8), (256, 4096, 12288, 8), (200, 1024, 3072, 1), (512, 4096, 12288, 8), (1000, 5120, 17408, 3), (256, 7168, 5120, 4), (300, 4096, 4096, 1), (128, 4096, 12288, 1), (256, 4096, 1024, 1), (1025, 4096, 12288, 1), (200, 1000, 2056, 1), (130, 6144, 2560, 5), (512, 2560, 9728, 6), (1024, 5120, 25600, 3), (256, 5120, 8192, 6), (256, 10240, 5120, 3)])
 def test_tile_split_plan_and_the_sum_of_its_slices(M, N, K, slices):
     """Narrow products of 129 to 1,024 rows go to the many-row tiled kernel with K cut into slices:
     the chosen number of slices, the dispatch (`linear_bf16` with `allow_split`), every slice
@@ -482,9 +479,9 @@ def test_tile_split_plan_and_the_sum_of_its_slices(M, N, K, slices):
     y = kernels.linear_bf16(x.to(DEV), w.to(DEV), torch.bfloat16, allow_split=True)
     if slices > 1:
         assert y.shape == (slices, M, N) and y.dtype == torch.float32
-        k0 = K // slices
-        for sl in range(slices):
-            part = x[:, sl * k0:(sl + 1) * k0].double() @ w[:, sl * k0:(sl + 1) * k0].double().T
+        for sl in range(slices):            # slice sl: the tiles of 64 k from sl * tiles / slices up to (sl + 1) * tiles / slices
+            lo, hi = 64 * (sl * (K // 64) // slices), 64 * ((sl + 1) * (K // 64) // slices)
+            part = x[:, lo:hi].double() @ w[:, lo:hi].double().T
             assert (y[sl].cpu().double() - part).abs().max() / part.abs().max() < 1e-5, sl
         total = y.cpu().double().sum(0)
         assert (total - ref).abs().max() / ref.abs().max() < 1e-5
@@ -505,7 +502,8 @@ def test_tile_split_plan_and_the_sum_of_its_slices(M, N, K, slices):
 
 @pytest.mark.parametrize("shape", [0, 1, 2])
 @pytest.mark.parametrize("M,N,K,slices", [(2048, 4096, 4096, 1), (129, 1000, 192, 1), (130, 264, 128, 2), (300, 516, 640, 5),
-                                          (1, 4, 64, 1), (257, 260, 3072, 3), (1111, 2560, 9728, 2), (640, 5120, 1024, 4)])
+                                          (1, 4, 64, 1), (257, 260, 3072, 3), (1111, 2560, 9728, 2), (640, 5120, 1024, 4),
+                                          (200, 132, 704, 3), (140, 256, 448, 7), (256, 5120, 17408, 6)])
 def test_linear_tile_every_shape(M, N, K, slices, shape):
     """The many-row tiled product alone, in its three tile shapes: rows and features that are no
     multiple of a tile (what a tile holds past the end is read from the last row and never
@@ -530,9 +528,10 @@ def test_linear_tile_refuses():
     from xinfer_amd import kernels
     x = torch.zeros((130, 192), dtype=torch.bfloat16, device=DEV)
     w = torch.zeros((64, 192), dtype=torch.bfloat16, device=DEV)
-    assert kernels.linear_tile_takes(130, 64, 192, 3) and not kernels.linear_tile_takes(130, 64, 192, 2)
+    assert kernels.linear_tile_takes(130, 64, 192, 3) and kernels.linear_tile_takes(130, 64, 192, 2)
+    assert not kernels.linear_tile_takes(130, 64, 192, 4)
     with pytest.raises(kernels.KernelError, match="not taken"):
-        kernels.linear_tile(x, w, 2, partial=True)                               # slices of 96
+        kernels.linear_tile(x, w, 4, partial=True)                               # more slices than tiles of 64
     with pytest.raises(kernels.KernelError, match="not taken"):
         kernels.linear_tile(x, torch.zeros((66, 192), dtype=torch.bfloat16, device=DEV))      # N no multiple of 4
     with pytest.raises(kernels.KernelError, match="not taken"):

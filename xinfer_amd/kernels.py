@@ -700,7 +700,7 @@ def tile_split_plan(M: int, N: int, K: int):
     narrow output at 129 to 1,024 rows, slices 1 = it is not used.  A narrow output gives too few
     tiles for the chip's 256 compute units (256 rows by 4,096 features: 32 tiles of 256 x 128), so K
     is cut into slices, each a workgroup's own, with float32 partial sums [slices, M, N] for the
-    caller to add in order.  Slices (a power of two, a slice at least 512 long) and tile shape are
+    caller to add in order.  Slices (2 to 16, whole tiles of 64 k, a slice at least 512 long) and tile shape are
     those with the least cost in a model of two terms that fits what was measured on MI355X within a
     tenth: a workgroup brings (rows of x + rows of w of its tile) x its slice of K into LDS at 58 GB/s
     (that, not the matrix cores, bounds these shapes: x is fetched again by every workgroup, so
@@ -715,30 +715,32 @@ def tile_split_plan(M: int, N: int, K: int):
             or N * K * 2 <= TILE_SPLIT_BYTES:
         return 1, 0
     best = None
+    k_tiles = K // 64
     for shape in ((1, 0, 2) if M <= 256 else (0, 1, 2)):      # (among equals: every row of w in one workgroup)
         bm, bn = TILE_SHAPES[shape]
         tiles = -(-M // bm) * -(-N // bn)
-        slices = 2
-        while slices <= 16 and K % (slices * 64) == 0 and K // slices >= TILE_SPLIT_K:
+        for slices in range(2, 17):
+            longest = -(-k_tiles // slices) * 64               # the slices differ by a tile at most
+            if longest < TILE_SPLIT_K:
+                break
             rounds = -(-tiles * slices // COMPUTE_UNITS)
-            fill = rounds * (bm + bn) * (K // slices) * 2 / TILE_FILL_RATE
+            fill = rounds * (bm + bn) * longest * 2 / TILE_FILL_RATE
             cost = max(fill, N * K * 2 / TILE_STREAM_RATE) + slices * M * N * 8 / TILE_STREAM_RATE
             if best is None or cost < best[0] - 1e-9:
                 best = (cost, slices, shape)
-            slices *= 2
     return (best[1], best[2]) if best is not None else (1, 0)
 
 
 def linear_tile_takes(M: int, N: int, K: int, slices: int = 1) -> bool:
-    """Whether the many-row tiled product takes a shape: K in whole tiles of 64 a slice, N in fours."""
+    """Whether the many-row tiled product takes a shape: K in whole tiles of 64, a tile a slice at least, N in fours."""
     return bool(lib().xi_linear_tile_takes(int(M), int(N), int(K), int(slices)))
 
 
 def linear_tile(x: torch.Tensor, w: torch.Tensor, slices: int = 1, partial: bool = False,
                 shape: Optional[int] = None) -> torch.Tensor:
     """bfloat16 x [M, K] @ w [N, K]^T on the matrix cores for many rows: bfloat16 [M, N], or with
-    `partial` (needed for more than one slice) float32 partial sums [slices, M, N] over equal
-    slices of K.  `shape` 0: workgroup tiles of 128 rows by 256 features, 1: 256 by 128; None: the
+    `partial` (needed for more than one slice) float32 partial sums [slices, M, N] over slices of K
+    (whole tiles of 64, equal but for one tile).  `shape` 0: workgroup tiles of 128 rows by 256 features, 1: 256 by 128; None: the
     one that makes fewer tiles (128 by 256 at equal numbers); 2: 256 by 256."""
     _dev(x, w)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
