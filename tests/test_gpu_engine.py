@@ -304,6 +304,24 @@ def test_eos_ids_of_config_and_generation_config_both_stop(model_dirs, tmp_path)
     assert _engine(str(d), "A", "f32", max_num_seqs=2, num_pages=16).eos_token_ids == {a, b}
 
 
+def test_engine_plans_pages_group_by_group(model_dirs):
+    """Left to plan its cache itself, the engine gives tiny W's layers with a window of 24 pages for a
+    window and a portion a request, its layer that keeps every key pages for the model's length,
+    and generates the plain model's greedy tokens on that: with two long requests the window
+    group's pages are used again and again."""
+    from xinfer_amd import SamplingParams
+    eng = _engine(model_dirs["W"], "W", "f32", max_num_seqs=2, max_model_len=320, prefill_chunk_size=32)
+    assert [g.window for g in eng.model.cache_groups] == [24, 0]
+    assert [g.num_pages for g in eng.runner.cache.groups] == [2 * (-(-(24 - 1 + 32) // 16) + 1), 2 * (320 // 16)]
+    rng = random.Random(17)
+    prompts = [harness.random_prompt(rng, n, 300) for n in (250, 301)]
+    outs = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))
+    pm = plain.PlainModel(model_dirs["W"])
+    for p, o in zip(prompts, outs):
+        assert o.token_ids == pm.greedy(p, 12)
+    assert eng.num_preemptions == 0 and eng.runner.cache.live_requests() == 0
+
+
 # ---- streaming -----------------------------------------------------------------------------------
 def test_streams_interleave_and_cancel(model_dirs):
     """Two streams read in turn give the tokens `generate` gives; a cancelled stream gives its

@@ -254,3 +254,36 @@ def test_running_one_step_ahead_keeps_the_books(seed):
     for g, grp in enumerate(cm.groups):
         assert cm.free_pages(g) == grp.num_pages
     assert wasted <= sum(1 for rid in reqs if ends_at[rid] is not None)
+
+
+def test_pages_are_planned_group_by_group():
+    """A group with a window gets pages for a window and a portion a request (what the scheduler
+    admits it with), not for the model's whole length; if memory is short every group keeps the
+    same share of what it could use; and the scheduler admits a full house on what was planned."""
+    from xinfer_amd.engine.llm_engine import plan_pages
+    page, seqs, length, portion = 16, 4, 4096, 64
+    full, windowed = (0, 1000), (24, 500)
+    got = plan_pages([full, windowed], page, seqs, length, portion, budget_bytes=1 << 40)
+    assert got == [seqs * (length // page), seqs * (-(-(24 - 1 + portion) // page) + 1)] == [1024, 28]
+    # a window longer than the model's length changes nothing
+    assert plan_pages([(10 ** 6, 500)], page, seqs, length, portion, 1 << 40) == [1024]
+    # short of memory: the same share of both, within a page
+    need = 1024 * 1000 * page + 28 * 500 * page
+    half = plan_pages([full, windowed], page, seqs, length, portion, need // 2)
+    assert half == [512, 14]
+    assert plan_pages([full, windowed], page, seqs, length, portion, 1) == [1, 1]
+    assert plan_pages([], page, seqs, length, portion, 1 << 40) == [1]
+    # what was planned is what the scheduler needs for max_num_seqs requests of the full length:
+    # all are admitted together and nothing is ever preempted
+    cm = PagedCacheManager([CacheGroup(page, got[0]), CacheGroup(page, got[1], window=24)], max_requests=seqs)
+    s = Scheduler(cm, seqs, seqs * portion, portion)       # a step's budget takes a portion of every request
+    for rid in range(seqs):
+        s.add(rid, length - 8, 8)
+    most = [0]
+
+    def on_step(plan):
+        most[0] = max(most[0], cm.live_requests())
+
+    seen, _ = drive(s, cm, {rid: (length - 8, 8) for rid in range(seqs)}, on_step=on_step)
+    assert most[0] == seqs and not any("preempted" in v for v in seen.values())
+    assert cm.free_pages(0) == got[0] and cm.free_pages(1) == got[1]

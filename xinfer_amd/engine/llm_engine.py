@@ -12,7 +12,7 @@ from __future__ import annotations
 import os
 import time
 from dataclasses import dataclass, field
-from typing import Dict, List, Optional, Sequence, Union
+from typing import Dict, List, Optional, Sequence, Tuple, Union
 
 import torch
 
@@ -66,6 +66,31 @@ class _Launched:
     host: torch.Tensor                 # the same in pinned memory once `ready` has happened
     ready: torch.cuda.Event
     row_of: Dict[int, int]             # request id -> its row
+
+
+def plan_pages(groups: Sequence[Tuple[int, int]], page: int, max_num_seqs: int, max_model_len: int, portion: int,
+               budget_bytes: int) -> List[int]:
+    """Pages for every cache group.  `groups`: per group (window, bytes a token over the group's
+    layers).  A group that keeps every key can use `max_num_seqs` requests of `max_model_len`
+    tokens; a group with a window holds of a request the window - 1 keys before the portion that
+    runs, the portion itself and one page more (they need not start at a page's edge), as the
+    scheduler admits it: a model with a small window over a long context gets a small pool for
+    those layers, not the context's.  If that is more than `budget_bytes`, every group gets the
+    same share of what it could use (one page at least)."""
+    could, size = [], []
+    for window, per_token in groups:
+        tokens = max_model_len
+        pages = -(-tokens // page)
+        if window > 0:
+            pages = min(pages, -(-min(tokens, window - 1 + portion) // page) + 1)
+        could.append(max_num_seqs * pages)
+        size.append(max(1, per_token * page))
+    if not could:
+        return [1]
+    need = sum(c * b for c, b in zip(could, size))
+    if need <= budget_bytes:
+        return [max(1, c) for c in could]
+    return [max(1, int(c * budget_bytes / need)) for c in could]
 
 
 class LLMEngine:
@@ -123,19 +148,20 @@ class LLMEngine:
         self._pin_turn = 0
 
     # ---- memory -------------------------------------------------------------------
-    def _plan_pages(self, page: int) -> int:
-        """Pages per group from a share of the memory that is free after loading the
+    def _plan_pages(self, page: int) -> List[int]:
+        """Pages of every cache group from a share of the memory that is free after loading the
         weights (the reference's kv_fraction, 0.6 by default on GPUs,
-        /root/reference/src/utils/kvcache_allocator.rs:336-346), capped by what
-        max_num_seqs requests of max_model_len tokens can use."""
+        /root/reference/src/utils/kvcache_allocator.rs:336-346); see `plan_pages`."""
         free, _ = torch.cuda.mem_get_info(self.model.device)
         frac = self.econfig.kv_fraction if self.econfig.kv_fraction is not None else 0.6
         esize = torch.tensor([], dtype=self.dtype).element_size()
-        per_token = sum(pool.bytes_per_token(esize) for kv in self.model.kv_needs.values() for pool in kv.pools)
-        per_page = max(1, per_token * page)
-        by_memory = int(free * frac) // per_page
-        by_use = self.econfig.max_num_seqs * (-(-self.max_model_len // page))
-        return max(1, min(by_memory, by_use))
+        groups = []
+        for grp in self.model.cache_groups:
+            per_token = sum(pool.bytes_per_token(esize) for layer in grp.layers for pool in self.model.kv_needs[layer].pools)
+            groups.append((grp.window, per_token))
+        portion = min(self.econfig.prefill_chunk_size,
+                      self.econfig.max_num_batched_tokens or max(self.econfig.prefill_chunk_size, self.econfig.max_num_seqs))
+        return plan_pages(groups, page, self.econfig.max_num_seqs, self.max_model_len, portion, int(free * frac))
 
     def get_num_cached_tokens(self) -> int:
         """Tokens held by the prefix cache (xinfer.pyi:215-222): there is none here, so none."""
