@@ -6,7 +6,10 @@
 Prints ONE JSON line.  `value` is decoded tokens per second at batch 8 and the context
 length the configuration names (the last timed step ends at that length); a "step" is one
 decode step through the engine's own step function (mixed-batch path, paged cache,
-kernels) followed by greedy sampling on the GPU.  Beside it: the prefill of one
+kernels) followed by greedy sampling on the GPU, launched as the engine launches its steps:
+the sampled ids reach the next step on the device and travel to the host beside it, so the
+host prepares a step while the GPU runs the one before (the timed steps lie between two
+synchronizations, and all of their tokens have reached the host at the second).  Beside it: the prefill of one
 2,048-token prompt, the decode step's bandwidth roofline, decode at batch 1 and 64 (`points`,
 and each one's own roofline in `points_roofline`), and decode at batch 8 with four times the
 context (`further`).
@@ -264,19 +267,34 @@ def main() -> int:
             runner.cache.reserve(rid, start)
             runner.cache.commit(rid, start)
         toks = torch.randint(0, cfg.vocab_size, (batch,), generator=cpu_gen).tolist()
+        places = list(range(batch))
+        pins = [torch.empty((batch,), dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        state = {"turn": 0}
 
-        def one(toks):
-            logits = runner.step([StepEntry(r, [t], [0]) for r, t in zip(rids, toks)])
-            return sampler.argmax(logits).tolist()
+        def one(prev):
+            """One decode step as the engine launches it (`LLMEngine.step` with its default
+            `run_ahead`): the tokens that the step before sampled are handed over on the device,
+            greedy sampling follows on the GPU, and the sampled ids start their way to the host
+            without anything waiting for them; the host prepares the next step meanwhile."""
+            if prev is None:
+                logits = runner.step([StepEntry(r, [t], [0]) for r, t in zip(rids, toks)])
+            else:
+                logits = runner.step([StepEntry(r, [0], [0]) for r in rids], device_tokens=(prev, places, places))
+            tok = sampler.argmax(logits)
+            pins[state["turn"]].copy_(tok, non_blocking=True)
+            state["turn"] ^= 1
+            return tok
 
+        prev = None
         for _ in range(prep + warmup):
-            toks = one(toks)
+            prev = one(prev)
         sync()
         t = time.perf_counter()
         for _ in range(steps):
-            toks = one(toks)
+            prev = one(prev)
         sync()
         dt = time.perf_counter() - t
+        assert 0 <= int(prev.min()) and int(prev.max()) < cfg.vocab_size
         for rid in rids:
             runner.release(rid)
         return dt / steps

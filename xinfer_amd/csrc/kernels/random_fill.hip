@@ -2,10 +2,10 @@
 // is the same whoever makes it, in whatever pieces, on the GPU (here) or on the CPU
 // (weights/counter_normal.py, the same operations on numpy arrays).
 //
-//   z      = splitmix64's (i + 1)-th output from state `key`
-//   u1     = ((z >> 40) + 1) / 2^24 in (0, 1],  u2 = ((z >> 8) & 0xFFFFFF) / 2^24 in [0, 1)
-//   normal = sqrt(-2 ln u1) * cos(2 pi u2)                                  (Box-Muller)
-//   value  = normal * scale + shift, rounded once to the output type
+//   z       = splitmix64's (i / 2 + 1)-th output from state `key`: one draw for elements 2p and 2p + 1
+//   u1      = ((z >> 40) + 1) / 2^24 in (0, 1],  u2 = ((z >> 8) & 0xFFFFFF) / 2^24 in [0, 1)
+//   normals = sqrt(-2 ln u1) * cos(2 pi u2) for the even element, * sin(2 pi u2) for the odd one   (Box-Muller)
+//   value   = normal * scale + shift, rounded once to the output type
 //
 // ln and cos are polynomials of float32 additions, multiplications, one division and one square
 // root, each rounded on its own (no fused multiply-add: `fp contract(off)`), in one fixed order:
@@ -14,9 +14,10 @@
 
 namespace xi {
 
-__device__ __forceinline__ float counter_normal(uint64_t key, uint64_t i) {
+// the two normal values of pair p (elements 2p and 2p + 1)
+__device__ __forceinline__ void counter_normal_pair(uint64_t key, uint64_t pair, float& even, float& odd) {
 #pragma clang fp contract(off)
-  uint64_t z = key + (i + 1) * 0x9E3779B97F4A7C15ull;
+  uint64_t z = key + (pair + 1) * 0x9E3779B97F4A7C15ull;
   z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
   z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
   z = z ^ (z >> 31);
@@ -57,16 +58,23 @@ __device__ __forceinline__ float counter_normal(uint64_t key, uint64_t i) {
   cs = cs * t2 + -0.5f;
   cs = cs * t2 + 1.0f;
   const float c = quarter == 0 ? cs : quarter == 1 ? -sn : quarter == 2 ? -cs : sn;
-  return radius * c;
+  const float sv = quarter == 0 ? sn : quarter == 1 ? cs : quarter == 2 ? -sn : -cs;
+  even = radius * c;
+  odd = radius * sv;
 }
 
 template <typename T>
 __global__ void __launch_bounds__(256) counter_normal_kernel(T* __restrict__ out, uint64_t n, uint64_t first,
                                                              uint64_t key, float scale, float shift) {
 #pragma clang fp contract(off)
-  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256) {
-    const float v = counter_normal(key, first + i) * scale + shift;
-    out[i] = from_float<T>(v);
+  // a thread a pair: elements 2p and 2p + 1 of the stream, those of them that lie in [first, first + n)
+  const uint64_t p0 = first >> 1, pairs = ((first + n + 1) >> 1) - p0;
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < pairs; i += (uint64_t)gridDim.x * 256) {
+    float a, b;
+    counter_normal_pair(key, p0 + i, a, b);
+    const uint64_t e = 2 * (p0 + i);
+    if (e >= first) out[e - first] = from_float<T>(a * scale + shift);
+    if (e + 1 >= first && e + 1 < first + n) out[e + 1 - first] = from_float<T>(b * scale + shift);
   }
 }
 
@@ -79,7 +87,7 @@ extern "C" int xi_counter_normal(void* out, unsigned long long n, unsigned long 
   XI_CHECK(out != nullptr || n == 0, "counter_normal: no output");
   XI_CHECK(dtype == kF32 || dtype == kBF16, "counter_normal: dtype %d is neither float32 nor bfloat16", dtype);
   if (n == 0) return 0;
-  const unsigned long long want = (n + 255) / 256;
+  const unsigned long long want = (n / 2 + 256) / 256;
   const unsigned grid = (unsigned)(want < 65536ull ? want : 65536ull);
   if (dtype == kF32)
     counter_normal_kernel<float><<<grid, 256, 0, stream>>>((float*)out, n, first, key, scale, shift);

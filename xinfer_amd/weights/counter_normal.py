@@ -1,7 +1,8 @@
 """Seeded normal values from a counter, on the CPU: the twin of csrc/kernels/random_fill.hip.
 
-Element i of a tensor depends on (key, i) alone: splitmix64's (i + 1)-th output from state
-`key` gives two 24-bit uniforms, Box-Muller turns them into a normal value.  The logarithm
+Element i of a tensor depends on (key, i) alone: splitmix64's (i // 2 + 1)-th output from state
+`key` gives two 24-bit uniforms, Box-Muller turns them into two normal values, the cosine's for
+element 2p and the sine's for element 2p + 1.  The logarithm
 and the cosine are polynomials of float32 additions, multiplications, one division and one
 square root, each rounded on its own and in the order of the kernel, so that the CPU and the
 GPU make the same bits.  The reference has no random-weights mode; this is what tests and
@@ -25,11 +26,17 @@ def counter_normal(key: int, first: int, n: int, scale: float = 1.0, shift: floa
         out = np.empty(n, dtype=_F)
     for lo in range(0, n, _BLOCK):
         hi = min(n, lo + _BLOCK)
-        out[lo:hi] = _block(key, first + lo, hi - lo, scale, shift)
+        a, b = first + lo, first + hi                      # elements [a, b): pairs a // 2 .. (b + 1) // 2
+        p0, p1 = a >> 1, (b + 1) >> 1
+        even, odd = _pairs(key, p0, p1 - p0)
+        both = np.empty(2 * (p1 - p0), dtype=_F)
+        both[0::2], both[1::2] = even, odd
+        out[lo:hi] = both[a - 2 * p0:b - 2 * p0] * _F(scale) + _F(shift)
     return out
 
 
-def _block(key: int, first: int, n: int, scale: float, shift: float) -> np.ndarray:
+def _pairs(key: int, first: int, n: int):
+    """(even, odd): the two normal values of pairs first .. first + n - 1."""
     with np.errstate(over="ignore"):
         i = np.arange(first + 1, first + 1 + n, dtype=np.uint64)
         z = np.uint64(key & 0xFFFFFFFFFFFFFFFF) + i * np.uint64(0x9E3779B97F4A7C15)
@@ -63,7 +70,7 @@ def _block(key: int, first: int, n: int, scale: float, shift: float) -> np.ndarr
     for c in (-2.75573192e-07, 2.48015876e-05, -1.38888892e-03, 4.16666679e-02, -0.5, 1.0):
         cs = cs * t2 + _F(c)
     c = np.where(quarter == 0, cs, np.where(quarter == 1, -sn, np.where(quarter == 2, -cs, sn)))
-    out = radius * c
-    out = out * _F(scale) + _F(shift)
-    assert out.dtype == _F
-    return out
+    sv = np.where(quarter == 0, sn, np.where(quarter == 1, cs, np.where(quarter == 2, -sn, -cs)))
+    even, odd = radius * c, radius * sv
+    assert even.dtype == _F and odd.dtype == _F
+    return even, odd
