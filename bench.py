@@ -14,6 +14,9 @@ synchronizations, and all of their tokens have reached the host at the second). 
 and each one's own roofline in `points_roofline`), and decode at batch 8 with four times the
 context (`further`).
 
+`--product M,N,K[,slices[,shape]]` times one bfloat16 product alone, in the hand-written many-row
+tiled kernel and in the vendor library.
+
 `--peaks` adds what this card itself reaches (a read-only stream, one large square product) and
 the fractions of those, beside the fractions of the published peaks that the line always has.
 
@@ -152,6 +155,52 @@ def serve(workload: str, layers, run_ahead: bool = True) -> int:
     return 0
 
 
+def product(spec: str, dev="cuda:0") -> int:
+    """One bfloat16 product x [M, K] @ w [N, K]^T alone: the many-row tiled kernel (with `slices` of K as
+    float32 partial sums, in tile `shape`; left out: what `kernels.tile_split_plan` chooses, or one slice
+    in the shape of fewest tiles) beside the vendor library's plain product, each the best of 5 runs of 20
+    launches in a HIP graph."""
+    import torch
+    from xinfer_amd import kernels
+    parts = [int(v) for v in spec.split(",")]
+    M, N, K = parts[:3]
+    slices, shape = (parts[3], parts[4] if len(parts) > 4 else None) if len(parts) > 3 else kernels.tile_split_plan(M, N, K)
+    g = torch.Generator(device=dev)
+    g.manual_seed(3)
+    x = torch.randn((M, K), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    w = (torch.randn((N, K), generator=g, device=dev, dtype=torch.float32) * 0.05).to(torch.bfloat16)
+
+    def timed(f, n=20):
+        f()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(n):
+                f()
+        best = None
+        for _ in range(5):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            graph.replay()
+            b.record()
+            torch.cuda.synchronize()
+            ms = a.elapsed_time(b) / n
+            best = ms if best is None else min(best, ms)
+        return best * 1e3
+
+    tile_us = timed(lambda: kernels.linear_tile(x, w, slices, partial=slices > 1, shape=shape))
+    lib_us = timed(lambda: torch.nn.functional.linear(x, w))
+    y = kernels.linear_tile(x, w, slices, partial=slices > 1, shape=shape)
+    y = y.sum(0) if y.dim() == 3 else y.float()
+    ref = x.float() @ w.float().t()
+    flops = 2.0 * M * N * K
+    print(json.dumps({"product": [M, N, K], "slices": slices, "tile_shape": shape, "linear_tile_us": round(tile_us, 1),
+                      "library_us": round(lib_us, 1), "linear_tile_tflops": round(flops / tile_us / 1e6, 1),
+                      "library_tflops": round(flops / lib_us / 1e6, 1),
+                      "max_error_of_largest": float((y - ref).abs().max() / ref.abs().max())}), flush=True)
+    return 0
+
+
 def measured_peaks(dev="cuda:0"):
     """(GB/s of a read-only stream over 4 GiB, TFLOP/s of one square bfloat16 product of 8192 in the
     vendor library): what this card reaches, beside the published peaks.  Best of five runs each."""
@@ -209,6 +258,8 @@ def main() -> int:
                     help="run one phase only (for profiling); the JSON line then lacks the other")
     ap.add_argument("--no-run-ahead", action="store_true",
                     help="serving workloads: read every step's tokens on the host before the next step is planned")
+    ap.add_argument("--product", default=None, metavar="M,N,K[,slices[,shape]]",
+                    help="time one bfloat16 product alone in the many-row tiled kernel and in the vendor library")
     ap.add_argument("--peaks", action="store_true",
                     help="also measure what this card reaches on a read-only stream of 4 GiB and on one square "
                          "bfloat16 product of 8192, and report the fractions of those beside the fractions of the "
@@ -217,6 +268,8 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.product:
+        return product(args.product)
     if args.workload != "decode":
         return serve(args.workload, args.layers, not args.no_run_ahead)
     full_layers = MODELS[args.model]["num_hidden_layers"]
