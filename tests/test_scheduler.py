@@ -69,6 +69,26 @@ def test_portions_budget_and_mixing():
     assert [(e.request, e.start, e.count, e.sample) for e in plan] == [(1, 10, 1, True), (0, 64, 6, True)]
 
 
+def test_decoding_requests_come_longest_first():
+    """The attention kernel's workgroups start in the batch's order; the long sequences' must not be the last."""
+    cm, s = make(num_pages=64, max_seqs=4, budget=64, chunk=32)
+    for rid, prompt in enumerate([5, 30, 12]):
+        s.add(rid, prompt, 4)
+    plan, _ = s.schedule()
+    assert [(e.request, e.count) for e in plan] == [(0, 5), (1, 30), (2, 12)]      # prompts: in the queue's order
+    s.commit()
+    for rid in range(3):
+        s.append_token(rid)
+    s.add(3, 20, 4)
+    plan, _ = s.schedule()
+    assert [(e.request, e.start, e.count) for e in plan] == [(1, 30, 1), (2, 12, 1), (0, 5, 1), (3, 0, 20)]
+    s.commit()
+    for rid in range(4):
+        s.append_token(rid)
+    plan, _ = s.schedule()
+    assert [(e.request, e.start) for e in plan] == [(1, 31), (3, 20), (2, 13), (0, 6)]
+
+
 def test_every_token_is_processed_exactly_once():
     cm, s = make(num_pages=64, budget=48, chunk=20)
     reqs = {0: (70, 4), 1: (1, 9), 2: (33, 1), 3: (20, 6), 4: (47, 3), 5: (5, 5)}

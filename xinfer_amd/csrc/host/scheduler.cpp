@@ -124,6 +124,18 @@ const std::vector<SchedEntry>& Scheduler::schedule(std::vector<int64_t>* preempt
     plan_.push_back(SchedEntry{id, 0, (int32_t)n, n == r.total_len ? 1 : 0});
     budget -= n;
   }
+
+  // The decoding requests at the head of the step, longest first: the attention kernel's workgroups
+  // start in the batch's order, and the long sequences' then do not run on alone at the end.
+  size_t decoding = 0;
+  while (decoding < plan_.size()) {
+    const SchedEntry& e = plan_[decoding];
+    const SchedRequest& r = requests_.at(e.id);
+    if (e.count != 1 || e.start < r.prompt_len || e.start + 1 != r.total_len) break;
+    ++decoding;
+  }
+  std::stable_sort(plan_.begin(), plan_.begin() + decoding,
+                   [](const SchedEntry& a, const SchedEntry& b) { return a.start > b.start; });
   return plan_;
 }
 
