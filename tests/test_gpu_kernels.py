@@ -19,6 +19,18 @@ def _tol(dtype, n_round=1):
     return 2e-5 if dtype == torch.float32 else 2.0 ** -8 * n_round
 
 
+def _grouped(vc):
+    """A V pool [pages, nkv, page, d] as the bfloat16 path keeps it: [pages, nkv, page / 8, d, 8], eight keys that
+    follow each other side by side for every dim."""
+    pages, nkv, page, d = vc.shape
+    return vc.reshape(pages, nkv, page // 8, 8, d).transpose(3, 4).contiguous()
+
+
+def _ungrouped(vg):
+    pages, nkv, groups, d, _ = vg.shape
+    return vg.transpose(3, 4).reshape(pages, nkv, groups * 8, d)
+
+
 def _rand(shape, dtype, gen, scale=1.0):
     return (torch.randn(shape, generator=gen) * scale).to(dtype)
 
@@ -605,7 +617,7 @@ def test_qk_norm_rope_kv(dtype, nq, nkv, d, rot, interleaved, norm):
     g = torch.Generator().manual_seed(7)
     # positions of the reference's probe (attention_misc_precision_probe.rs:36-40)
     positions = torch.tensor([0, 7, 2, 31, 9, 16, 3, 63, 4, 12, 5], dtype=torch.int32)
-    T, page, pages, eps = positions.numel(), 4, 9, 1e-5
+    T, page, pages, eps = positions.numel(), 8, 5, 1e-5
     cos, sin = plain.rope_tables(10000.0, rot, 64)
     qkv = _rand((T, (nq + 2 * nkv) * d), dtype, g)
     qw = (1 + 0.3 * torch.randn(d, generator=g)) if norm else None
@@ -631,14 +643,14 @@ def test_qk_norm_rope_kv(dtype, nq, nkv, d, rot, interleaved, norm):
         p, o = int(slots[t]) // page, int(slots[t]) % page
         assert (kcd[p, :, o] - k[t]).abs().max() / k.abs().max() < tol, t
         assert torch.equal(vcd[p, :, o].double(), v[t]), t
-    # the transposed V pool [pages, nkv, d, page] holds the same values
-    vt = torch.zeros((pages, nkv, d, page), dtype=dtype, device=DEV)
+    # the V pool in groups of eight keys [pages, nkv, page / 8, d, 8] holds the same values
+    vt = torch.zeros((pages, nkv, page // 8, d, 8), dtype=dtype, device=DEV)
     q_out_t = kernels.qk_norm_rope_kv(
         qkv.to(DEV), qw.to(DEV) if norm else None, kw.to(DEV) if norm else None, eps, cos.to(DEV),
         sin.to(DEV), rot, interleaved, positions.to(DEV), slots.to(DEV), (kct := kc.to(DEV)), vt, nq, nkv, d,
-        v_transposed=True, vector_min_tokens=1)
-    assert torch.equal(vt.cpu().transpose(2, 3), vcd)
-    # q and K of the transposed form (another kernel for bfloat16) against the same reference
+        v_grouped=True, vector_min_tokens=1)
+    assert torch.equal(_ungrouped(vt.cpu()), vcd)
+    # q and K of that form (another kernel for bfloat16) against the same reference
     assert (q_out_t.cpu().double() - q).abs().max() / q.abs().max() < tol
     kct = kct.cpu().double()
     for t in range(T):
@@ -655,7 +667,7 @@ def test_qk_norm_rope_kv(dtype, nq, nkv, d, rot, interleaved, norm):
 @pytest.mark.parametrize("nq,nkv,d,rot,interleaved", [(32, 8, 128, 128, False), (6, 3, 48, 32, False), (4, 4, 64, 64, True),
                                                     (10, 2, 80, 80, False)])
 def test_qk_norm_rope_kv_many_tokens(nq, nkv, d, rot, interleaved):
-    """The bfloat16 form with the transposed V pool over several blocks of 64 tokens: runs of
+    """The bfloat16 form with the V pool in groups of eight keys over several blocks of 64 tokens: runs of
     tokens that follow each other in a page, a block that is not full, and tokens whose slot is
     negative (nothing of theirs may be stored)."""
     from xinfer_amd import kernels
@@ -670,10 +682,10 @@ def test_qk_norm_rope_kv_many_tokens(nq, nkv, d, rot, interleaved):
                        page_of[7 + torch.arange(50) // page] * page + torch.arange(50) % page]).to(torch.int64)
     slots[torch.tensor([3, 64, 149])] = -1
     kc = torch.zeros((pages, nkv, page, d), dtype=torch.bfloat16, device=DEV)
-    vt = torch.zeros((pages, nkv, d, page), dtype=torch.bfloat16, device=DEV)
+    vt = torch.zeros((pages, nkv, page // 8, d, 8), dtype=torch.bfloat16, device=DEV)
     q_out = kernels.qk_norm_rope_kv(qkv.to(DEV), qw.to(DEV), kw.to(DEV), eps, cos.to(DEV), sin.to(DEV), rot,
                                     interleaved, positions.to(DEV), slots.to(DEV), kc, vt, nq, nkv, d,
-                                    v_transposed=True)
+                                    v_grouped=True)
     x = qkv.double().reshape(T, nq + 2 * nkv, d)
     q = _rope_ref(plain.rms_norm(x[:, :nq], qw.double(), eps), positions.long(), cos, sin, rot, interleaved)
     k = _rope_ref(plain.rms_norm(x[:, nq:nq + nkv], kw.double(), eps), positions.long(), cos, sin, rot, interleaved)
@@ -686,7 +698,7 @@ def test_qk_norm_rope_kv_many_tokens(nq, nkv, d, rot, interleaved):
     want_k[slots[keep]] = k[keep]
     want_v[slots[keep]] = v[keep]
     got_k = kc.cpu().double().permute(0, 2, 1, 3).reshape(pages * page, nkv, d)
-    got_v = vt.cpu().double().permute(0, 3, 1, 2).reshape(pages * page, nkv, d)
+    got_v = _ungrouped(vt.cpu()).double().permute(0, 2, 1, 3).reshape(pages * page, nkv, d)
     assert (got_k - want_k).abs().max() / k.abs().max() < tol
     assert torch.equal(got_v, want_v)
 
@@ -710,9 +722,9 @@ def test_qk_norm_rope_kv_bias(dtype, T, nq, nkv, d, rot, interleaved):
     slots = torch.randperm(pages * page, generator=g)[:T].to(torch.int64)
     vt_form = dtype == torch.bfloat16
     kc = torch.zeros((pages, nkv, page, d), dtype=dtype, device=DEV)
-    vc = torch.zeros((pages, nkv, d, page) if vt_form else (pages, nkv, page, d), dtype=dtype, device=DEV)
+    vc = torch.zeros((pages, nkv, page // 8, d, 8) if vt_form else (pages, nkv, page, d), dtype=dtype, device=DEV)
     q_out = kernels.qk_norm_rope_kv(qkv.to(DEV), qw.to(DEV), kw.to(DEV), eps, cos.to(DEV), sin.to(DEV), rot, interleaved,
-                                    positions.to(DEV), slots.to(DEV), kc, vc, nq, nkv, d, v_transposed=vt_form,
+                                    positions.to(DEV), slots.to(DEV), kc, vc, nq, nkv, d, v_grouped=vt_form,
                                     bias=bias.to(DEV))
     x = (qkv.double() + bias.double()).reshape(T, nq + 2 * nkv, d)
     q = _rope_ref(plain.rms_norm(x[:, :nq], qw.double(), eps), positions.long(), cos, sin, rot, interleaved)
@@ -721,12 +733,12 @@ def test_qk_norm_rope_kv_bias(dtype, T, nq, nkv, d, rot, interleaved):
     tol = _tol(dtype)
     assert (q_out.cpu().double() - q).abs().max() / q.abs().max() < tol
     got_k = kc.cpu().double().permute(0, 2, 1, 3).reshape(pages * page, nkv, d)
-    got_v = (vc.cpu().permute(0, 3, 1, 2) if vt_form else vc.cpu().permute(0, 2, 1, 3)).reshape(pages * page, nkv, d)
+    got_v = (_ungrouped(vc.cpu()) if vt_form else vc.cpu()).permute(0, 2, 1, 3).reshape(pages * page, nkv, d)
     assert (got_k[slots] - k).abs().max() / k.abs().max() < tol
     assert torch.equal(got_v[slots], v)
     with pytest.raises(kernels.KernelError, match="bias"):
         kernels.qk_norm_rope_kv(qkv.to(DEV), qw.to(DEV), kw.to(DEV), eps, cos.to(DEV), sin.to(DEV), rot, interleaved,
-                                positions.to(DEV), slots.to(DEV), kc, vc, nq, nkv, d, v_transposed=vt_form,
+                                positions.to(DEV), slots.to(DEV), kc, vc, nq, nkv, d, v_grouped=vt_form,
                                 bias=bias[:-1].contiguous().to(DEV))
 
 
@@ -748,9 +760,9 @@ def test_qk_norm_rope_kv_of_partial_sums(T, nq, nkv, d, rot, interleaved, slices
     qw, kw = 1 + 0.3 * torch.randn(d, generator=g), 1 + 0.3 * torch.randn(d, generator=g)
     slots = torch.randperm(pages * page, generator=g)[:T].to(torch.int64)
     kc = torch.zeros((pages, nkv, page, d), dtype=torch.bfloat16, device=DEV)
-    vc = torch.zeros((pages, nkv, d, page), dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros((pages, nkv, page // 8, d, 8), dtype=torch.bfloat16, device=DEV)
     q_out = kernels.qk_norm_rope_kv(parts.to(DEV), qw.to(DEV), kw.to(DEV), eps, cos.to(DEV), sin.to(DEV), rot, interleaved,
-                                    positions.to(DEV), slots.to(DEV), kc, vc, nq, nkv, d, v_transposed=True,
+                                    positions.to(DEV), slots.to(DEV), kc, vc, nq, nkv, d, v_grouped=True,
                                     bias=None if bias is None else bias.to(DEV))
     assert q_out.dtype == torch.bfloat16 and tuple(q_out.shape) == (T, nq, d)
     total = parts.double().sum(0) + (0 if bias is None else bias.double())
@@ -761,12 +773,12 @@ def test_qk_norm_rope_kv_of_partial_sums(T, nq, nkv, d, rot, interleaved, slices
     tol = _tol(torch.bfloat16)
     assert (q_out.cpu().double() - q).abs().max() / q.abs().max() < tol
     got_k = kc.cpu().double().permute(0, 2, 1, 3).reshape(pages * page, nkv, d)
-    got_v = vc.cpu().double().permute(0, 3, 1, 2).reshape(pages * page, nkv, d)
+    got_v = _ungrouped(vc.cpu()).double().permute(0, 2, 1, 3).reshape(pages * page, nkv, d)
     assert (got_k[slots] - k).abs().max() / k.abs().max() < tol
     assert (got_v[slots] - v).abs().max() / v.abs().max() < tol
     with pytest.raises(kernels.KernelError, match="partial sums"):
         kernels.qk_norm_rope_kv(parts.to(DEV).to(torch.bfloat16), qw.to(DEV), kw.to(DEV), eps, cos.to(DEV), sin.to(DEV), rot,
-                                interleaved, positions.to(DEV), slots.to(DEV), kc, vc, nq, nkv, d, v_transposed=True)
+                                interleaved, positions.to(DEV), slots.to(DEV), kc, vc, nq, nkv, d, v_grouped=True)
 
 
 def _paged_case(g, dtype, nq, nkv, d, page, seqs, extra_pages=3):
@@ -860,10 +872,9 @@ def test_attention_far_key_stands_out(dtype):
     assert err < _tol(dtype, 2), err
 
 
-# ---- the matrix-core attention kernels (bfloat16, V transposed in the cache) -------------------
+# ---- the matrix-core attention kernels (bfloat16, V in groups of eight keys in the cache) -----
 def _mfma_inputs(case):
-    return (torch.cat(case["qs"]).contiguous().to(DEV), case["kc"].to(DEV),
-            case["vc"].transpose(2, 3).contiguous().to(DEV), case["bt"].to(DEV))
+    return (torch.cat(case["qs"]).contiguous().to(DEV), case["kc"].to(DEV), _grouped(case["vc"]).to(DEV), case["bt"].to(DEV))
 
 
 def _cu_ctx(seqs):
@@ -923,9 +934,9 @@ def test_attention_prefill_mfma(nq, nkv, d, page, window, seqs):
     if not kernels.prefill_ring_supported(d):
         with pytest.raises(kernels.KernelError, match="two groups"):
             kernels.attention_prefill_bf16(q, kc, vt, bt, tiles.to(DEV), cu.to(DEV), ctx.to(DEV), scale, window, small=2)
-    # the generic kernel reads the transposed pool too
+    # the generic kernel reads the grouped pool too
     out2 = kernels.attention_generic(q, kc, vt, bt, case["tok_seq"].to(DEV), case["positions"].to(DEV), scale,
-                                     window, v_transposed=True)
+                                     window, v_grouped=True)
     err = (out2.cpu().double() - ref).abs().max() / ref.abs().max()
     assert err < _tol(torch.bfloat16, 2), err
 
@@ -988,7 +999,7 @@ def test_attention_of_a_mixed_batch_splits_between_the_kernels(nq, nkv, d, page,
         kernels_work = kernels.MIXED_DECODE_WORK
         kernels.MIXED_DECODE_WORK = 1000          # small sizes here: the rule's threshold is for real ones
         try:
-            out = kernels.attention(q, kc, vt, ctx, 0, scale, window, v_transposed=True)
+            out = kernels.attention(q, kc, vt, ctx, 0, scale, window, v_grouped=True)
         finally:
             kernels.MIXED_DECODE_WORK = kernels_work
         (tiles, small, lead, lead_ctx), = ctx.scratch.values()
@@ -1110,7 +1121,7 @@ def test_attention_decode_packed_gives_the_bits_of_the_two_kernels(nq, nkv, d, p
     def both(packed):
         k1, v1 = kc.clone(), vt.clone()
         q = kernels.qk_norm_rope_kv(packed.to(DEV), qw, kw, eps, cos, sin, rot, interleaved, positions, slots, k1, v1,
-                                    nq, nkv, d, v_transposed=True, vector_min_tokens=1 << 30, bias=bs)
+                                    nq, nkv, d, v_grouped=True, vector_min_tokens=1 << 30, bias=bs)
         one = kernels.attention_decode_bf16(q, k1, v1, bt, ctx_d, longest, scale, window, keys_per_workgroup=kpw)
         k2, v2 = kc.clone(), vt.clone()
         two = kernels.attention_decode_packed_bf16(packed.to(DEV), qw, kw, eps, cos, sin, rot, interleaved, positions,
@@ -1125,7 +1136,7 @@ def test_attention_decode_packed_gives_the_bits_of_the_two_kernels(nq, nkv, d, p
     # the sequence with the negative slot: its place in the cache is as it was
     c = contexts[B - 1]
     pg, off = int(case["bt"][B - 1, (c - 1) // page]), (c - 1) % page
-    assert torch.equal(k2[pg, :, off], kc[pg, :, off]) and torch.equal(v2[pg, :, :, off], vt[pg, :, :, off])
+    assert torch.equal(k2[pg, :, off], kc[pg, :, off]) and torch.equal(v2[pg, :, off >> 3, :, off & 7], vt[pg, :, off >> 3, :, off & 7])
     if not norm and not rot and not slices:
         # the new key of sequence 0 points along its first query head of every group, far longer than any other
         x = packed.clone().reshape(B, heads, d)
@@ -1143,7 +1154,7 @@ def test_attention_decode_packed_refuses():
     from xinfer_amd import kernels
     nq, nkv, d, page = 4, 2, 32, 16
     kc = torch.zeros((4, nkv, page, d), dtype=torch.bfloat16, device=DEV)
-    vt = torch.zeros((4, nkv, d, page), dtype=torch.bfloat16, device=DEV)
+    vt = torch.zeros((4, nkv, page // 8, d, 8), dtype=torch.bfloat16, device=DEV)
     bt = torch.zeros((2, 2), dtype=torch.int32, device=DEV)
     ctx = torch.tensor([3, 5], dtype=torch.int32, device=DEV)
     pos = (ctx - 1).to(torch.int32)

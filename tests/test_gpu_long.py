@@ -216,10 +216,10 @@ def test_matrix_core_attention_agrees_with_the_generic_kernel_inside_the_model(s
 
     inner_attention, inner_packed = kernels.attention, kernels.attention_decode_packed_bf16
 
-    def attention(q, k_cache, v_cache, ctx, group, scale, window=0, v_transposed=False):
-        a = inner_attention(q, k_cache, v_cache, ctx, group, scale, window, v_transposed=v_transposed)
+    def attention(q, k_cache, v_cache, ctx, group, scale, window=0, v_grouped=False):
+        a = inner_attention(q, k_cache, v_cache, ctx, group, scale, window, v_grouped=v_grouped)
         note(a, kernels.attention_generic(q, k_cache, v_cache, ctx.block_tables[group], ctx.tok_seq, ctx.positions, scale,
-                                          window, v_transposed=v_transposed), v_cache)
+                                          window, v_grouped=v_grouped), v_cache)
         return a
 
     def packed(qkv, q_weight, k_weight, eps, cos, sin, rotary_dim, interleaved, positions, slots, k_cache, vt_cache,
@@ -231,9 +231,9 @@ def test_matrix_core_attention_agrees_with_the_generic_kernel_inside_the_model(s
         B = positions.shape[0]
         q = kernels.qk_norm_rope_kv(qkv, q_weight, k_weight, eps, cos, sin, rotary_dim, interleaved, positions,
                                     torch.full((B,), -1, dtype=torch.int64, device=DEV), k_cache, vt_cache, num_heads,
-                                    k_cache.shape[1], k_cache.shape[3], v_transposed=True, vector_min_tokens=1 << 30, bias=bias)
+                                    k_cache.shape[1], k_cache.shape[3], v_grouped=True, vector_min_tokens=1 << 30, bias=bias)
         note(a, kernels.attention_generic(q, k_cache, vt_cache, block_tables, torch.arange(B, dtype=torch.int32, device=DEV),
-                                          positions, scale, window, v_transposed=True), vt_cache)
+                                          positions, scale, window, v_grouped=True), vt_cache)
         return a
 
     kernels.attention, kernels.attention_decode_packed_bf16 = attention, packed
@@ -333,11 +333,13 @@ def test_reference_attention_probe_cases(prefix, append, hq, hkv, page_map):
     else:
         phys = (torch.randperm(n_pages + 3, generator=g)[:n_pages]).tolist()
     kc = torch.zeros((n_pages + 3, hkv, page, d), dtype=torch.bfloat16)
-    vt = torch.zeros((n_pages + 3, hkv, d, page), dtype=torch.bfloat16)
+    vc = torch.zeros((n_pages + 3, hkv, page, d), dtype=torch.bfloat16)
     for lp in range(-(-prefix // page)):
         n = min(page, prefix - lp * page)
         kc[phys[lp], :, :n] = k[lp * page:lp * page + n].transpose(0, 1)
-        vt[phys[lp], :, :, :n] = v[lp * page:lp * page + n].permute(1, 2, 0)
+        vc[phys[lp], :, :n] = v[lp * page:lp * page + n].transpose(0, 1)
+    # the bfloat16 path keeps V in groups of eight keys: [pages, kv heads, page / 8, d, 8]
+    vt = vc.reshape(n_pages + 3, hkv, page // 8, 8, d).transpose(3, 4).contiguous()
     kc, vt = kc.to(DEV), vt.to(DEV)
     bt = torch.tensor([phys], dtype=torch.int32, device=DEV)
     positions = torch.arange(prefix, kv_len, dtype=torch.int32)
@@ -345,12 +347,12 @@ def test_reference_attention_probe_cases(prefix, append, hq, hkv, page_map):
     packed = torch.cat([q.reshape(append, -1), k[prefix:].reshape(append, -1), v[prefix:].reshape(append, -1)], dim=1)
     none = torch.empty((1, 0), dtype=torch.float32, device=DEV)
     q_dev = kernels.qk_norm_rope_kv(packed.contiguous().to(DEV), None, None, 1e-6, none, none, 0, False,
-                                    positions.to(DEV), slots.to(DEV), kc, vt, hq, hkv, d, v_transposed=True)
+                                    positions.to(DEV), slots.to(DEV), kc, vt, hq, hkv, d, v_grouped=True)
     assert torch.equal(q_dev.cpu(), q)
     # the pages read back through the table hold k and v in order (compare_flashinfer_probe.py:102-113)
     idx = torch.tensor(phys, device=DEV)
     assert torch.equal(kc[idx].permute(0, 2, 1, 3).reshape(-1, hkv, d)[:kv_len].cpu(), k)
-    assert torch.equal(vt[idx].permute(0, 3, 1, 2).reshape(-1, hkv, d)[:kv_len].cpu(), v)
+    assert torch.equal(vt[idx].transpose(3, 4).reshape(len(phys), hkv, page, d).permute(0, 2, 1, 3).reshape(-1, hkv, d)[:kv_len].cpu(), v)
 
     gold = _rows_golden(q, positions.long(), k, v, scale)
     assert (gold[-1, 0] - v[far, 0].float()).abs().max() < 0.05            # the far key won that row
@@ -380,5 +382,5 @@ def test_reference_attention_probe_cases(prefix, append, hq, hkv, page_map):
                                             keys_per_workgroup=kpw, similar=similar)
         check(out, slice(append - n_last, append), f"decode kpw={kpw} span={span} similar={similar}")
     out = kernels.attention_generic(q_dev[-n_last:].contiguous(), kc, vt, bt, torch.zeros(n_last, dtype=torch.int32, device=DEV),
-                                    positions[-n_last:].to(DEV), scale, 0, v_transposed=True)
+                                    positions[-n_last:].to(DEV), scale, 0, v_grouped=True)
     check(out, slice(append - n_last, append), "generic")

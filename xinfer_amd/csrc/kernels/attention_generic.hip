@@ -3,7 +3,7 @@
 // the attention of the 32-bit path; the bfloat16 path uses it where no faster kernel
 // applies.  Keys of a token at position p are the cached positions lo..p of its own
 // request, lo = max(0, p - window + 1), read through the request's block table.  K is
-// [page, kv_head, offset, d]; V is the same or, with v_transposed, [page, kv_head, d, offset].
+// [page, kv_head, offset, d]; V is the same or, with v_grouped, [page, kv_head, offset / 8, d, 8].
 //
 // Reference: PagedAttention::forward at /root/reference/src/models/layers/attention.rs:947-958
 // (external kernel); golden formula tests/probes/compare_flashinfer_probe.py:51-73:
@@ -25,7 +25,7 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attention_generic_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int max_pages, const int* __restrict__ tok_seq,
     const int* __restrict__ positions, T* __restrict__ out, float scale, int window, int page_size,
-    int nq, int nkv, int d, int v_transposed) {
+    int nq, int nkv, int d, int v_grouped) {
   __shared__ float q_s[kMaxHeadDim];
   __shared__ float acc_s[kAttnWaves][kMaxHeadDim];
   __shared__ float m_s[kAttnWaves], l_s[kAttnWaves];
@@ -56,7 +56,7 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attention_generic_kernel(
     const int key = lo + c * kWave + lane;
     const bool valid = key <= pos;
     int row = 0;  // row of this lane's key in the cache, in units of d elements
-    int vrow = 0, voff = 0;  // transposed V: first row of the (page, kv head) block and the offset
+    int vrow = 0, voff = 0;  // grouped V: first row of the (page, kv head) block and the offset
     float s = -INFINITY;
     if (valid) {
       const int page = bt[key / page_size];
@@ -82,12 +82,12 @@ __global__ __launch_bounds__(kAttnWaves* kWave) void attention_generic_kernel(
       const int vrj = __shfl(vrow, j, kWave);
       const int voj = __shfl(voff, j, kWave);
       const T* vp = v_cache + (size_t)rj * d;
-      const T* vtp = v_cache + (size_t)vrj * page_size + voj;  // [d, page_size] block
+      const T* vtp = v_cache + (size_t)vrj * page_size + (size_t)(voj >> 3) * d * 8 + (voj & 7);  // [offset / 8, d, 8] block
 #pragma unroll
       for (int e = 0; e < NE; ++e) {
         const int i = lane + e * kWave;
         if (i < d) {
-          const float vv = v_transposed ? to_float(vtp[(size_t)i * page_size]) : to_float(vp[i]);
+          const float vv = v_grouped ? to_float(vtp[(size_t)i * 8]) : to_float(vp[i]);
           acc[e] = fmaf(pj, vv, acc[e]);
         }
       }
@@ -130,22 +130,23 @@ extern "C" int xi_attention_generic(const void* q, const void* k_cache, const vo
                                     int dtype, const int* block_tables, int max_pages,
                                     const int* tok_seq, const int* positions, void* out,
                                     float scale, int window, int page_size, int n_tok, int nq,
-                                    int nkv, int d, int v_transposed, hipStream_t stream) {
+                                    int nkv, int d, int v_grouped, hipStream_t stream) {
   XI_CHECK(n_tok >= 0 && nq > 0 && nkv > 0 && page_size > 0 && max_pages > 0,
            "attention: bad sizes T=%d nq=%d nkv=%d page=%d max_pages=%d", n_tok, nq, nkv, page_size, max_pages);
   XI_CHECK(nq % nkv == 0, "attention: %d query heads are not a multiple of %d kv heads", nq, nkv);
   XI_CHECK(d > 0 && d <= kMaxHeadDim, "attention: head_dim %d is outside 1..%d", d, kMaxHeadDim);
   XI_CHECK(nq <= 65535, "attention: too many heads (%d)", nq);
+  XI_CHECK(!v_grouped || page_size % 8 == 0, "attention: V in groups of eight keys needs pages of a multiple of 8 tokens, not %d", page_size);
   if (n_tok == 0) return 0;
   dim3 grid(n_tok, nq);
   if (dtype == kF32)
     attention_generic_kernel<float><<<grid, kAttnWaves * kWave, 0, stream>>>(
         (const float*)q, (const float*)k_cache, (const float*)v_cache, block_tables, max_pages,
-        tok_seq, positions, (float*)out, scale, window, page_size, nq, nkv, d, v_transposed);
+        tok_seq, positions, (float*)out, scale, window, page_size, nq, nkv, d, v_grouped);
   else if (dtype == kBF16)
     attention_generic_kernel<bf16><<<grid, kAttnWaves * kWave, 0, stream>>>(
         (const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache, block_tables, max_pages,
-        tok_seq, positions, (bf16*)out, scale, window, page_size, nq, nkv, d, v_transposed);
+        tok_seq, positions, (bf16*)out, scale, window, page_size, nq, nkv, d, v_grouped);
   else
     XI_CHECK(false, "attention: unknown dtype %d", dtype);
   XI_LAUNCH_CHECK("attention_generic");

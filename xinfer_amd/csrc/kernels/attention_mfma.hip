@@ -16,9 +16,12 @@
 // same slots.  Row m of the two K tiles of a step is therefore key 8*(m/4) + m%4 (tile 0)
 // and that + 4 (tile 1): lane group j then holds keys 8j..8j+7, one 16-byte load from V^T.
 //
-// The cache keeps K as [page, kv_head, offset, d] and V transposed as
-// [page, kv_head, d, offset], so both operands are read from global memory in the layout
-// the matrix cores want.  Softmax runs in float32 (exp2 with log2(e) folded into the
+// The cache keeps K as [page, kv_head, offset, d] and V in groups of eight keys as
+// [page, kv_head, offset / 8, d, 8], so both operands are read from global memory in the layout
+// the matrix cores want: a lane's 16 bytes of V^T are eight keys of one dim, sixteen dims lie side
+// by side (a wave's load of a step takes four runs of 256 bytes a tile; with a whole page's keys
+// side by side it took sixteen half lines, and a new token's value d lines of the pool instead of
+// d / 8: 64 sequences of 4,096 keys went from 190 to 178 us, 256 of 1,024 from 233 to 202).  Softmax runs in float32 (exp2 with log2(e) folded into the
 // scale); all per-query state (running max, sum, correction) lives in the lanes of that
 // query's column.
 //
@@ -150,14 +153,14 @@ __global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
       }
     }
   };
-  // V^T operands: row 16*dt + r, keys k_base + 8j .. +7
+  // V^T operands: row 16*dt + r, keys k_base + 8j .. +7 (one group of eight of the pool)
   auto load_v = [&](int k_base) {
     int vgrp = k_base + 8 * j;
     if (vgrp > pos) vgrp = pos & ~7;
     const int vpage = pages[(vgrp >> page_shift) - first_page];
-    const bf16* vp = vt_cache + (((size_t)vpage * nkv + kvh) * d + r) * page + (vgrp & (page - 1));
+    const bf16* vp = vt_cache + ((size_t)vpage * nkv + kvh) * d * page + ((size_t)((vgrp & (page - 1)) >> 3) * d + r) * 8;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) va[dt] = (16 * dt < d) ? load8(vp + (size_t)16 * dt * page) : zero8();
+    for (int dt = 0; dt < DT; ++dt) va[dt] = (16 * dt < d) ? load8(vp + (size_t)16 * dt * 8) : zero8();
   };
 
   // this lane's query column: head kvh*g + r of the sequence, or none
@@ -198,7 +201,7 @@ __global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
     const long long spage = slot >> page_shift;
     const int soff = (int)(slot & (page - 1));
     bf16* k_new = k_cache_w + (((size_t)spage * nkv + kvh) * page + soff) * d;
-    bf16* v_new = vt_cache_w + ((size_t)spage * nkv + kvh) * d * page + soff;
+    bf16* v_new = vt_cache_w + ((size_t)spage * nkv + kvh) * d * page + (size_t)(soff >> 3) * d * 8 + (soff & 7);
     lds_barrier();     // the page numbers are in LDS
     // The first keys and values are asked for before the heads are worked on, except in a chunk so
     // short that a wave's first step holds the new key: that waits until the key is written.
@@ -210,7 +213,7 @@ __global__ __launch_bounds__(256, DT > 8 ? 1 : 2) void attn_decode_split_kernel(
     for (int row = wave; row < n_rows; row += 4) {
       const auto x = packed_head(head_of(row));
       if (row == 1 && owner)
-        copy_head<bf16, PARTS>(x, d, lane, v_new, (size_t)page);
+        copy_head<bf16, PARTS>(x, d, lane, v_new, (size_t)8);
       else      // a query head into LDS, or the new key into the cache
         norm_rope_head<bf16, PARTS>(x, row >= first_q ? ps.qw : ps.kw, ps.eps, ps.cos_t, ps.sin_t, ps.rot, ps.interleaved,
                                     tok_pos, d, lane, row >= first_q ? qs + (size_t)(row - first_q) * d : k_new);

@@ -161,8 +161,8 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_prefill_lds_kernel(
       key0 = key0 > k_last ? (k_last & ~7) : key0;
       const int vp = bt_s[key0 >> page_shift];
       const int vr = (idx >> 3) < d ? (idx >> 3) : d - 1;     // rows past head_dim are not stored
-      vreg[i] = ld8(vt_cache + ((size_t)vp * nkv + kvh) * kv_head_stride + ((size_t)vr << page_shift) +
-                    (key0 & (page - 1)));
+      vreg[i] = ld8(vt_cache + ((size_t)vp * nkv + kvh) * kv_head_stride +
+                    ((size_t)((key0 & (page - 1)) >> 3) * d + vr) * 8);     // [offset / 8, d, 8]
     }
   };
   auto stash = [&](int buf) {

@@ -131,7 +131,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_prefill_ring_kernel(
   for (int t = 0; t < LPW; ++t) {
     const int ii = wave_abs + NWV * t;
     ld_lane[t] = ii < KI ? 2u * (unsigned)(ld_key[t] * D + ld_off[t])
-                         : 2u * (((unsigned)ld_off[t] << page_shift) + (unsigned)ld_key[t]);
+                         : 2u * (unsigned)(((ld_key[t] >> 3) * D + ld_off[t]) * 8);      // V: [offset / 8, d, 8]
   }
   // where this lane reads the matrix operands within a stage (bytes): K rows r and 16 + r of a step,
   // chunk 4c + j at its permuted place; V^T rows 16 dt + r, chunk 4 sub + j at its permuted place.
@@ -203,7 +203,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_prefill_ring_kernel(
       const int pid = __builtin_amdgcn_readfirstlane(bt_s[kb >> page_shift]);
       const size_t blk = ((size_t)pid * nkv + kvh) * kv_head_stride;
       const bf16* kbase = k_cache + blk + (size_t)(kb & (page - 1)) * D;
-      const bf16* vbase = vt_cache + blk + (kb & (page - 1));
+      const bf16* vbase = vt_cache + blk + (size_t)((kb & (page - 1)) >> 3) * D * 8;
 #pragma unroll
       for (int t = 0; t < LPW; ++t) {
         const int ii = wave_abs + NWV * t;
@@ -228,8 +228,7 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_prefill_ring_kernel(
         int key0 = kb + ld_key[t];
         key0 = key0 > k_last ? (k_last & ~7) : key0;
         const int vp = bt_s[key0 >> page_shift];
-        src = vt_cache + ((size_t)vp * nkv + kvh) * kv_head_stride + ((size_t)ld_off[t] << page_shift) +
-              (key0 & (page - 1));
+        src = vt_cache + ((size_t)vp * nkv + kvh) * kv_head_stride + ((size_t)((key0 & (page - 1)) >> 3) * D + ld_off[t]) * 8;
       }
       load_lds16(src, __builtin_amdgcn_readfirstlane(base + ld_dst[t]));
     }

@@ -250,7 +250,9 @@ __global__ void silu_mul_vec8_kernel(const bf16* __restrict__ gu, bf16* __restri
 //     o_a = a*cos - b*sin;  o_b = a*sin + b*cos
 //   q goes to q_out [T, nq, d]; k and v go to cache[page, kv_head, offset, :] with
 //   slot = page*page_size + offset (reference slot formula runner.rs:1344-1362); with
-//   v_transposed the V pool is [page, kv_head, d, offset] (what the MFMA attention reads).
+//   v_grouped the V pool is [page, kv_head, offset / 8, d, 8]: eight keys that follow each other lie
+//   side by side for every dim (the 16 bytes a lane of the MFMA attention reads), and a token's d
+//   values fall into d / 8 lines of 128 bytes (into d lines if a whole page's keys lay side by side).
 //   A negative slot means: do not store (the token's cache belongs to another run).
 //   `bias` (float32, one value per element of the packed row, or null) is the projections'
 //   bias: it is added here, in float32, to the product the row holds (q, k and v alike;
@@ -268,7 +270,7 @@ __global__ void qk_norm_rope_kv_kernel(const void* __restrict__ qkv_v, int slice
                                        const int* __restrict__ positions,
                                        const long long* __restrict__ slots, T* __restrict__ q_out,
                                        T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                       int page_size, int n_tok, int nq, int nkv, int d, int v_transposed) {
+                                       int page_size, int n_tok, int nq, int nkv, int d, int v_grouped) {
   const int heads = nq + 2 * nkv;
   const int lane = threadIdx.x & (kWave - 1);
   const long long wid = (long long)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
@@ -291,19 +293,20 @@ __global__ void qk_norm_rope_kv_kernel(const void* __restrict__ qkv_v, int slice
   if (is_k)
     norm_rope_head<T, PARTS>(x, kw, eps, cos_t, sin_t, rot, interleaved, positions[t], d, lane,
                              k_cache + (((size_t)page * nkv + kvh) * page_size + off) * d);
-  else if (v_transposed)   // V kept as [page, kv_head, d, offset]
-    copy_head<T, PARTS>(x, d, lane, v_cache + ((size_t)page * nkv + kvh) * d * page_size + off, (size_t)page_size);
+  else if (v_grouped)      // V kept as [page, kv_head, offset / 8, d, 8]
+    copy_head<T, PARTS>(x, d, lane, v_cache + ((size_t)page * nkv + kvh) * d * page_size + (size_t)(off >> 3) * d * 8 + (off & 7),
+                        (size_t)8);
   else
     copy_head<T, PARTS>(x, d, lane, v_cache + (((size_t)page * nkv + kvh) * page_size + off) * d, 1);
 }
 
-// The same for bfloat16 with the transposed V pool, 16 bytes per lane and one pass: a
+// The same for bfloat16 with the V pool in groups of eight keys, 16 bytes per lane and one pass: a
 // workgroup owns one head of the packed row for a block of consecutive tokens.  A head of a
 // token is d/8 lanes of 8 elements (sums and the rotary partner are exchanged inside that
 // group of lanes), a wave holds 64/(d/8) tokens, the workgroup's waves hold the block.  The
-// workgroup of a V head turns its [tokens, d] tile through LDS so that the transposed pool
-// is written with lanes along the token axis: tokens that follow each other in a page
-// become one contiguous store.
+// workgroup of a V head turns its [tokens, d] tile through LDS so that a wave's store takes eight
+// tokens by eight dims: where the eight tokens follow each other in a group of the pool, one line
+// of 128 bytes.
 // Needs d % 8 == 0 and, for the half layout, rotary_dim % 16 == 0 (the partner of a lane's
 // 8 elements is then another lane's 8 elements).
 struct alignas(16) bf16x8v { bf16 v[8]; };
@@ -346,14 +349,17 @@ __global__ __launch_bounds__(1024) void qk_norm_rope_kvt_bf16_kernel(
       dst[3] = raw.w;
     }
     __syncthreads();
-    const int tok = lane;   // token of the block this lane writes
-    const long long slot = (tok < tpw && t0 + tok < n_tok) ? slots[t0 + tok] : -1;
-    if (slot >= 0) {
-      const long long page = slot / page_size;
-      const int off = (int)(slot - page * page_size);
-      bf16* dst = vt_cache + ((size_t)page * nkv + kvh) * d * page_size + off;
-      const bf16* src = vs + tok * vstride;
-      for (int i = wave; i < d; i += (int)(blockDim.x >> 6)) dst[(size_t)i * page_size] = src[i];
+    // lane: token 8 tg + (lane & 7) of the block, dim i0 + (lane >> 3)
+    const int units = ((tpw + 7) >> 3) * (d >> 3);
+    for (int u = wave; u < units; u += (int)(blockDim.x >> 6)) {
+      const int tg = u / (d >> 3), i = 8 * (u - tg * (d >> 3)) + (lane >> 3);
+      const int tok = 8 * tg + (lane & 7);
+      const long long slot = (tok < tpw && t0 + tok < n_tok) ? slots[t0 + tok] : -1;
+      if (slot >= 0) {
+        const long long page = slot / page_size;
+        const int off = (int)(slot - page * page_size);
+        vt_cache[((size_t)page * nkv + kvh) * d * page_size + ((size_t)(off >> 3) * d + i) * 8 + (off & 7)] = vs[tok * vstride + i];
+      }
     }
     return;
   }
@@ -570,7 +576,7 @@ int xi_silu_mul(const void* gate_up, void* out, int dtype, int n_tok, int I, hip
 int xi_qk_norm_rope_kv(const void* qkv, int dtype, int slices, const float* bias, const float* qw, const float* kw, float eps,
                        const float* cos_t, const float* sin_t, int rot, int interleaved,
                        const int* positions, const long long* slots, void* q_out, void* k_cache,
-                       void* v_cache, int page_size, int n_tok, int nq, int nkv, int d, int v_transposed,
+                       void* v_cache, int page_size, int n_tok, int nq, int nkv, int d, int v_grouped,
                        int vector_min_tokens, hipStream_t stream) {
   XI_CHECK(n_tok >= 0 && nq > 0 && nkv > 0 && d > 0 && page_size > 0,
            "qk_norm_rope_kv: bad sizes T=%d nq=%d nkv=%d d=%d page=%d", n_tok, nq, nkv, d, page_size);
@@ -581,7 +587,9 @@ int xi_qk_norm_rope_kv(const void* qkv, int dtype, int slices, const float* bias
   // Many tokens (prompt portions): the vectorized form.  Few (decode steps): one wave per
   // (token, head) below, whose shorter chain of dependent loads finishes sooner.
   XI_CHECK(slices >= 0 && slices <= 64, "qk_norm_rope_kv: %d slices", slices);
-  if (slices == 0 && n_tok >= vector_min_tokens && dtype == kBF16 && v_transposed && d % 8 == 0 && d <= 256 &&
+  XI_CHECK(!v_grouped || page_size % 8 == 0, "qk_norm_rope_kv: V in groups of eight keys needs pages of a multiple of 8 tokens, not %d",
+           page_size);
+  if (slices == 0 && n_tok >= vector_min_tokens && dtype == kBF16 && v_grouped && d % 8 == 0 && d <= 256 &&
       (interleaved || rot % 16 == 0) &&
       ((uintptr_t)qkv | (uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)cos_t | (uintptr_t)sin_t) % 16 == 0) {
     const int lph = d / 8, hpw = 64 / lph;
@@ -605,7 +613,7 @@ int xi_qk_norm_rope_kv(const void* qkv, int dtype, int slices, const float* bias
 #define XI_QK(TT, PARTS)                                                                        \
   qk_norm_rope_kv_kernel<TT, PARTS><<<(unsigned)blocks, wpb * kWave, 0, stream>>>(              \
       qkv, slices, slice_stride, bias, qw, kw, eps, cos_t, sin_t, rot, interleaved, positions, slots, (TT*)q_out, \
-      (TT*)k_cache, (TT*)v_cache, page_size, n_tok, nq, nkv, d, v_transposed)
+      (TT*)k_cache, (TT*)v_cache, page_size, n_tok, nq, nkv, d, v_grouped)
   if (dtype == kF32 && slices == 0) XI_QK(float, false);
   else if (dtype == kF32) XI_QK(float, true);
   else if (dtype == kBF16 && slices == 0) XI_QK(bf16, false);

@@ -24,7 +24,7 @@ import numpy as np
 import torch
 
 from ..cache import DecodeStepError, BatchArrays, CacheGroup, PagedCacheManager
-from ..parts import PAGE, LayerCache, StepContext
+from ..parts import LayerCache, StepContext
 from .model import CausalLM
 
 
@@ -173,10 +173,14 @@ class ModelRunner:
             g = model.group_of_layer[layer]
             pools = {}
             for pool in kv.pools:         # what the mixer declares, page by page
-                if pool.name in pools or sum(1 for s in pool.shape if s == PAGE) != 1:
+                if pool.name in pools or sum(1 for s in pool.shape if s < 0) != 1:
                     raise ValueError(f"layer {layer}: pool {pool.name!r} of shape {pool.shape} must have a name of its "
                                      "own and exactly one axis of the page's length")
-                shape = (groups[g].num_pages, *(self.page_size if s == PAGE else int(s) for s in pool.shape))
+                by = -min(pool.shape)      # PAGE: 1; PAGE_BY_8: 8
+                if self.page_size % by:
+                    raise ValueError(f"layer {layer}: pool {pool.name!r} keeps its pages in groups of {by} tokens: "
+                                     f"the page size {self.page_size} must be a multiple of {by}")
+                shape = (groups[g].num_pages, *(self.page_size // by if s < 0 else int(s) for s in pool.shape))
                 pools[pool.name] = torch.zeros(shape, dtype=pool.dtype or model.dtype, device=self.device)
             self.layer_caches[layer] = LayerCache(group=g, pools=pools)
         self._state_arenas: List[torch.Tensor] = []

@@ -196,12 +196,13 @@ def qk_norm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor],
                     sin: torch.Tensor, rotary_dim: int, interleaved: bool,
                     positions: torch.Tensor, slots: torch.Tensor, k_cache: torch.Tensor,
                     v_cache: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
-                    q_out: Optional[torch.Tensor] = None, v_transposed: bool = False,
+                    q_out: Optional[torch.Tensor] = None, v_grouped: bool = False,
                     vector_min_tokens: int = 128, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Per-head RMSNorm of q and k (if weights are given), rotation by position, q to q_out
     [T, nq, d], k and v into the paged cache [pages, nkv, page_size, d] at `slots`; with
-    `v_transposed` the V pool is [pages, nkv, d, page_size].  From `vector_min_tokens` tokens
-    on, bfloat16 with the transposed pool runs the vectorized kernel.  `bias` (float32, one
+    `v_grouped` the V pool is [pages, nkv, page_size / 8, d, 8] (eight keys side by side for every
+    dim: what the matrix-core attention reads).  From `vector_min_tokens` tokens
+    on, bfloat16 with the grouped pool runs the vectorized kernel.  `bias` (float32, one
     value per element of a packed row) is added to the rows first, in float32.  `qkv` may be a
     stack [slices, T, width] of float32 partial sums (`linear_mid`), added here in slice order;
     q and the cache then have the cache's dtype and the form of one wave per head runs."""
@@ -233,7 +234,7 @@ def qk_norm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor],
         _want(bias, torch.float32, "qk_norm_rope_kv: bias")
         if bias.shape != (qkv.shape[-1],):
             raise KernelError(f"qk_norm_rope_kv: bias {tuple(bias.shape)} is not [{qkv.shape[-1]}]")
-    _check_cache(k_cache, v_cache, nkv, d, dtype, v_transposed, "qk_norm_rope_kv")
+    _check_cache(k_cache, v_cache, nkv, d, dtype, v_grouped, "qk_norm_rope_kv")
     if q_out is None:
         q_out = torch.empty((T, nq, d), dtype=dtype, device=qkv.device)
     elif q_out.shape != (T, nq, d) or q_out.dtype != dtype:
@@ -242,17 +243,19 @@ def qk_norm_rope_kv(qkv: torch.Tensor, q_weight: Optional[torch.Tensor],
         _p(qkv), _code(q_out, "qk_norm_rope_kv"), slices, _p(bias), _p(q_weight), _p(k_weight), ctypes.c_float(eps),
         _p(cos), _p(sin), int(rotary_dim), int(bool(interleaved)), _p(positions), _p(slots),
         _p(q_out), _p(k_cache), _p(v_cache), int(k_cache.shape[2]), T, nq, nkv, d,
-        int(bool(v_transposed)), int(vector_min_tokens), _stream()))
+        int(bool(v_grouped)), int(vector_min_tokens), _stream()))
     return q_out
 
 
-def _check_cache(k_cache, v_cache, nkv, d, dtype, v_transposed, what):
-    """K pool [pages, nkv, page, d]; V pool the same, or [pages, nkv, d, page] if transposed."""
+def _check_cache(k_cache, v_cache, nkv, d, dtype, v_grouped, what):
+    """K pool [pages, nkv, page, d]; V pool the same, or [pages, nkv, page / 8, d, 8] if in groups of eight keys."""
     if k_cache.dim() != 4 or k_cache.shape[1] != nkv or k_cache.shape[3] != d or k_cache.dtype != dtype:
         raise KernelError(f"{what}: K pool {tuple(k_cache.shape)} {k_cache.dtype} does not match "
                           f"[pages, {nkv}, page_size, {d}] {dtype}")
     pages, _, page, _ = k_cache.shape
-    want = (pages, nkv, d, page) if v_transposed else (pages, nkv, page, d)
+    if v_grouped and page % 8:
+        raise KernelError(f"{what}: V in groups of eight keys needs pages of a multiple of 8 tokens, not {page}")
+    want = (pages, nkv, page // 8, d, 8) if v_grouped else (pages, nkv, page, d)
     if tuple(v_cache.shape) != want or v_cache.dtype != dtype:
         raise KernelError(f"{what}: V pool {tuple(v_cache.shape)} {v_cache.dtype} does not match {want} {dtype}")
 
@@ -260,7 +263,7 @@ def _check_cache(k_cache, v_cache, nkv, d, dtype, v_transposed, what):
 def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       block_tables: torch.Tensor, tok_seq: torch.Tensor, positions: torch.Tensor,
                       scale: float, window: int = 0, out: Optional[torch.Tensor] = None,
-                      v_transposed: bool = False) -> torch.Tensor:
+                      v_grouped: bool = False) -> torch.Tensor:
     """Causal paged GQA attention for any mix of tokens.  q [T, nq, d]; caches
     [pages, nkv, page_size, d]; block_tables int32 [B, max_pages]; tok_seq / positions
     int32 [T] name each token's row of block_tables and its absolute position.
@@ -272,7 +275,7 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     if k_cache.dim() != 4:
         raise KernelError("attention: the K pool must be [pages, nkv, page_size, d]")
     nkv, page = k_cache.shape[1], k_cache.shape[2]
-    _check_cache(k_cache, v_cache, nkv, d, q.dtype, v_transposed, "attention")
+    _check_cache(k_cache, v_cache, nkv, d, q.dtype, v_grouped, "attention")
     for t, name in ((block_tables, "block_tables"), (tok_seq, "tok_seq"), (positions, "positions")):
         _want(t, torch.int32, f"attention: {name}")
     if block_tables.dim() != 2 or tok_seq.shape != (T,) or positions.shape != (T,):
@@ -284,7 +287,7 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     _ok(lib().xi_attention_generic(
         _p(q), _p(k_cache), _p(v_cache), _code(q, "attention"), _p(block_tables),
         int(block_tables.shape[1]), _p(tok_seq), _p(positions), _p(out), ctypes.c_float(scale),
-        int(window), int(page), T, nq, nkv, d, int(bool(v_transposed)), _stream()))
+        int(window), int(page), T, nq, nkv, d, int(bool(v_grouped)), _stream()))
     return out
 
 
@@ -555,7 +558,7 @@ def attention_decode_packed_bf16(qkv, q_weight, k_weight, eps, cos, sin, rotary_
 
 
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx, group: int,
-              scale: float, window: int = 0, v_transposed: bool = False) -> torch.Tensor:
+              scale: float, window: int = 0, v_grouped: bool = False) -> torch.Tensor:
     """Attention of one step's tokens over the paged cache of `group`; chooses the kernel
     from the precision and the shape of the batch: float32, or sizes the matrix-core
     kernels do not take, go to the generic kernel; bfloat16 batches of single tokens to
@@ -563,7 +566,7 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx
     T, nq, d = q.shape
     nkv, page = k_cache.shape[1], k_cache.shape[2]
     bt = ctx.block_tables[group]
-    if q.dtype == torch.bfloat16 and v_transposed and mfma_attention_supported(nq, nkv, d, page):
+    if q.dtype == torch.bfloat16 and v_grouped and mfma_attention_supported(nq, nkv, d, page):
         g = nq // nkv
         if ctx.max_q_len == 1 and decode_attention_takes(nq, nkv, d):
             return attention_decode_bf16(q, k_cache, v_cache, bt, ctx.ctx_lens, ctx.max_ctx_len, scale, window,
@@ -600,7 +603,7 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx
         return attention_prefill_bf16(q, k_cache, v_cache, bt, tiles, ctx.cu_q, ctx.ctx_lens, scale, window,
                                       out=out, small=small)
     return attention_generic(q, k_cache, v_cache, bt, ctx.tok_seq, ctx.positions, scale, window,
-                             v_transposed=v_transposed)
+                             v_grouped=v_grouped)
 
 
 SKINNY_MAX_ROWS = 64      # most rows the streaming kernel takes

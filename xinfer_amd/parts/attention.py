@@ -87,8 +87,8 @@ class PagedAttention(Mixer):
 
     # ---- cache ---------------------------------------------------------------
     def cache_need(self) -> KVNeed:
-        # the matrix-core kernels of the bfloat16 path read V transposed
-        return KVNeed.keys_values(self.nkv, self.d, self.window, v_transposed=self.dtype == torch.bfloat16)
+        # the matrix-core kernels of the bfloat16 path read V in groups of eight keys
+        return KVNeed.keys_values(self.nkv, self.d, self.window, v_grouped=self.dtype == torch.bfloat16)
 
     # ---- step ----------------------------------------------------------------
     takes_sink = True
@@ -125,7 +125,7 @@ class PagedAttention(Mixer):
             pos.sin if pos is not None else ctx.empty_f32,
             pos.rotary_dim if pos is not None else 0,
             pos.interleaved if pos is not None else False,
-            ctx.positions, slots, cache.k, cache.v, self.nq, self.nkv, self.d, v_transposed=vt,
+            ctx.positions, slots, cache.k, cache.v, self.nq, self.nkv, self.d, v_grouped=vt,
             vector_min_tokens=128 if ctx.max_q_len > 1 else self.VECTOR_MIN_DECODE, bias=self.qkv_bias)
-        a = kernels.attention(q, cache.k, cache.v, ctx, cache.group, self.scale, self.window, v_transposed=vt)
+        a = kernels.attention(q, cache.k, cache.v, ctx, cache.group, self.scale, self.window, v_grouped=vt)
         return self.o(a, out_dtype=self.dtype, allow_split=True, sink=sink)     # the next norm adds the parts

@@ -39,21 +39,26 @@ from ..weights.store import TensorDecl, WeightStore
 
 # ---- what a layer may ask of the cache ------------------------------------------------
 PAGE = -1      # in a pool's shape: the axis that is as long as a page has tokens
+PAGE_BY_8 = -8 # the axis that is an eighth of that (-n: the page's tokens divided by n, which must divide them)
 
 
 @dataclass(frozen=True)
 class PoolNeed:
     """One paged pool of a layer: the runner allocates [pages, *shape] with PAGE replaced by the
-    page size, in `dtype` (None: the activation dtype), and hands it to the mixer under `name`."""
+    page size (PAGE_BY_8: by an eighth of it), in `dtype` (None: the activation dtype), and hands it to
+    the mixer under `name`.  A shape has one such axis."""
     name: str
     shape: Tuple[int, ...]
     dtype: Optional[torch.dtype] = None
 
     def bytes_per_token(self, element_size: int) -> int:
-        n = 1
+        n, by = 1, 1
         for s in self.shape:
-            n *= 1 if s == PAGE else int(s)
-        return n * (element_size if self.dtype is None else torch.tensor([], dtype=self.dtype).element_size())
+            if s < 0:
+                by = -int(s)
+            else:
+                n *= int(s)
+        return n // by * (element_size if self.dtype is None else torch.tensor([], dtype=self.dtype).element_size())
 
 
 @dataclass(frozen=True)
@@ -66,11 +71,11 @@ class KVNeed:
     pools: Tuple[PoolNeed, ...] = ()
 
     @staticmethod
-    def keys_values(num_kv_heads: int, head_dim: int, window: int = 0, v_transposed: bool = False) -> "KVNeed":
+    def keys_values(num_kv_heads: int, head_dim: int, window: int = 0, v_grouped: bool = False) -> "KVNeed":
         """K pool "k" [pages, kv_heads, page_size, head_dim]; V pool "v" the same, or with
-        `v_transposed` [pages, kv_heads, head_dim, page_size]."""
+        `v_grouped` [pages, kv_heads, page_size / 8, head_dim, 8] (eight keys side by side for every dim)."""
         k = PoolNeed("k", (num_kv_heads, PAGE, head_dim))
-        v = PoolNeed("v", (num_kv_heads, head_dim, PAGE) if v_transposed else (num_kv_heads, PAGE, head_dim))
+        v = PoolNeed("v", (num_kv_heads, PAGE_BY_8, head_dim, 8) if v_grouped else (num_kv_heads, PAGE, head_dim))
         return KVNeed(window, (k, v))
 
 
