@@ -1182,7 +1182,8 @@ def test_decode_keys_per_workgroup_grow_with_the_work():
     """Sequences of about one length: the splits that make the fewest rounds of workgroups over the
     256 compute units, one round of large chunks where there is one, whole sequences from 256
     (sequence, kv head) pairs on, and workgroups for seven eighths of the units at least where the keys allow.  Mixed
-    lengths: chunks of 128 to 512 keys, about 512 workgroups."""
+    lengths: chunks of 128 to 512 keys, about 512 workgroups; chunks of 1,024 from one pair a compute unit on, whole
+    sequences (up to 2,048 keys) from one and a half."""
     from xinfer_amd import kernels
     plan = lambda pairs, span: kernels.decode_keys_per_workgroup(pairs, span, similar=True)
     assert plan(8, 4096) == 128                  # 32 splits: 256 workgroups
@@ -1199,7 +1200,8 @@ def test_decode_keys_per_workgroup_grow_with_the_work():
     assert plan(4, 1024) == 128                  # too few keys for 256 workgroups: as many as there are
     mixed = lambda pairs, span: kernels.decode_keys_per_workgroup(pairs, span, similar=False)
     assert mixed(8, 4096) == 128 and mixed(32, 4096) == 256 and mixed(64, 4096) == 512
-    assert mixed(512, 2304) == 512 and mixed(8, 131072) == 512
+    assert mixed(200, 2304) == 512 and mixed(8, 131072) == 512
+    assert mixed(256, 2304) == 1024 and mixed(512, 2304) == 2048 and mixed(512, 2048) == 2176     # many pairs: longer chunks, whole sequences
 
 
 @pytest.mark.parametrize("window", [0, 100])

@@ -39,9 +39,12 @@ def test_decode_keys_per_workgroup_is_a_multiple_of_128_and_covers_the_span(simi
             assert span // kpw + 1 <= 1025
 
 
-def test_decode_mixed_lengths_take_whole_sequences_from_three_pairs_a_compute_unit():
-    assert kernels.decode_keys_per_workgroup(767, 1024, False) == 512
-    assert kernels.decode_keys_per_workgroup(768, 1024, False) == 1152          # one split: no second kernel
+def test_decode_mixed_lengths_take_whole_sequences_where_there_are_many():
+    assert kernels.decode_keys_per_workgroup(255, 4096, False) == 512
+    assert kernels.decode_keys_per_workgroup(256, 4096, False) == 1024             # a pair a compute unit
+    assert kernels.decode_keys_per_workgroup(256, 1024, False) == 512
+    assert kernels.decode_keys_per_workgroup(383, 1024, False) == 512
+    assert kernels.decode_keys_per_workgroup(384, 1024, False) == 1152             # one split: no second kernel
     assert kernels.decode_keys_per_workgroup(1536, 2048, False) == 2176
     assert kernels.decode_keys_per_workgroup(2048, 3072, False) == 2048
     assert kernels.decode_keys_per_workgroup(2048, 16384, False) == 2048

@@ -318,7 +318,7 @@ DECODE_KEYS_LEAST = 128             # keys of a workgroup: from one 32-key step 
 DECODE_KEYS_MOST = 512              # to four, in batches of mixed lengths
 DECODE_WORKGROUP_KEYS = 32          # what a workgroup costs beyond its keys (start, page numbers, merge, partial results), in keys
 DECODE_SPLITS_MOST = 1024           # splits of a sequence that the search below tries
-DECODE_WHOLE_KEYS = 2048            # mixed lengths, three pairs a compute unit and more: a workgroup's keys at most
+DECODE_WHOLE_KEYS = 2048            # mixed lengths, one and a half pairs a compute unit and more: a workgroup's keys at most
 
 
 def decode_keys_per_workgroup(pairs: int, span: int, similar: bool = False) -> int:
@@ -342,12 +342,14 @@ def _decode_keys_per_workgroup(pairs: int, span: int, similar: bool) -> int:
 
     Otherwise (mixed lengths): 128, 256 or 512 keys, whichever makes about DECODE_WORKGROUPS
     workgroups: larger chunks lose there (64 sequences of 256 to 2,304 keys: 75 us at 512, 81 at
-    1,024), since the short sequences' workgroups end early and the long ones' run on.  From three
-    pairs a compute unit on there are enough workgroups to even that out (the scheduler puts the long
-    sequences first), and a workgroup's start and end cost more than the chunks' balance gains:
-    whole sequences up to DECODE_WHOLE_KEYS keys, chunks of that many beyond (192 sequences of 100
-    to 768 keys, longest first: 68.9 us against 77.3 in chunks of 512, and 84.6 in chunks of 512 in
-    random order; 128 sequences of 500 to 4,000: 253 against 257)."""
+    1,024), since the short sequences' workgroups end early and the long ones' run on.  From one
+    and a half pairs a compute unit on there are enough workgroups to even that out (the scheduler
+    puts the long sequences first), and a workgroup's start and end cost more than the chunks'
+    balance gains: whole sequences up to DECODE_WHOLE_KEYS keys, chunks of that many beyond (192
+    sequences of 100 to 768 keys, longest first: 64 us against 72 in chunks of 512, and 80 in chunks
+    of 512 in random order; 64 of 256 to 2,304: 64 against 68; 48 of 100 to 768: 20.5 against 21.9);
+    from one pair a compute unit on chunks of 1,024 (32 sequences of 500 to 4,000: 60 us against 65
+    at 512 and 63 whole)."""
     if similar:
         chunks = max(1, -(-int(span) // 128))
         plans = []
@@ -365,8 +367,10 @@ def _decode_keys_per_workgroup(pairs: int, span: int, similar: bool) -> int:
         if best[2] == 1:
             return (span + 128) // 128 * 128          # more than span: one split
         return best[1]
-    if pairs >= 3 * COMPUTE_UNITS:
+    if 2 * pairs >= 3 * COMPUTE_UNITS:
         return (span + 128) // 128 * 128 if span <= DECODE_WHOLE_KEYS else DECODE_WHOLE_KEYS
+    if pairs >= COMPUTE_UNITS and span > 1024:
+        return 1024
     kpw = DECODE_KEYS_LEAST
     while kpw < DECODE_KEYS_MOST and pairs * span >= 2 * kpw * DECODE_WORKGROUPS:
         kpw *= 2
