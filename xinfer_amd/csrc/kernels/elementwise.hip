@@ -334,6 +334,16 @@ __global__ __launch_bounds__(1024) void qk_norm_rope_kvt_bf16_kernel(
     const int kvh = h - nq - nkv;
     bf16* vs = reinterpret_cast<bf16*>(smem_raw);  // [tpw][d + 2]
     const int vstride = d + 2;                      // an odd number of 32-bit words per row
+    // Every lane looks up where its own token of the block goes (lane = token); a store then takes eight
+    // tokens by eight dims: lane -> token 8 tg + (lane & 7), dim i0 + (lane >> 3), the place handed over
+    // from the token's lane.
+    const long long slot = (lane < tpw && t0 + lane < n_tok) ? slots[t0 + lane] : -1;
+    unsigned long long place = ~0ull;          // of the token's dim 0 in the pool, in elements
+    if (slot >= 0) {
+      const long long page = slot / page_size;
+      const int off = (int)(slot - page * page_size);
+      place = ((unsigned long long)page * nkv + kvh) * d * page_size + (unsigned long long)(off >> 3) * d * 8 + (off & 7);
+    }
     if (on) {
       uint4 raw = *reinterpret_cast<const uint4*>(qkv + ((size_t)t * heads + h) * d + 8 * c);
       if (bias) {
@@ -349,17 +359,13 @@ __global__ __launch_bounds__(1024) void qk_norm_rope_kvt_bf16_kernel(
       dst[3] = raw.w;
     }
     __syncthreads();
-    // lane: token 8 tg + (lane & 7) of the block, dim i0 + (lane >> 3)
     const int units = ((tpw + 7) >> 3) * (d >> 3);
     for (int u = wave; u < units; u += (int)(blockDim.x >> 6)) {
       const int tg = u / (d >> 3), i = 8 * (u - tg * (d >> 3)) + (lane >> 3);
       const int tok = 8 * tg + (lane & 7);
-      const long long slot = (tok < tpw && t0 + tok < n_tok) ? slots[t0 + tok] : -1;
-      if (slot >= 0) {
-        const long long page = slot / page_size;
-        const int off = (int)(slot - page * page_size);
-        vt_cache[((size_t)page * nkv + kvh) * d * page_size + ((size_t)(off >> 3) * d + i) * 8 + (off & 7)] = vs[tok * vstride + i];
-      }
+      const unsigned lo = __shfl((unsigned)place, tok, kWave), hi = __shfl((unsigned)(place >> 32), tok, kWave);
+      const unsigned long long at = ((unsigned long long)hi << 32) | lo;
+      if (at != ~0ull) vt_cache[at + (size_t)i * 8] = vs[tok * vstride + i];
     }
     return;
   }
