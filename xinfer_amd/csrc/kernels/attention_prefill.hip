@@ -131,10 +131,11 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_prefill_lds_kernel(
   // head_dim are zero), thread t moves chunks t, t + 256, ...; in LDS the keys of each
   // 32-key step are permuted so that the 16 rows one matrix operand reads are consecutive:
   // key k sits at row 16*((k>>2)&1) + 4*(k>>3) + (k&3) of its step.  V^T tile: d rows of 8
-  // key groups, same distribution.
+  // key groups; thread t moves row t % d of key group t / d, .. (the pool keeps a key group's rows
+  // side by side: threads that follow each other read 16 bytes that follow each other).
   constexpr int CPK = 4 * KC;        // chunks per K row in LDS
   const int n_vchunks = 8 * d;
-  int c_kl[LI], c_koff[LI], c_kdst[LI], c_vdst[LI];
+  int c_kl[LI], c_koff[LI], c_kdst[LI], c_vdst[LI], c_vrow[LI], c_vkg[LI];
 #pragma unroll
   for (int i = 0; i < LI; ++i) {
     const int idx = tid + NT * i;
@@ -143,26 +144,27 @@ __global__ __launch_bounds__(64 * NWV, 2) void attn_prefill_lds_kernel(
     c_kl[i] = kl;
     c_koff[i] = 8 * ch < d ? 8 * ch : -1;       // -1: a chunk of zeros
     c_kdst[i] = ((kl & 32) + 16 * ((k32 >> 2) & 1) + 4 * (k32 >> 3) + (k32 & 3)) * krow + 8 * ch;
-    c_vdst[i] = (idx >> 3) * vrow + 8 * (idx & 7);
+    c_vkg[i] = idx / d;
+    c_vrow[i] = idx - c_vkg[i] * d;
+    if (c_vkg[i] > 7) { c_vkg[i] = 7; c_vrow[i] = d - 1; }      // past the tile: read again what the last chunk reads, store nothing
+    c_vdst[i] = c_vrow[i] * vrow + 8 * c_vkg[i];
   }
   const size_t kv_head_stride = (size_t)d << page_shift;     // elements of one (page, kv head) block
   bf16x8 kreg[LI], vreg[LI];
   auto fetch = [&](int kb) {
 #pragma unroll
     for (int i = 0; i < LI; ++i) {
-      const int idx = tid + NT * i;
       int key = kb + c_kl[i];
       key = key > k_last ? k_last : key;
       const int kp = bt_s[key >> page_shift];
       const bf16* ksrc = k_cache + ((size_t)kp * nkv + kvh) * kv_head_stride +
                          (size_t)(key & (page - 1)) * d + (c_koff[i] < 0 ? 0 : c_koff[i]);
       kreg[i] = ld8(ksrc);
-      int key0 = kb + 8 * (idx & 7);
+      int key0 = kb + 8 * c_vkg[i];
       key0 = key0 > k_last ? (k_last & ~7) : key0;
       const int vp = bt_s[key0 >> page_shift];
-      const int vr = (idx >> 3) < d ? (idx >> 3) : d - 1;     // rows past head_dim are not stored
       vreg[i] = ld8(vt_cache + ((size_t)vp * nkv + kvh) * kv_head_stride +
-                    ((size_t)((key0 & (page - 1)) >> 3) * d + vr) * 8);     // [offset / 8, d, 8]
+                    ((size_t)((key0 & (page - 1)) >> 3) * d + c_vrow[i]) * 8);     // [offset / 8, d, 8]
     }
   };
   auto stash = [&](int buf) {
