@@ -511,6 +511,26 @@ def test_first_tokens(name, dtype, model_dirs):
     harness.compare(got, ref, harness.TOL[dtype], f"first tokens {name} {dtype}")
 
 
+def test_bfloat16_cache_keeps_values_in_groups_of_eight_keys(model_dirs):
+    """The bfloat16 path keeps V as [pages, kv heads, page / 8, head_dim, 8] (what its matrix-core kernels read), the
+    32-bit path as [pages, kv heads, page, head_dim]; a page that is no multiple of 8 tokens is refused in bfloat16 with a
+    clear error and runs in 32 bits."""
+    from xinfer_amd.engine import ModelRunner, StepEntry, load_model
+    cfg = TINY["A"]["config"]
+    nkv, d = cfg["num_key_value_heads"], cfg["head_dim"]
+    model = load_model(model_dirs["A"], "bfloat16", DEV)
+    runner = ModelRunner(model, page_size=16, num_pages=3, max_requests=1)
+    lc = next(iter(runner.layer_caches.values()))
+    assert tuple(lc.k.shape) == (3, nkv, 16, d) and tuple(lc.v.shape) == (3, nkv, 2, d, 8)
+    with pytest.raises(ValueError, match="multiple of 8"):
+        ModelRunner(model, page_size=12, num_pages=3, max_requests=1)
+    wide = ModelRunner(load_model(model_dirs["A"], "float32", DEV), page_size=12, num_pages=3, max_requests=1)
+    lc = next(iter(wide.layer_caches.values()))
+    assert tuple(lc.v.shape) == tuple(lc.k.shape) == (3, nkv, 12, d)
+    wide.add_request(0)
+    assert torch.isfinite(wide.step([StepEntry(0, list(range(1, 20)), [18])])).all()
+
+
 def test_step_refuses_bad_input(model_dirs):
     from xinfer_amd.cache import OutOfPages
     from xinfer_amd.engine import ModelRunner, StepEntry, StepError, load_model
